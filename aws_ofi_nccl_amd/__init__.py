@@ -1,0 +1,168 @@
+"""Python bindings (ctypes) onto libofi_amd_hotpath.so for tests and benchmarks.
+
+The product is the C-ABI library declared in include/ofi_amd_hotpath.h; this
+module only loads it and sets argument types.  There is no CPU implementation
+behind these bindings: if the library has not been built, loading raises.
+"""
+import ctypes
+import os
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "lib", "libofi_amd_hotpath.so")
+
+_lib = None
+
+c_u8p = ctypes.c_void_p
+c_u32 = ctypes.c_uint32
+c_u64 = ctypes.c_uint64
+c_i32 = ctypes.c_int32
+c_vp = ctypes.c_void_p
+
+
+class SchedState(ctypes.Structure):
+    """ofi_amd_sched_state_t"""
+    _fields_ = [("rr_small_counter", c_u32), ("rr_counter", c_u32),
+                ("max_small_msg_size", c_u64), ("min_stripe_size", c_u64),
+                ("num_rails", c_i32), ("pad", c_i32)]
+
+
+class XferInfo(ctypes.Structure):
+    """ofi_amd_xfer_info_t (24 bytes)"""
+    _fields_ = [("rail_id", ctypes.c_uint16), ("pad0", ctypes.c_uint16), ("pad1", c_u32),
+                ("offset", c_u64), ("msg_size", c_u64)]
+
+
+class GinDesc(ctypes.Structure):
+    """ofi_amd_gin_desc_t (64 bytes)"""
+    _fields_ = [("src_off", c_u64), ("dst_off", c_u64), ("size", c_u64), ("signal_off", c_u64),
+                ("signal_value", c_u64), ("rank", c_u32), ("signal_op", c_u32),
+                ("opt_flags", c_u32), ("context", c_u32), ("src_mr", ctypes.c_uint16),
+                ("dst_mr", ctypes.c_uint16), ("sig_mr", ctypes.c_uint16),
+                ("kind", ctypes.c_uint16)]
+
+
+class GinMr(ctypes.Structure):
+    """ofi_amd_gin_mr_t"""
+    _fields_ = [("local_base", c_u64), ("remote_address", c_u64),
+                ("remote_address_offset", c_u64), ("key", c_u64 * 4)]
+
+
+class GinWrite(ctypes.Structure):
+    _fields_ = [("src", c_u64), ("len", c_u64), ("dest", c_u64), ("key", c_u64),
+                ("rail", c_u32), ("more", c_u32)]
+
+
+class GinWire(ctypes.Structure):
+    """ofi_amd_gin_wire_t (192 bytes)"""
+    _fields_ = [("seq", c_u32), ("nseg", c_u32), ("imm", c_u32), ("num_writes", c_u32),
+                ("has_meta", c_u32), ("meta_rail", c_u32), ("meta_more", c_u32),
+                ("ack_req", c_u32), ("writes", GinWrite * 4), ("meta", c_u64 * 4)]
+
+
+class GinComm(ctypes.Structure):
+    """ofi_amd_gin_comm_t"""
+    _fields_ = [("sched", SchedState), ("comm_id", c_u32), ("num_rails", c_u32),
+                ("tx_head", c_u32), ("tx_tail", c_u32),
+                ("consecutive_puts_without_ack", c_u32), ("last_ack_requested_seq", c_u32),
+                ("has_pending_ack_request", c_u32), ("pinned_rail_id", c_i32),
+                ("pinned_rail_run", c_u32), ("next_rail_id", c_u32), ("ack_model", c_u32),
+                ("pad", c_u32)]
+
+
+class GinProxyStats(ctypes.Structure):
+    _fields_ = [("descriptors", c_u64), ("signals", c_u64), ("writes", c_u64),
+                ("checksum", c_u64), ("seconds", ctypes.c_double), ("empty_polls", c_u64)]
+
+
+class TunerVariant(ctypes.Structure):
+    _fields_ = [("platform", c_i32), ("pipe_ops", c_i32), ("num_channels", c_i32),
+                ("net_comp_overhead", c_i32)]
+
+
+# name -> (restype, argtypes); every symbol include/ofi_amd_hotpath.h declares
+PROTOTYPES = {
+    "ofi_amd_gpu_init": (ctypes.c_int, []),
+    "ofi_amd_gpu_get_device_for_addr": (ctypes.c_int, [c_vp, ctypes.POINTER(ctypes.c_int)]),
+    "ofi_amd_gpu_flush_gpudirect_rdma_writes": (ctypes.c_int, []),
+    "ofi_amd_gpu_mem_alloc": (ctypes.c_int, [ctypes.POINTER(c_vp), ctypes.c_size_t]),
+    "ofi_amd_gpu_mem_free": (ctypes.c_int, [c_vp]),
+    "ofi_amd_gpu_mem_copy_host_to_device": (ctypes.c_int, [c_vp, c_vp, ctypes.c_size_t]),
+    "ofi_amd_gpu_mem_copy_device_to_host": (ctypes.c_int, [c_vp, c_vp, ctypes.c_size_t]),
+    "ofi_amd_gpu_stream_synchronize": (ctypes.c_int, [c_vp]),
+    "ofi_amd_async_error_fetch": (ctypes.c_int, [ctypes.POINTER(c_u32)]),
+    "ofi_amd_gpu_get_dma_buf_fd": (ctypes.c_int, [c_vp, ctypes.c_size_t,
+                                                  ctypes.POINTER(ctypes.c_int),
+                                                  ctypes.POINTER(ctypes.c_size_t)]),
+    "ofi_amd_gpu_have_dma_buf_attr": (ctypes.c_int, []),
+    "ofi_amd_gpu_have_gdr_support_attr": (ctypes.c_int, []),
+    "ofi_amd_gpu_set_current_device": (ctypes.c_int, [ctypes.c_int]),
+    "ofi_amd_gpu_get_current_device": (ctypes.c_int, [ctypes.POINTER(ctypes.c_int)]),
+    "ofi_amd_gpu_get_address_range": (ctypes.c_int, [c_vp, ctypes.POINTER(c_vp),
+                                                     ctypes.POINTER(ctypes.c_size_t)]),
+    "ofi_amd_gpu_seg_is_host": (ctypes.c_int, [c_vp, ctypes.POINTER(ctypes.c_int)]),
+    "ofi_amd_gpu_host_alloc": (ctypes.c_int, [ctypes.POINTER(c_vp), ctypes.c_size_t]),
+    "ofi_amd_gpu_host_free": (ctypes.c_int, [c_vp]),
+    "ofi_amd_gpu_host_get_device_pointer": (ctypes.c_int, [ctypes.POINTER(c_vp), c_vp]),
+    "ofi_amd_sched_batch": (ctypes.c_int, [c_vp, c_vp, c_u64, c_u64, c_vp, c_vp, c_vp]),
+    "ofi_amd_sched_get_schedule": (ctypes.c_int, [ctypes.POINTER(SchedState), c_u64, c_u64,
+                                                  ctypes.POINTER(XferInfo)]),
+    "ofi_amd_bounce_scatter": (ctypes.c_int, [c_vp, c_vp, c_u64, c_vp, c_vp, c_vp, c_u32, c_vp,
+                                              c_vp]),
+    "ofi_amd_flush_read": (ctypes.c_int, [c_vp, c_vp, c_u32, c_vp, c_vp]),
+    "ofi_amd_devcopy_register": (ctypes.c_int, [c_vp, ctypes.c_size_t, ctypes.POINTER(c_vp)]),
+    "ofi_amd_devcopy_to_device": (ctypes.c_int, [c_vp, c_vp, ctypes.c_size_t, ctypes.c_size_t]),
+    "ofi_amd_devcopy_from_device": (ctypes.c_int, [c_vp, ctypes.c_size_t, c_vp,
+                                                   ctypes.c_size_t]),
+    "ofi_amd_devcopy_forced_pcie_copy": (ctypes.c_int, []),
+    "ofi_amd_devcopy_deregister": (ctypes.c_int, [c_vp]),
+    "ofi_amd_gin_rings_create": (ctypes.c_int, [c_u32, c_u32, ctypes.POINTER(c_vp)]),
+    "ofi_amd_gin_rings_destroy": (ctypes.c_int, [c_vp]),
+    "ofi_amd_gin_rings_view": (ctypes.c_int, [c_vp, ctypes.POINTER(c_vp), ctypes.POINTER(c_vp),
+                                              ctypes.POINTER(c_u32), ctypes.POINTER(c_u32)]),
+    "ofi_amd_gin_produce_seeded": (ctypes.c_int, [c_vp, c_u64, c_u64, c_u32, c_u32, c_u32, c_u32,
+                                                  c_u64, c_vp]),
+    "ofi_amd_gin_producer_status": (ctypes.c_int, [c_vp]),
+    "ofi_amd_gin_ring_push": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(GinDesc)]),
+    "ofi_amd_gin_ring_pop": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(GinDesc)]),
+    "ofi_amd_gin_comm_init": (ctypes.c_int, [ctypes.POINTER(GinComm), c_u32, c_u32, c_u64, c_u64,
+                                             c_u32]),
+    "ofi_amd_gin_iput_signal": (ctypes.c_int, [ctypes.POINTER(GinComm), ctypes.POINTER(GinMr),
+                                               ctypes.POINTER(GinDesc), ctypes.POINTER(GinWire)]),
+    "ofi_amd_gin_apply_ack": (None, [ctypes.POINTER(GinComm), c_u32]),
+    "ofi_amd_gin_imm": (c_u32, [c_u32, c_u32, c_u32, c_u32]),
+    "ofi_amd_gin_meta_header": (c_u64, [c_u32, c_u32, c_u32, c_u32]),
+    "ofi_amd_gin_ack_msg": (c_u64, [c_u32, c_u32]),
+    "ofi_amd_gin_proxy_drain": (ctypes.c_int, [c_vp, c_u64, ctypes.c_int, c_vp, c_vp, c_vp, c_vp,
+                                               c_u32, ctypes.POINTER(GinProxyStats)]),
+    "ofi_amd_tuner_plan_create": (ctypes.c_int, [c_vp, c_u32, c_vp, c_u32, c_vp, c_u32, c_vp,
+                                                 c_u32, c_vp, c_u32, ctypes.POINTER(c_vp)]),
+    "ofi_amd_tuner_plan_destroy": (ctypes.c_int, [c_vp]),
+    "ofi_amd_tuner_plan_points": (c_u64, [c_vp]),
+    "ofi_amd_tuner_plan_cells": (c_u64, [c_vp]),
+    "ofi_amd_tuner_model_grid": (ctypes.c_int, [c_vp, c_vp, c_u32, c_vp, c_vp, c_vp]),
+    "ofi_amd_tuner_region_grid": (ctypes.c_int, [c_vp, c_vp, c_u32, c_vp, c_vp]),
+}
+
+
+def load(path=None):
+    """Load the product library; raises if it is missing (there is no fallback)."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    p = path or LIB_PATH
+    if not os.path.exists(p):
+        raise RuntimeError(
+            "%s not built: run `python -m aws_ofi_nccl_amd.build` (hipcc, gfx950)" % p)
+    lib = ctypes.CDLL(p)
+    for name, (res, args) in PROTOTYPES.items():
+        fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
+        fn.restype = res
+        fn.argtypes = args
+    if path is None:
+        _lib = lib
+    return lib
+
+
+def check(rc, what="call"):
+    if rc != 0:
+        raise RuntimeError("%s failed: %d (%s)" % (what, rc, os.strerror(-rc) if rc < 0 else rc))

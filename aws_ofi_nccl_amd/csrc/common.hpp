@@ -1,0 +1,58 @@
+/*
+ * Shared host-side helpers of libofi_amd_hotpath.so: HIP error -> errno
+ * translation (the convention of include/nccl_ofi_rocm.h in the reference),
+ * device presence check, and the pinned-host word kernels use to report a
+ * precondition violation they detected on the device.
+ */
+#ifndef OFI_AMD_COMMON_HPP_
+#define OFI_AMD_COMMON_HPP_
+
+#include <cerrno>
+#include <cstdint>
+#include <cstdio>
+
+#include <hip/hip_runtime.h>
+
+namespace ofi_amd {
+
+inline int errno_of(hipError_t e)
+{
+	switch (e) {
+	case hipSuccess: return 0;
+	case hipErrorNoDevice:
+	case hipErrorInvalidDevice:
+	case hipErrorInsufficientDriver: return -ENODEV;
+	case hipErrorOutOfMemory: return -ENOMEM;
+	case hipErrorInvalidValue:
+	case hipErrorInvalidDevicePointer: return -EINVAL;
+	case hipErrorNotSupported: return -ENOTSUP;
+	default: return -EIO;
+	}
+}
+
+#define OFI_AMD_HIP_TRY(expr)                                                           \
+	do {                                                                            \
+		hipError_t e_ = (expr);                                                 \
+		if (e_ != hipSuccess) {                                                 \
+			return ::ofi_amd::errno_of(e_);                                 \
+		}                                                                       \
+	} while (0)
+
+/* 0 when at least one GPU is usable, else -ENODEV.  Never falls back. */
+int require_device();
+
+/* Device-visible error word (pinned host memory): kernels OR a bit into it when
+ * they skip work because a documented precondition does not hold. */
+uint32_t *async_error_word();
+
+inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
+
+enum : uint32_t {
+	ASYNC_ERR_BOUNCE_RANGE = 1u << 0, /* destination range outside arena or misaligned */
+	ASYNC_ERR_GIN_TIMEOUT = 1u << 1,  /* producer gave up on a full ring */
+	ASYNC_ERR_SCHED_STATE = 1u << 2,  /* scheduler state unusable (rails, stripe size) */
+};
+
+} // namespace ofi_amd
+
+#endif

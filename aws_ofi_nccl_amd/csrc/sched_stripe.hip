@@ -1,0 +1,427 @@
+/*
+ * Batched rail striping (threshold scheduler) for gfx950.
+ *
+ * The reference schedules one message per call on a stateful object: messages
+ * below max_small_msg_size take one rail from rr_small_counter, larger ones take
+ * get_num_stripes(size) consecutive rails starting at rr_counter; both counters
+ * advance modulo num_rails (src/nccl_ofi_scheduler.cpp:47-133).  For a batch in
+ * index order that is two exclusive prefix sums:
+ *
+ *   small_rail_i = (rr_small + #{j < i : size_j <  max_small}) mod R
+ *   start_rail_i = (rr      + sum{j < i : size_j >= max_small} n_j) mod R
+ *
+ * Three launches on one stream:
+ *   1. stripe_count_kernel  per-tile totals of (small count, stripe count)
+ *   2. stripe_scan_kernel   one workgroup scans the tile totals, seeds them with
+ *                           the counters in *state, writes the new counters back
+ *   3. stripe_emit_kernel   re-reads the tile, scans inside the workgroup with
+ *                           wavefront shuffles, builds the 96-byte stripe rows in
+ *                           LDS and writes them out as coalesced 16-byte stores
+ *
+ * HBM traffic per message: 8 B read twice + 4 B + 96 B written.
+ */
+#include <mutex>
+
+#include "common.hpp"
+#include "ofi_amd_hotpath.h"
+
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr uint32_t kThreads = 256;
+constexpr uint32_t kPasses = 4;
+constexpr uint32_t kTile = kThreads * kPasses; /* messages per workgroup */
+constexpr uint32_t kScanThreads = 1024;
+constexpr uint64_t kMaxBatch = 1ull << 28;
+
+struct params_t {
+	uint64_t max_small;
+	uint64_t min_stripe;
+	uint64_t align;
+	int32_t min_stripe_shift; /* log2 when a power of two, else -1 */
+	int32_t align_shift;
+	uint32_t num_rails;
+};
+
+__device__ __forceinline__ uint64_t div_by(uint64_t x, uint64_t d, int32_t shift)
+{
+	return shift >= 0 ? (x >> shift) : (x / d);
+}
+
+/* NCCL_OFI_DIV_CEIL, include/nccl_ofi_math.h:23-26 */
+__device__ __forceinline__ uint64_t div_ceil_by(uint64_t x, uint64_t d, int32_t shift)
+{
+	return x == 0 ? 0 : 1 + div_by(x - 1, d, shift);
+}
+
+/* get_num_stripes, src/nccl_ofi_scheduler.cpp:47-64 */
+__device__ __forceinline__ uint32_t num_stripes(uint64_t size, const params_t &p)
+{
+	uint64_t want = div_ceil_by(size, p.min_stripe, p.min_stripe_shift);
+	uint32_t n = (uint32_t)(want < p.num_rails ? want : p.num_rails);
+	n = n > 1 ? n : 1;
+	for (uint32_t i = n; i > 1; i--) {
+		if ((p.num_rails % i) == 0) {
+			return i;
+		}
+	}
+	return n;
+}
+
+/* Thresholds come from the device-resident state; a power-of-two divisor becomes a
+ * shift.  False when the state is unusable (rails outside 1..4, zero stripe size). */
+__device__ __forceinline__ int32_t log2_if_pow2_dev(uint64_t v)
+{
+	return (v != 0 && (v & (v - 1)) == 0) ? (int32_t)(__ffsll((unsigned long long)v) - 1) : -1;
+}
+
+__device__ __forceinline__ bool load_params(const ofi_amd_sched_state_t *st, uint64_t align,
+					    params_t &p)
+{
+	p.max_small = st->max_small_msg_size;
+	p.min_stripe = st->min_stripe_size;
+	p.align = align;
+	p.min_stripe_shift = log2_if_pow2_dev(p.min_stripe);
+	p.align_shift = log2_if_pow2_dev(align);
+	p.num_rails = (uint32_t)st->num_rails;
+	return st->num_rails >= 1 && st->num_rails <= OFI_AMD_MAX_NUM_RAILS && p.min_stripe != 0;
+}
+
+/* x / k for k in 1..4 without a general 64-bit division */
+__device__ __forceinline__ uint64_t div_small(uint64_t x, uint32_t k)
+{
+	switch (k) {
+	case 1: return x;
+	case 2: return x >> 1;
+	case 3: return x / 3;
+	default: return x >> 2;
+	}
+}
+
+/* packed (small count << 16 | stripe count) contribution of one message */
+__device__ __forceinline__ uint32_t contribution(uint64_t size, const params_t &p, uint32_t &n_out)
+{
+	if (size < p.max_small) {
+		n_out = 1;
+		return 1u << 16;
+	}
+	n_out = num_stripes(size, p);
+	return n_out;
+}
+
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, uint32_t lane)
+{
+#pragma unroll
+	for (uint32_t d = 1; d < 64; d <<= 1) {
+		uint32_t up = __shfl_up(v, d, 64);
+		if (lane >= d) {
+			v += up;
+		}
+	}
+	return v;
+}
+
+__global__ __launch_bounds__(kThreads) void stripe_count_kernel(
+	const uint64_t *__restrict__ sizes, uint32_t n, const ofi_amd_sched_state_t *__restrict__ state,
+	uint64_t align, uint32_t *__restrict__ tile_totals)
+{
+	__shared__ uint32_t wave_sum[kThreads / 64];
+	params_t p;
+	if (!load_params(state, align, p)) {
+		return;
+	}
+	const uint32_t base = blockIdx.x * kTile;
+	uint32_t acc = 0;
+#pragma unroll
+	for (uint32_t pass = 0; pass < kPasses; pass++) {
+		uint32_t i = base + pass * kThreads + threadIdx.x;
+		if (i < n) {
+			uint32_t k;
+			acc += contribution(sizes[i], p, k);
+		}
+	}
+#pragma unroll
+	for (uint32_t d = 32; d > 0; d >>= 1) {
+		acc += __shfl_xor(acc, d, 64);
+	}
+	if ((threadIdx.x & 63u) == 0) {
+		wave_sum[threadIdx.x >> 6] = acc;
+	}
+	__syncthreads();
+	if (threadIdx.x == 0) {
+		tile_totals[blockIdx.x] = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
+	}
+}
+
+/* One workgroup: exclusive scan of the tile totals.  tile_prefix[t] holds the two
+ * rail seeds of tile t (already reduced mod R); *state gets the final counters. */
+__global__ __launch_bounds__(kScanThreads) void stripe_scan_kernel(
+	const uint32_t *__restrict__ tile_totals, uint32_t num_tiles,
+	ofi_amd_sched_state_t *__restrict__ state, uint32_t *__restrict__ tile_prefix,
+	uint32_t *__restrict__ err)
+{
+	__shared__ uint32_t wave_small[kScanThreads / 64];
+	__shared__ uint32_t wave_big[kScanThreads / 64];
+	const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+	if (state->num_rails < 1 || state->num_rails > OFI_AMD_MAX_NUM_RAILS ||
+	    state->min_stripe_size == 0) {
+		if (threadIdx.x == 0) {
+			atomicOr(err, ofi_amd::ASYNC_ERR_SCHED_STATE);
+		}
+		return;
+	}
+	const uint32_t num_rails = (uint32_t)state->num_rails;
+	/* totals can reach 2^28 each, so the two sums are scanned unpacked */
+	uint32_t carry_small = state->rr_small_counter % num_rails;
+	uint32_t carry_big = state->rr_counter % num_rails;
+
+	for (uint32_t start = 0; start < num_tiles; start += kScanThreads) {
+		uint32_t t = start + threadIdx.x;
+		uint32_t packed = t < num_tiles ? tile_totals[t] : 0;
+		uint32_t s = packed >> 16, b = packed & 0xffffu;
+		uint32_t inc_s = wave_inclusive_scan(s, lane);
+		uint32_t inc_b = wave_inclusive_scan(b, lane);
+		if (lane == 63) {
+			wave_small[wave] = inc_s;
+			wave_big[wave] = inc_b;
+		}
+		__syncthreads();
+		uint32_t off_s = 0, off_b = 0, tot_s = 0, tot_b = 0;
+		for (uint32_t w = 0; w < kScanThreads / 64; w++) {
+			uint32_t ws = wave_small[w], wb = wave_big[w];
+			if (w < wave) {
+				off_s += ws;
+				off_b += wb;
+			}
+			tot_s += ws;
+			tot_b += wb;
+		}
+		if (t < num_tiles) {
+			uint32_t ex_s = (carry_small + off_s + inc_s - s) % num_rails;
+			uint32_t ex_b = (carry_big + off_b + inc_b - b) % num_rails;
+			tile_prefix[t] = (ex_s << 16) | ex_b;
+		}
+		carry_small = (carry_small + tot_s) % num_rails;
+		carry_big = (carry_big + tot_b) % num_rails;
+		__syncthreads();
+	}
+	if (threadIdx.x == 0) {
+		state->rr_small_counter = carry_small;
+		state->rr_counter = carry_big;
+	}
+}
+
+__global__ __launch_bounds__(kThreads) void stripe_emit_kernel(
+	const uint64_t *__restrict__ sizes, uint32_t n, const ofi_amd_sched_state_t *__restrict__ state,
+	uint64_t align, const uint32_t *__restrict__ tile_prefix, uint32_t *__restrict__ num_xfers,
+	u32x4 *__restrict__ xfers)
+{
+	params_t p;
+	if (!load_params(state, align, p)) {
+		return;
+	}
+	/* 256 rows of 96 bytes = 6 x 16 B each */
+	__shared__ u32x4 rows[kThreads * 6];
+	__shared__ uint32_t wave_sum[kThreads / 64];
+	const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+	const uint32_t base = blockIdx.x * kTile;
+	const uint32_t R = p.num_rails;
+
+	uint32_t seed = tile_prefix[blockIdx.x];
+	uint32_t carry_small = seed >> 16, carry_big = seed & 0xffffu; /* both < R */
+
+	for (uint32_t pass = 0; pass < kPasses; pass++) {
+		const uint32_t first = base + pass * kThreads;
+		if (first >= n) {
+			break;
+		}
+		const uint32_t i = first + threadIdx.x;
+		const bool live = i < n;
+		const uint64_t size = live ? sizes[i] : 0;
+		uint32_t k = 0;
+		const uint32_t c = live ? contribution(size, p, k) : 0;
+
+		uint32_t inc = wave_inclusive_scan(c, lane);
+		if (lane == 63) {
+			wave_sum[wave] = inc;
+		}
+		__syncthreads();
+		uint32_t off = 0, tot = 0;
+#pragma unroll
+		for (uint32_t w = 0; w < kThreads / 64; w++) {
+			uint32_t ws = wave_sum[w];
+			off += (w < wave) ? ws : 0;
+			tot += ws;
+		}
+		const uint32_t excl = off + inc - c;
+
+		/* set_schedule_by_threshold, src/nccl_ofi_scheduler.cpp:77-133 */
+		const bool small = (c >> 16) != 0;
+		uint32_t rail = small ? (carry_small + (excl >> 16)) % R
+				      : (carry_big + (excl & 0xffffu)) % R;
+		uint64_t max_stripe = size;
+		if (!small) {
+			uint64_t per = size == 0 ? 0 : 1 + div_small(size - 1, k);
+			max_stripe = div_ceil_by(per, p.align, p.align_shift) * p.align;
+		}
+		uint64_t left = size, offset = 0;
+		u32x4 *row = &rows[threadIdx.x * 6];
+		uint64_t f[12]; /* 4 x {rail word, offset, msg_size} */
+#pragma unroll
+		for (uint32_t s = 0; s < 4; s++) {
+			if (live && s < k) {
+				uint64_t stripe = left < max_stripe ? left : max_stripe;
+				f[3 * s + 0] = rail; /* rail_id in the low 16 bits, padding zero */
+				f[3 * s + 1] = offset;
+				f[3 * s + 2] = stripe;
+				offset += stripe;
+				left -= stripe;
+				rail = (rail + 1) % R;
+			} else {
+				f[3 * s + 0] = 0;
+				f[3 * s + 1] = 0;
+				f[3 * s + 2] = 0;
+			}
+		}
+#pragma unroll
+		for (uint32_t q = 0; q < 6; q++) {
+			u32x4 v;
+			v.x = (uint32_t)f[2 * q];
+			v.y = (uint32_t)(f[2 * q] >> 32);
+			v.z = (uint32_t)f[2 * q + 1];
+			v.w = (uint32_t)(f[2 * q + 1] >> 32);
+			row[q] = v;
+		}
+		if (live) {
+			num_xfers[i] = k;
+		}
+		__syncthreads();
+
+		/* coalesced write-out of the tile's rows */
+		const uint32_t valid = (n - first) < kThreads ? (n - first) : kThreads;
+		u32x4 *out = xfers + (uint64_t)first * 6;
+		for (uint32_t v = threadIdx.x; v < valid * 6; v += kThreads) {
+			__builtin_nontemporal_store(rows[v], &out[v]);
+		}
+
+		carry_small = (carry_small + (tot >> 16)) % R;
+		carry_big = (carry_big + (tot & 0xffffu)) % R;
+		__syncthreads();
+	}
+}
+
+/* Per-process scratch for tile totals / prefixes, grown on demand. */
+struct workspace_t {
+	std::mutex lock;
+	uint32_t *totals = nullptr;
+	uint32_t *prefix = nullptr;
+	uint32_t tiles = 0;
+};
+workspace_t g_ws;
+
+} // namespace
+
+using namespace ofi_amd;
+
+extern "C" {
+
+int ofi_amd_sched_batch(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes, uint64_t n,
+			uint64_t align, uint32_t *d_num_xfers, ofi_amd_xfer_info_t *d_xfers,
+			void *stream)
+{
+	int rc = require_device();
+	if (rc != 0) {
+		return rc;
+	}
+	if (!d_state || align == 0 || n > kMaxBatch) {
+		return -EINVAL;
+	}
+	if (n == 0) {
+		return 0;
+	}
+	if (!d_sizes || !d_num_xfers || !d_xfers) {
+		return -EINVAL;
+	}
+
+	uint32_t *err = async_error_word();
+	if (!err) {
+		return -ENOMEM;
+	}
+
+	const uint32_t tiles = (uint32_t)((n + kTile - 1) / kTile);
+	uint32_t *totals, *prefix;
+	{
+		std::lock_guard<std::mutex> g(g_ws.lock);
+		if (tiles > g_ws.tiles) {
+			uint32_t want = tiles < 4096 ? 4096 : tiles;
+			uint32_t *a = nullptr, *b = nullptr;
+			OFI_AMD_HIP_TRY(hipMalloc((void **)&a, sizeof(uint32_t) * want));
+			if (hipMalloc((void **)&b, sizeof(uint32_t) * want) != hipSuccess) {
+				(void)hipFree(a);
+				return -ENOMEM;
+			}
+			/* older buffers may still be in use by queued launches: sync first */
+			(void)hipDeviceSynchronize();
+			(void)hipFree(g_ws.totals);
+			(void)hipFree(g_ws.prefix);
+			g_ws.totals = a;
+			g_ws.prefix = b;
+			g_ws.tiles = want;
+		}
+		totals = g_ws.totals;
+		prefix = g_ws.prefix;
+	}
+
+	hipStream_t s = as_stream(stream);
+	hipLaunchKernelGGL(stripe_count_kernel, dim3(tiles), dim3(kThreads), 0, s, d_sizes,
+			   (uint32_t)n, d_state, align, totals);
+	hipLaunchKernelGGL(stripe_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, totals, tiles,
+			   d_state, prefix, err);
+	hipLaunchKernelGGL(stripe_emit_kernel, dim3(tiles), dim3(kThreads), 0, s, d_sizes,
+			   (uint32_t)n, d_state, align, prefix, d_num_xfers,
+			   reinterpret_cast<u32x4 *>(d_xfers));
+	OFI_AMD_HIP_TRY(hipGetLastError());
+	return 0;
+}
+
+/* Host form: one get_schedule() call, src/nccl_ofi_scheduler.cpp:77-133. */
+int ofi_amd_sched_get_schedule(ofi_amd_sched_state_t *st, uint64_t size, uint64_t align,
+			       ofi_amd_xfer_info_t *xfers)
+{
+	if (!st || !xfers || st->num_rails < 1 || st->num_rails > OFI_AMD_MAX_NUM_RAILS ||
+	    st->min_stripe_size == 0 || align == 0) {
+		return -EINVAL;
+	}
+	const uint32_t R = (uint32_t)st->num_rails;
+	auto ceil_div = [](uint64_t x, uint64_t y) -> uint64_t { return x == 0 ? 0 : 1 + (x - 1) / y; };
+
+	if (size < st->max_small_msg_size) {
+		xfers[0] = ofi_amd_xfer_info_t{(uint16_t)st->rr_small_counter, 0, 0, 0, size};
+		st->rr_small_counter = (st->rr_small_counter + 1) % R;
+		return 1;
+	}
+	uint64_t want = ceil_div(size, st->min_stripe_size);
+	uint32_t n = (uint32_t)(want < R ? want : R);
+	n = n > 1 ? n : 1;
+	for (uint32_t i = n; i > 1; i--) {
+		if (R % i == 0) {
+			n = i;
+			break;
+		}
+	}
+	uint32_t rail = st->rr_counter;
+	st->rr_counter = (st->rr_counter + n) % R;
+	const uint64_t max_stripe = ceil_div(ceil_div(size, n), align) * align;
+	uint64_t left = size, offset = 0;
+	for (uint32_t k = 0; k < n; k++) {
+		uint64_t stripe = left < max_stripe ? left : max_stripe;
+		xfers[k] = ofi_amd_xfer_info_t{(uint16_t)rail, 0, 0, offset, stripe};
+		offset += stripe;
+		left -= stripe;
+		rail = (rail + 1) % R;
+	}
+	return (int)n;
+}
+
+} /* extern "C" */

@@ -1,0 +1,356 @@
+/*
+ * C ABI of libofi_amd_hotpath.so: the gfx950 (MI355X) implementation of the
+ * data-parallel hot path of the OFI NCCL/RCCL network plugin.
+ *
+ * Conventions (those of the reference's internal GPU layer,
+ * include/nccl_ofi_rocm.h:11-63): every function returns 0 on success or a
+ * negative errno; no exception and no HIP type crosses this boundary.  A
+ * `stream` argument is a hipStream_t passed as void* (NULL = the default
+ * stream).  Pointers named d_* must be device-accessible (HBM or pinned host
+ * memory); all others are ordinary host pointers.  Every entry point that needs
+ * the GPU returns -ENODEV when no device is present; nothing falls back to the
+ * CPU.
+ */
+#ifndef OFI_AMD_HOTPATH_H_
+#define OFI_AMD_HOTPATH_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OFI_AMD_MAX_NUM_RAILS 4 /* MAX_NUM_RAILS, include/nccl_ofi_rdma.h:37 */
+
+/* ======================================================================
+ * 1. GPU runtime glue: replaces src/nccl_ofi_rocm.cpp (8 functions of
+ *    include/nccl_ofi_rocm.h:11-63) and covers the CUDA-only calls GIN needs
+ *    (include/nccl_ofi_cuda.h:34-139).
+ * ====================================================================== */
+
+/* nccl_net_ofi_gpu_init, include/nccl_ofi_rocm.h:12 */
+int ofi_amd_gpu_init(void);
+/* nccl_net_ofi_get_gpu_device_for_addr, :25.  Unlike the ROCm stub of the
+ * reference (src/nccl_ofi_rocm.cpp:58-76, always -1) this reports the ordinal. */
+int ofi_amd_gpu_get_device_for_addr(void *data, int *dev_id);
+/* nccl_net_ofi_gpu_flush_gpudirect_rdma_writes, :32.  -EPERM: not available,
+ * callers use the read-back flush (ofi_amd_flush_read) instead. */
+int ofi_amd_gpu_flush_gpudirect_rdma_writes(void);
+/* nccl_net_ofi_gpu_mem_alloc / _free / _copy_host_to_device, :39-53 */
+int ofi_amd_gpu_mem_alloc(void **ptr, size_t size);
+int ofi_amd_gpu_mem_free(void *ptr);
+int ofi_amd_gpu_mem_copy_host_to_device(void *dst, const void *src, size_t size);
+/* nccl_net_ofi_gpu_get_dma_buf_fd, :60 */
+int ofi_amd_gpu_get_dma_buf_fd(void *aligned_ptr, size_t aligned_size, int *fd, size_t *offset);
+/* nccl_net_ofi_gpu_have_dma_buf_attr / _have_gdr_support_attr, :62-63 (1/0) */
+int ofi_amd_gpu_have_dma_buf_attr(void);
+int ofi_amd_gpu_have_gdr_support_attr(void);
+/* nccl_net_ofi_gpu_set/get_current_context, include/nccl_ofi_cuda.h:50-60.
+ * HIP has no driver contexts; the "context" is the device ordinal. */
+int ofi_amd_gpu_set_current_device(int dev_id);
+int ofi_amd_gpu_get_current_device(int *dev_id);
+/* nccl_net_ofi_gpu_get_address_range, include/nccl_ofi_cuda.h:71 */
+int ofi_amd_gpu_get_address_range(void *ptr, void **base_out, size_t *size_out);
+/* nccl_net_ofi_gpu_seg_is_host, include/nccl_ofi_cuda.h:82 */
+int ofi_amd_gpu_seg_is_host(void *seg_base, int *is_host_out);
+/* Pinned host memory the GPU can address.  Stands in for
+ * nccl_net_ofi_gpu_host_register_iomem / _host_unregister
+ * (include/nccl_ofi_cuda.h:107-113): memory is allocated pinned rather than
+ * registered after the fact. */
+int ofi_amd_gpu_host_alloc(void **ptr, size_t size);
+int ofi_amd_gpu_host_free(void *ptr);
+/* nccl_net_ofi_gpu_host_get_device_pointer, include/nccl_ofi_cuda.h:121 */
+int ofi_amd_gpu_host_get_device_pointer(void **dev_ptr, void *host_ptr);
+int ofi_amd_gpu_mem_copy_device_to_host(void *dst, const void *src, size_t size);
+int ofi_amd_gpu_stream_synchronize(void *stream);
+/* Kernels that skip work because a documented precondition does not hold (a
+ * destination range outside the arena, a producer giving up on a full ring) set
+ * a bit in a library-owned pinned word.  Fetch-and-clear it after synchronising:
+ * bit 0 = bounce destination out of range / misaligned, bit 1 = GIN producer
+ * timed out, bit 2 = scheduler state unusable (num_rails outside 1..4 or a zero
+ * min_stripe_size; the batch is then left unwritten). */
+int ofi_amd_async_error_fetch(uint32_t *bits);
+
+/* ======================================================================
+ * 2. Rail striping (threshold scheduler), batched.
+ *    Replaces per-message nccl_net_ofi_threshold_scheduler::get_schedule,
+ *    src/nccl_ofi_scheduler.cpp:47-190.
+ * ====================================================================== */
+
+/* nccl_net_ofi_xfer_info_t, include/nccl_ofi_scheduler.h:20-27 (24 bytes) */
+typedef struct {
+	uint16_t rail_id;
+	uint16_t pad0;
+	uint32_t pad1;
+	uint64_t offset;
+	uint64_t msg_size;
+} ofi_amd_xfer_info_t;
+
+/* Scheduler state, include/nccl_ofi_scheduler.h:115-121.  Lives in device
+ * memory so consecutive batches chain on a stream without a host round trip. */
+typedef struct {
+	uint32_t rr_small_counter;
+	uint32_t rr_counter;
+	uint64_t max_small_msg_size; /* OFI_NCCL_SCHED_MAX_SMALL_MSG_SIZE, default 64 */
+	uint64_t min_stripe_size;    /* OFI_NCCL_MIN_STRIPE_SIZE, default 131072 */
+	int32_t num_rails;           /* 1..4 */
+	int32_t pad;
+} ofi_amd_sched_state_t;
+
+/*
+ * Schedules d_sizes[0..n) in index order, exactly as n consecutive
+ * get_schedule(size, num_rails) calls on one scheduler would, and advances the
+ * two round-robin counters in *d_state.  Output is fixed width:
+ * d_num_xfers[i] = number of stripes, d_xfers[4*i .. 4*i+3] = the stripes
+ * (unused entries all-zero).  align is the stripe alignment (128 in the
+ * reference, src/nccl_ofi_scheduler.cpp:168).  n <= 2^28 per call.
+ */
+int ofi_amd_sched_batch(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes, uint64_t n,
+			uint64_t align, uint32_t *d_num_xfers, ofi_amd_xfer_info_t *d_xfers,
+			void *stream);
+
+/* Host-side single-message form with the reference's semantics, for per-op
+ * callers (the GIN proxy).  `state` is a host struct. Returns the stripe count. */
+int ofi_amd_sched_get_schedule(ofi_amd_sched_state_t *state, uint64_t size, uint64_t align,
+			       ofi_amd_xfer_info_t *xfers);
+
+/* ======================================================================
+ * 3. Bounce / eager copy and flush, batched, plus the device-copy interface.
+ *    Replaces one loop-back fi_read per eager buffer
+ *    (rdma_eager_copy_req::post, src/nccl_ofi_rdma.cpp:2729-2776) and the
+ *    read-back flush (rdma_flush_req::post, :2664-2713).
+ * ====================================================================== */
+
+/*
+ * For i in [0,n): copies d_len[i] bytes from d_src + d_src_off[i] to
+ * d_arena + d_dst_off[i] (d_dst_off[i] 64-byte aligned, destination ranges
+ * disjoint, each inside [0, arena_bytes)), then, if d_flush is not NULL, reads
+ * back the first 4 bytes at each destination into d_flush[i] (device or pinned
+ * host memory) after the copy is visible device-wide.  No byte outside the
+ * destination ranges is written.
+ */
+int ofi_amd_bounce_scatter(const void *d_src, void *d_arena, uint64_t arena_bytes,
+			   const uint64_t *d_src_off, const uint64_t *d_dst_off,
+			   const uint32_t *d_len, uint32_t n, uint32_t *d_flush, void *stream);
+
+/* Flush only: d_flush[i] = 4 bytes at d_arena + d_dst_off[i], read with
+ * device-scope acquire semantics (the C5 read-back without a copy). */
+int ofi_amd_flush_read(const void *d_arena, const uint64_t *d_dst_off, uint32_t n,
+		       uint32_t *d_flush, void *stream);
+
+/* nccl_ofi_device_copy, include/nccl_ofi_device_copy.h:14-69: register a device
+ * region, then small synchronous host<->device copies at an offset. */
+typedef struct ofi_amd_devcopy_region ofi_amd_devcopy_region_t;
+int ofi_amd_devcopy_register(void *device_ptr, size_t size, ofi_amd_devcopy_region_t **out);
+int ofi_amd_devcopy_to_device(const void *host_ptr, ofi_amd_devcopy_region_t *h, size_t offset,
+			      size_t size);
+int ofi_amd_devcopy_from_device(ofi_amd_devcopy_region_t *h, size_t offset, void *host_ptr,
+				size_t size);
+int ofi_amd_devcopy_forced_pcie_copy(void); /* 0: no alternative path to force */
+int ofi_amd_devcopy_deregister(ofi_amd_devcopy_region_t *h);
+
+/* ======================================================================
+ * 4. GIN put / put-signal descriptors: GPU producers, pinned-host rings,
+ *    host proxy.  Ring protocol of include/nccl_ofi_mpsc_ring.h:56-163; the
+ *    descriptor is the argument tuple of iputSignal
+ *    (include/nccl_ofi_gin_base.h:83-91); what the proxy derives from it
+ *    follows src/rdma/gin/nccl_ofi_gin.cpp:568-864.
+ * ====================================================================== */
+
+typedef struct {
+	uint64_t src_off;
+	uint64_t dst_off;
+	uint64_t size;
+	uint64_t signal_off;
+	uint64_t signal_value;
+	uint32_t rank;
+	uint32_t signal_op;  /* 0 none, 1 INC, 2 ADD (nccl/net.h:28-29) */
+	uint32_t opt_flags;  /* bit 0: aggregate (nccl/rma_v15.h:19-21) */
+	uint32_t context;
+	uint16_t src_mr;
+	uint16_t dst_mr;
+	uint16_t sig_mr;     /* 0xffff: no signal handle */
+	uint16_t kind;       /* 1 put, 2 put-signal */
+} ofi_amd_gin_desc_t;    /* 64 bytes */
+
+typedef struct ofi_amd_gin_rings ofi_amd_gin_rings_t;
+
+/* n_contexts rings of `capacity` (power of two, >= 64) descriptors each, in
+ * pinned host memory: record array (64 B each) + sequence array (u32 each). */
+int ofi_amd_gin_rings_create(uint32_t n_contexts, uint32_t capacity, ofi_amd_gin_rings_t **out);
+int ofi_amd_gin_rings_destroy(ofi_amd_gin_rings_t *rings);
+/* Raw views for tests / external consumers (host addresses of pinned memory). */
+int ofi_amd_gin_rings_view(ofi_amd_gin_rings_t *rings, void **records, uint32_t **sequences,
+			   uint32_t *n_contexts, uint32_t *capacity);
+
+/*
+ * Launches the synthetic producer: one workgroup per context, each emitting
+ * ops_per_context descriptors of the seeded stream in op order (slot =
+ * position & (capacity-1), publication by release-store of position+1 to the
+ * slot's sequence word).  Returns right after the launch; a host proxy must be
+ * draining concurrently or the kernel gives up after spin_limit polls of a
+ * still-occupied slot (0 = default) and ofi_amd_gin_producer_status reports
+ * -ETIMEDOUT.
+ */
+int ofi_amd_gin_produce_seeded(ofi_amd_gin_rings_t *rings, uint64_t seed,
+			       uint64_t ops_per_context, uint32_t peer_rank,
+			       uint32_t signal_every, uint32_t signal_op, uint32_t aggregate_mask,
+			       uint64_t spin_limit, void *stream);
+/* After the stream has been synchronised: 0, or -ETIMEDOUT if any producer gave up. */
+int ofi_amd_gin_producer_status(ofi_amd_gin_rings_t *rings);
+
+/* Host-side push with the same protocol (CPU producer threads; CAS claim as in
+ * nccl_ofi_mpsc_ring::push).  1 pushed, 0 full. */
+int ofi_amd_gin_ring_push(ofi_amd_gin_rings_t *rings, uint32_t context,
+			  const ofi_amd_gin_desc_t *desc);
+/* Single pop (nccl_ofi_mpsc_ring::pop).  1 popped, 0 empty. */
+int ofi_amd_gin_ring_pop(ofi_amd_gin_rings_t *rings, uint32_t context, ofi_amd_gin_desc_t *desc);
+
+/* Memory registration table entry the proxy resolves descriptor handles with
+ * (gin_remote_mr, include/rdma/gin/nccl_ofi_gin.h:168-183). */
+typedef struct {
+	uint64_t local_base;
+	uint64_t remote_address;
+	uint64_t remote_address_offset;
+	uint64_t key[OFI_AMD_MAX_NUM_RAILS];
+} ofi_amd_gin_mr_t;
+
+/* One RDMA write the proxy would post (fi_writemsg arguments minus libfabric handles). */
+typedef struct {
+	uint64_t src;
+	uint64_t len;
+	uint64_t dest;
+	uint64_t key;
+	uint32_t rail;
+	uint32_t more; /* FI_MORE */
+} ofi_amd_gin_write_t;
+
+/* Everything iputSignal derives from one descriptor (192 bytes). */
+typedef struct {
+	uint32_t seq;
+	uint32_t nseg;
+	uint32_t imm;        /* GIN_IMM_SEG_DATA, include/rdma/gin/nccl_ofi_gin_types.h:76-79 */
+	uint32_t num_writes;
+	uint32_t has_meta;
+	uint32_t meta_rail;
+	uint32_t meta_more;
+	uint32_t ack_req;
+	ofi_amd_gin_write_t writes[OFI_AMD_MAX_NUM_RAILS];
+	uint64_t meta[4];    /* nccl_net_ofi_gin_signal_metadata_msg_t, :150-159 */
+} ofi_amd_gin_wire_t;
+
+/* Initiator-side comm state (nccl_ofi_gin_peer_rank_info,
+ * include/rdma/gin/nccl_ofi_gin.h:111-163, plus pin state). */
+typedef struct {
+	ofi_amd_sched_state_t sched;
+	uint32_t comm_id;
+	uint32_t num_rails;
+	uint32_t tx_head;
+	uint32_t tx_tail;
+	uint32_t consecutive_puts_without_ack;
+	uint32_t last_ack_requested_seq;
+	uint32_t has_pending_ack_request;
+	int32_t pinned_rail_id;
+	uint32_t pinned_rail_run;
+	uint32_t next_rail_id;
+	uint32_t ack_model; /* 0: ACKs only via ofi_amd_gin_apply_ack; 1: immediate ACK on request */
+	uint32_t pad;
+} ofi_amd_gin_comm_t;
+
+int ofi_amd_gin_comm_init(ofi_amd_gin_comm_t *c, uint32_t comm_id, uint32_t num_rails,
+			  uint64_t min_stripe, uint64_t max_small, uint32_t ack_model);
+/* iputSignal's derivation for one descriptor.  0, -EINVAL (signal op),
+ * -EAGAIN (TX window full; the reference blocks in await_tx_window). */
+int ofi_amd_gin_iput_signal(ofi_amd_gin_comm_t *c, const ofi_amd_gin_mr_t *mrs,
+			    const ofi_amd_gin_desc_t *d, ofi_amd_gin_wire_t *out);
+/* apply_rx_consumed, include/rdma/gin/nccl_ofi_gin.h:535-543 */
+void ofi_amd_gin_apply_ack(ofi_amd_gin_comm_t *c, uint32_t wire_rx_consumed);
+/* Wire encoders, include/rdma/gin/nccl_ofi_gin_types.h:39-181 */
+uint32_t ofi_amd_gin_imm(uint32_t comm_id, uint32_t seq, uint32_t nseg, uint32_t ack_req);
+uint64_t ofi_amd_gin_meta_header(uint32_t comm_id, uint32_t seq, uint32_t nseg, uint32_t ack_req);
+uint64_t ofi_amd_gin_ack_msg(uint32_t comm_id, uint32_t rx_consumed);
+
+typedef struct {
+	uint64_t descriptors;   /* drained in this call */
+	uint64_t signals;       /* of which put-signal */
+	uint64_t writes;        /* RDMA writes derived (mode 2) */
+	uint64_t checksum;      /* order-sensitive per context, summed over contexts */
+	double seconds;         /* wall time from first poll to last descriptor */
+	uint64_t empty_polls;
+} ofi_amd_gin_proxy_stats_t;
+
+/*
+ * The host proxy loop, on the calling thread: drains all rings round-robin until
+ * each has delivered ops_per_context descriptors, or timeout_ms passes without
+ * progress (-ETIMEDOUT).
+ *   mode 0: pop + fold every descriptor into the checksum;
+ *   mode 1: also store the descriptors: out_desc[c * ops_per_context + i];
+ *   mode 2: also run the iputSignal derivation per context (comms[c], mrs) and
+ *           fold the wire records into the checksum; out_wire (may be NULL)
+ *           receives them at [c * ops_per_context + i].
+ */
+int ofi_amd_gin_proxy_drain(ofi_amd_gin_rings_t *rings, uint64_t ops_per_context, int mode,
+			    ofi_amd_gin_desc_t *out_desc, ofi_amd_gin_comm_t *comms,
+			    const ofi_amd_gin_mr_t *mrs, ofi_amd_gin_wire_t *out_wire,
+			    uint32_t timeout_ms, ofi_amd_gin_proxy_stats_t *stats);
+
+/* ======================================================================
+ * 5. Tuner: batched cost model and region lookup.
+ *    Model: nccl_ofi_tuner_compute_cost + model_get_coll_info_internal_v3,
+ *    src/tuner/nccl_ofi_model.cpp:46-234.  Regions:
+ *    region_get_coll_info_internal_v3, src/tuner/nccl_ofi_regions.cpp:2070-2157.
+ * ====================================================================== */
+
+enum {
+	OFI_AMD_PLATFORM_P5_P5E = 0, /* enum nccl_ofi_tuner_platform, */
+	OFI_AMD_PLATFORM_P5EN = 1,   /* include/tuner/nccl_ofi_tuner_common.h:18-25 */
+	OFI_AMD_PLATFORM_P6 = 2,
+	OFI_AMD_PLATFORM_P6_B300 = 3,
+};
+
+/* One grid variant: everything that is fixed per tuner context / call. */
+typedef struct {
+	int32_t platform;
+	int32_t pipe_ops;          /* numPipeOps */
+	int32_t num_channels;      /* OFI_NCCL_TUNER_NUM_CHANNELS, default 8 */
+	int32_t net_comp_overhead; /* OFI_NCCL_TUNER_NET_COMP_OVERHEAD, default 3 */
+} ofi_amd_tuner_variant_t;
+
+typedef struct ofi_amd_tuner_plan ofi_amd_tuner_plan_t;
+
+/*
+ * A plan fixes the grid axes (host arrays, copied): collectives (ncclFunc_t
+ * values), message sizes, node counts, ranks-per-node values, and the
+ * algorithm list whose cost cells are emitted (all three protocols each).
+ * Point index = ((coll * n_sizes + size) * n_nodes + node) * n_ppn + ppn.
+ */
+int ofi_amd_tuner_plan_create(const int32_t *colls, uint32_t n_colls, const uint64_t *sizes,
+			      uint32_t n_sizes, const uint64_t *nodes, uint32_t n_nodes,
+			      const uint32_t *ppn, uint32_t n_ppn, const int32_t *algos,
+			      uint32_t n_algos, ofi_amd_tuner_plan_t **out);
+int ofi_amd_tuner_plan_destroy(ofi_amd_tuner_plan_t *plan);
+uint64_t ofi_amd_tuner_plan_points(const ofi_amd_tuner_plan_t *plan);
+uint64_t ofi_amd_tuner_plan_cells(const ofi_amd_tuner_plan_t *plan); /* points * n_algos * 3 */
+
+/*
+ * Model grid for n_variants variants in one launch.
+ *   d_cost[v * cells + point * n_algos * 3 + a * 3 + proto]  (fp64 of the fp32 cost, -1 = no model)
+ *   d_choice[(v * points + point) * 2 + {0,1}] = chosen {algo, proto} or {-1,-1}
+ * Either output may be NULL.
+ */
+int ofi_amd_tuner_model_grid(ofi_amd_tuner_plan_t *plan, const ofi_amd_tuner_variant_t *variants,
+			     uint32_t n_variants, double *d_cost, int8_t *d_choice, void *stream);
+
+/*
+ * Region grid for n_platforms platforms in one launch.
+ *   d_choice[(p * points + point) * 4 + {0,1}] = {algo, proto} or {-1,-1} (fall back to NCCL),
+ *   bytes 2..3 = int16 nChannels override, or -1 when the tuner leaves nChannels alone.
+ */
+int ofi_amd_tuner_region_grid(ofi_amd_tuner_plan_t *plan, const int32_t *platforms,
+			      uint32_t n_platforms, int8_t *d_choice, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OFI_AMD_HOTPATH_H_ */

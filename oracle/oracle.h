@@ -1,0 +1,229 @@
+/*
+ * CPU oracle: a scalar restatement of the aws-ofi-nccl algorithms on the hot
+ * path, one function per reference function, each citing the reference
+ * file:line it follows.
+ *
+ * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  Only the test-suite, the
+ * smoke check and the benchmark's cpu_baseline leg load liboracle.so, and only
+ * as the checker / timed baseline.  Nothing under aws_ofi_nccl_amd/ links or
+ * calls it.
+ *
+ * Parity status of each function (what pins it beyond reading the code):
+ *   scheduler        24 known answers of tests/unit/scheduler.cpp:126-309, plus
+ *                    invariants and brute force vs an independent big-int model
+ *   mpsc/spsc ring   reference headers compiled as-is (oracle/_ref) and driven
+ *                    side by side; behaviour cases of tests/unit/mpsc_ring.cpp
+ *   gin imm/meta/ack reference macros + bit-field structs compiled as-is
+ *                    (oracle/_ref), encode/decode cross-checked field by field
+ *   gin iputSignal   state machine (window, pin, FI_MORE flags): PARITY UNPINNED
+ *                    beyond the encoders above -- the reference has no
+ *                    wire-level test for it and its source does not build here
+ *   region geometry  ~70 points + 4 extend_region cases of
+ *                    tests/unit/region_based_tuner.cpp
+ *   region tables    re-parsed from the reference source text and compared
+ *   region decisions full-grid fp bits: PARITY UNPINNED (reference object not
+ *                    buildable here); pinned only through the two rows above
+ *   model cost       exact-rational closed forms to 1e-6 rel., linearity and
+ *                    protocol-ratio identities; exact fp32 bit pattern of the
+ *                    reference binary: PARITY UNPINNED (not buildable here)
+ *   bounce copy      memcpy semantics; patterns of tests/unit/gdrcopy.cpp:15-133
+ */
+#ifndef ORACLE_H_
+#define ORACLE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ORACLE_MAX_RAILS 4
+
+/* ---------------------------------------------------------------- scheduler */
+
+/* Same field order and padding as nccl_net_ofi_xfer_info_t
+ * (include/nccl_ofi_scheduler.h:20-27): 24 bytes. */
+typedef struct {
+	uint16_t rail_id;
+	uint16_t pad0;
+	uint32_t pad1;
+	uint64_t offset;
+	uint64_t msg_size;
+} oracle_xfer_t;
+
+/* State of nccl_net_ofi_threshold_scheduler (include/nccl_ofi_scheduler.h:115-121). */
+typedef struct {
+	uint32_t rr_small_counter;
+	uint32_t rr_counter;
+	uint64_t max_small_msg_size;
+	uint64_t min_stripe_size;
+	int32_t num_rails;
+	int32_t pad;
+} oracle_sched_t;
+
+void oracle_sched_init(oracle_sched_t *s, int num_rails, uint64_t min_stripe_size,
+		       uint64_t max_small_msg_size);
+int oracle_sched_num_stripes(const oracle_sched_t *s, uint64_t size);
+/* One get_schedule() call; writes up to num_rails entries, returns the count. */
+int oracle_sched_get_schedule(oracle_sched_t *s, uint64_t size, uint64_t align,
+			      oracle_xfer_t *xfers);
+/* n calls in index order on one instance.  Output is fixed width: num_xfers[i]
+ * and xfers[i*4 .. i*4+3], unused entries zero. */
+void oracle_sched_batch(oracle_sched_t *s, const uint64_t *sizes, uint64_t n, uint64_t align,
+			uint32_t *num_xfers, oracle_xfer_t *xfers);
+/* The same loop with one heap allocation + free per message, mirroring the
+ * reference's freelist alloc per schedule (src/nccl_ofi_scheduler.cpp:172). */
+void oracle_sched_batch_alloc(oracle_sched_t *s, const uint64_t *sizes, uint64_t n,
+			      uint64_t align, uint32_t *num_xfers, oracle_xfer_t *xfers);
+
+/* ------------------------------------------------------------- bounce copy */
+
+/* Batched eager copy (src/nccl_ofi_rdma.cpp:2729-2776 semantics, one call per
+ * buffer there): arena[dst_off[i] .. +len[i]) = src[src_off[i] .. +len[i]).
+ * flush[i] = first 4 bytes at arena+dst_off[i] read after the copy (little
+ * endian, zero-extended when len[i] < 4 reads whatever the arena holds). */
+void oracle_bounce_scatter(const uint8_t *src, uint8_t *arena, const uint64_t *src_off,
+			   const uint64_t *dst_off, const uint32_t *len, uint32_t n,
+			   uint32_t *flush);
+
+/* ------------------------------------------------------------------- rings */
+
+typedef struct oracle_mpsc oracle_mpsc_t;
+oracle_mpsc_t *oracle_mpsc_create(uint32_t capacity, uint32_t payload_bytes);
+void oracle_mpsc_destroy(oracle_mpsc_t *r);
+int oracle_mpsc_push(oracle_mpsc_t *r, const void *entry); /* 1 pushed, 0 full */
+int oracle_mpsc_pop(oracle_mpsc_t *r, void *entry);        /* 1 popped, 0 empty */
+/* For tests: place both cursors at `pos` (sequence words re-seeded accordingly). */
+void oracle_mpsc_set_positions(oracle_mpsc_t *r, uint32_t pos);
+
+typedef struct oracle_spsc oracle_spsc_t;
+oracle_spsc_t *oracle_spsc_create(uint32_t capacity, uint32_t payload_bytes);
+void oracle_spsc_destroy(oracle_spsc_t *r);
+int oracle_spsc_push(oracle_spsc_t *r, const void *entry);
+int oracle_spsc_pop(oracle_spsc_t *r, void *entry);
+
+/* --------------------------------------------------------------------- GIN */
+
+/* The 64-byte put / put-signal descriptor: the argument tuple of iputSignal
+ * (include/nccl_ofi_gin_base.h:83-91, nccl/rma_v15.h:43-50). */
+typedef struct {
+	uint64_t src_off;
+	uint64_t dst_off;
+	uint64_t size;
+	uint64_t signal_off;
+	uint64_t signal_value;
+	uint32_t rank;
+	uint32_t signal_op;
+	uint32_t opt_flags;
+	uint32_t context;
+	uint16_t src_mr;
+	uint16_t dst_mr;
+	uint16_t sig_mr;
+	uint16_t kind;
+} oracle_gin_desc_t;
+
+uint32_t oracle_gin_imm(uint32_t comm_id, uint32_t seq, uint32_t nseg, uint32_t ack_req);
+uint64_t oracle_gin_meta_header(uint32_t comm_id, uint32_t seq, uint32_t nseg, uint32_t ack_req);
+uint64_t oracle_gin_ack_msg(uint32_t comm_id, uint32_t rx_consumed);
+
+/* Counter-based synthetic op stream: descriptor i of context c under `seed`. */
+void oracle_gin_gen_desc(uint64_t seed, uint32_t context, uint64_t i, uint32_t peer_rank,
+			 uint32_t signal_every, uint32_t signal_op, uint32_t aggregate_mask,
+			 oracle_gin_desc_t *out);
+
+/* One fi_writemsg the reference would post (src/rdma/gin/nccl_ofi_gin.cpp:737-784). */
+typedef struct {
+	uint64_t src;
+	uint64_t len;
+	uint64_t dest;
+	uint64_t key;
+	uint32_t rail;
+	uint32_t more; /* FI_MORE set */
+} oracle_gin_write_t;
+
+/* Everything iputSignal derives from one descriptor. 192 bytes. */
+typedef struct {
+	uint32_t seq;
+	uint32_t nseg;
+	uint32_t imm;
+	uint32_t num_writes;
+	uint32_t has_meta;
+	uint32_t meta_rail;
+	uint32_t meta_more;
+	uint32_t ack_req;
+	oracle_gin_write_t writes[ORACLE_MAX_RAILS];
+	uint64_t meta[4];
+} oracle_gin_wire_t;
+
+/* Memory registration as the harness fixes it: local base address, the peer's
+ * address / address_offset, per-rail keys (include/rdma/gin/nccl_ofi_gin.h:168-183). */
+typedef struct {
+	uint64_t local_base;
+	uint64_t remote_address;
+	uint64_t remote_address_offset;
+	uint64_t key[ORACLE_MAX_RAILS];
+} oracle_gin_mr_t;
+
+typedef struct {
+	oracle_sched_t sched;
+	uint32_t comm_id;      /* remote comm id */
+	uint32_t num_rails;
+	uint32_t tx_head;
+	uint32_t tx_tail;
+	uint32_t consecutive_puts_without_ack;
+	uint32_t last_ack_requested_seq;
+	uint32_t has_pending_ack_request;
+	int32_t pinned_rail_id;
+	uint32_t pinned_rail_run;
+	uint32_t next_rail_id;
+	/* 0: ACKs never arrive (call fails with -11 once the window is full);
+	 * 1: the ACK for an ack-requesting op arrives right after that op. */
+	uint32_t ack_model;
+	uint32_t pad;
+} oracle_gin_comm_t;
+
+void oracle_gin_comm_init(oracle_gin_comm_t *c, uint32_t comm_id, uint32_t num_rails,
+			  uint64_t min_stripe, uint64_t max_small, uint32_t ack_model);
+/* src/rdma/gin/nccl_ofi_gin.cpp:568-864.  Returns 0, -22 (bad signal op) or
+ * -11 (window full and no ACK can arrive). */
+int oracle_gin_iput_signal(oracle_gin_comm_t *c, const oracle_gin_mr_t *mrs,
+			   const oracle_gin_desc_t *d, oracle_gin_wire_t *out);
+
+/* ------------------------------------------------------------------- tuner */
+
+enum { ORACLE_PLAT_P5_P5E = 0, ORACLE_PLAT_P5EN = 1, ORACLE_PLAT_P6 = 2, ORACLE_PLAT_P6_B300 = 3 };
+
+/* nccl_ofi_tuner_compute_cost, src/tuner/nccl_ofi_model.cpp:46-122. */
+float oracle_model_cost(int platform, int coll, int algo, int proto, int pipe_ops,
+			uint64_t size, uint64_t num_ranks, uint64_t num_nodes,
+			int num_channels, int net_comp_overhead);
+/* model_get_coll_info_internal_v3, :154-234.  algo and proto are -1 when nothing is chosen. */
+void oracle_model_decide(int platform, int coll, int pipe_ops, uint64_t size,
+			 uint64_t num_ranks, uint64_t num_nodes, int num_channels,
+			 int net_comp_overhead, int *algo, int *proto);
+
+typedef struct { double x, y; } oracle_point_t;
+/* extend_region, src/tuner/nccl_ofi_regions.cpp:254-289 (linear in, linear out). */
+oracle_point_t oracle_region_extend(oracle_point_t a, oracle_point_t b, oracle_point_t z);
+/* transform_log2, include/tuner/nccl_ofi_tuner_region.h:87-109. */
+oracle_point_t oracle_region_log2(oracle_point_t p);
+/* is_inside_region, :159-221; polygon and point in log2 space. */
+int oracle_region_inside(oracle_point_t p, const oracle_point_t *verts, size_t n);
+/* region_get_coll_info_internal_v3, :2070-2157, on a table with no ignored cell.
+ * algo and proto are -1 on fall-back; nchannels is left alone unless overridden. */
+void oracle_region_decide(int platform, int coll, uint64_t size, uint64_t num_ranks,
+			  uint64_t num_nodes, int *algo, int *proto, int *nchannels);
+/* Number of polygons and log2-space vertices for one (platform, shape, coll):
+ * used by tests to inspect the built table. Returns polygon count. */
+int oracle_region_polys(int platform, uint64_t num_ranks, uint64_t num_nodes, int coll,
+			int *algos, int *protos, int *nverts, oracle_point_t *verts, int max_polys);
+/* region_get_chunk_size_internal, :2276-2306.  Returns 1 when *chunk was set. */
+int oracle_region_chunk_size(int platform, int coll, uint64_t size, int algo, int proto,
+			     uint64_t num_ranks, uint64_t num_nodes, uint64_t *chunk);
+uint64_t oracle_chunk_tree_ll128(uint64_t message_size, int nchannels, int log2_nnodes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ORACLE_H_ */
