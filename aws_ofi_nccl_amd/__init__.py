@@ -53,7 +53,7 @@ class GinWrite(ctypes.Structure):
 
 
 class GinWire(ctypes.Structure):
-    """ofi_amd_gin_wire_t (192 bytes)"""
+    """ofi_amd_gin_wire_t (224 bytes)"""
     _fields_ = [("seq", c_u32), ("nseg", c_u32), ("imm", c_u32), ("num_writes", c_u32),
                 ("has_meta", c_u32), ("meta_rail", c_u32), ("meta_more", c_u32),
                 ("ack_req", c_u32), ("writes", GinWrite * 4), ("meta", c_u64 * 4)]

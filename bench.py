@@ -1,0 +1,317 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+A "step" is one pass of the batched bounce/eager copy + flush over the configured batch
+(65,536 eager buffers of 0..8 KiB, packed source, scattered to 64-byte-aligned offsets in a
+2 GiB HBM arena, one 4-byte flush read per buffer) with all inputs already resident in HBM.
+The same JSON line also reports the other three paths (rail striping, tuner grids, GIN
+descriptor production) and, for each, the scalar CPU restatement timed on this host.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-extra] [--skip-cpu]
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
+SEED = 1234
+
+
+def log(msg):
+    print("[bench] " + msg, file=sys.stderr, flush=True)
+
+
+def timed_steps(fn, steps, warmup, torch):
+    """W untimed + K timed launches; returns (wall ms/step, event ms/step) on the launch stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return wall, e0.elapsed_time(e1) / steps
+
+
+def bench_bounce(lib, oracle, torch, np, args):
+    import _gpu
+    import _oracle
+    from aws_ofi_nccl_amd import synthetic
+    w = synthetic.bounce_workload(SEED)
+    n = len(w["len"])
+    src = synthetic.random_bytes(SEED, w["src_bytes"] + 16)
+    d_src = _gpu.to_dev(src)
+    d_arena = torch.zeros(w["arena_bytes"], dtype=torch.uint8, device="cuda")
+    d_so, d_do, d_len = _gpu.to_dev(w["src_off"]), _gpu.to_dev(w["dst_off"]), _gpu.to_dev(w["len"])
+    d_flush = torch.zeros(n, dtype=torch.int32, device="cuda")
+    stream = _gpu.stream()
+
+    def step():
+        rc = lib.ofi_amd_bounce_scatter(d_src.data_ptr(), d_arena.data_ptr(), w["arena_bytes"],
+                                        d_so.data_ptr(), d_do.data_ptr(), d_len.data_ptr(), n,
+                                        d_flush.data_ptr(), stream)
+        if rc != 0:
+            raise RuntimeError("ofi_amd_bounce_scatter: %d" % rc)
+
+    wall_ms, ev_ms = timed_steps(step, args.steps, args.warmup, torch)
+    algo_bytes = 2 * w["src_bytes"] + 8 * n          # payload read + write, 4 B flush read + 4 B write
+    # result check of the timed configuration: flush words and an arena checksum against the oracle
+    arena = np.zeros(w["arena_bytes"], dtype=np.uint8)
+    flush = np.zeros(n, dtype=np.uint32)
+    t0 = time.perf_counter()
+    oracle.oracle_bounce_scatter(_oracle.ptr(src), _oracle.ptr(arena), _oracle.ptr(w["src_off"]),
+                                 _oracle.ptr(w["dst_off"]), _oracle.ptr(w["len"]), n, _oracle.ptr(flush))
+    first_cpu_s = time.perf_counter() - t0
+    ok = bool(np.array_equal(_gpu.to_host(d_flush, np.uint32), flush)) and \
+        int(d_arena.sum(dtype=torch.int64)) == int(arena.sum(dtype=np.int64))
+    # plain device copy of the same payload, as the practical ceiling
+    d_tmp = torch.empty(w["src_bytes"], dtype=torch.uint8, device="cuda")
+    _, copy_ms = timed_steps(lambda: d_tmp.copy_(d_src[:w["src_bytes"]]), args.steps, 3, torch)
+    out = {"ms_wall": wall_ms, "ms_kernel": ev_ms, "algo_bytes": algo_bytes,
+           "gbs": algo_bytes / ev_ms / 1e6, "gbs_wall": algo_bytes / wall_ms / 1e6,
+           "device_copy_gbs": 2 * w["src_bytes"] / copy_ms / 1e6, "parity_ok": ok, "buffers": n,
+           "payload_bytes": w["src_bytes"]}
+    cpu = None
+    if not args.skip_cpu:
+        reps = max(2, min(40, int(8.0 / max(first_cpu_s, 1e-3))))
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            oracle.oracle_bounce_scatter(_oracle.ptr(src), _oracle.ptr(arena), _oracle.ptr(w["src_off"]),
+                                         _oracle.ptr(w["dst_off"]), _oracle.ptr(w["len"]), n,
+                                         _oracle.ptr(flush))
+        cpu_s = (time.perf_counter() - t0) / reps
+        cpu = {"value": algo_bytes / cpu_s / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+               "sample": "%d passes of the full batch (per-buffer memcpy loop, 1 thread)" % reps}
+    del d_arena, d_src, d_tmp
+    torch.cuda.empty_cache()
+    return out, cpu
+
+
+def bench_sched(lib, oracle, torch, np, args):
+    import _gpu
+    import _oracle
+    import aws_ofi_nccl_amd as m
+    from aws_ofi_nccl_amd import synthetic
+    n = 1_000_000
+    sizes = synthetic.stripe_sizes(2024, n)
+    st = m.SchedState(1, 3, 64, 131072, 4, 0)
+    d_state = _gpu.to_dev(np.frombuffer(bytes(st), dtype=np.uint8).copy())
+    d_sizes = _gpu.to_dev(sizes)
+    d_num = torch.zeros(n, dtype=torch.int32, device="cuda")
+    d_xf = torch.zeros(n * 12, dtype=torch.int64, device="cuda")
+    stream = _gpu.stream()
+
+    def step():
+        rc = lib.ofi_amd_sched_batch(d_state.data_ptr(), d_sizes.data_ptr(), n, 128, d_num.data_ptr(),
+                                     d_xf.data_ptr(), stream)
+        if rc != 0:
+            raise RuntimeError("ofi_amd_sched_batch: %d" % rc)
+
+    # parity of the first pass from the seeded state
+    step()
+    torch.cuda.synchronize()
+    want_num, want_xf, _ = _oracle.sched_batch(oracle, sizes, 4, 131072, 64, (1, 3))
+    ok = bool(np.array_equal(_gpu.to_host(d_num, np.uint32), want_num)) and \
+        bool(np.array_equal(_gpu.to_host(d_xf, np.uint64).reshape(n, 4, 3), want_xf))
+    wall_ms, ev_ms = timed_steps(step, args.steps, args.warmup, torch)
+    out = {"messages": n, "ms_wall": wall_ms, "ms_kernels": ev_ms, "msgs_per_s": n / ev_ms * 1e3,
+           "algo_gbs": 108.0 * n / ev_ms / 1e6, "hbm_frac": 108.0 * n / ev_ms / 1e6 / HBM_PEAK_GBS,
+           "parity_ok": ok}
+    if not args.skip_cpu:
+        num = np.zeros(n, dtype=np.uint32)
+        xf = np.zeros((n, 4, 3), dtype=np.uint64)
+        for name, fn in (("cpu_msgs_per_s", oracle.oracle_sched_batch),
+                         ("cpu_msgs_per_s_alloc_per_message", oracle.oracle_sched_batch_alloc)):
+            ost = _oracle.Sched(1, 3, 64, 131072, 4, 0)
+            reps, t0 = 0, time.perf_counter()
+            while time.perf_counter() - t0 < 2.0:
+                fn(ctypes.byref(ost), _oracle.ptr(sizes), n, 128, _oracle.ptr(num), _oracle.ptr(xf))
+                reps += 1
+            out[name] = n * reps / (time.perf_counter() - t0)
+        out["cpu_cores"] = 1
+    return out
+
+
+def bench_tuner(lib, oracle, torch, np, args):
+    import _gpu
+    import aws_ofi_nccl_amd as m
+    from aws_ofi_nccl_amd import synthetic
+    colls, sizes, nodes, ppn, algos = synthetic.tuner_axes()
+    plan = ctypes.c_void_p()
+    m.check(lib.ofi_amd_tuner_plan_create(colls.ctypes.data, len(colls), sizes.ctypes.data, len(sizes),
+                                          nodes.ctypes.data, len(nodes), ppn.ctypes.data, len(ppn),
+                                          algos.ctypes.data, len(algos), ctypes.byref(plan)), "plan_create")
+    points, cells = lib.ofi_amd_tuner_plan_points(plan), lib.ofi_amd_tuner_plan_cells(plan)
+    nv = 64                                   # 2 modelled platforms x numPipeOps 1..32
+    variants = (m.TunerVariant * nv)(*[m.TunerVariant(i % 2, 1 + i // 2, 8, 3) for i in range(nv)])
+    d_cost = torch.zeros(nv * cells, dtype=torch.float64, device="cuda")
+    d_choice = torch.zeros(nv * points * 2, dtype=torch.int8, device="cuda")
+    plats = np.array([i % 4 for i in range(nv)], dtype=np.int32)
+    d_reg = torch.zeros(nv * points * 4, dtype=torch.int8, device="cuda")
+    stream = _gpu.stream()
+
+    def model_step():
+        m.check(lib.ofi_amd_tuner_model_grid(plan, variants, nv, d_cost.data_ptr(), d_choice.data_ptr(),
+                                             stream), "model_grid")
+
+    def region_step():
+        m.check(lib.ofi_amd_tuner_region_grid(plan, plats.ctypes.data, nv, d_reg.data_ptr(), stream),
+                "region_grid")
+
+    _, model_ms = timed_steps(model_step, args.steps, args.warmup, torch)
+    _, region_ms = timed_steps(region_step, args.steps, args.warmup, torch)
+    one = (m.TunerVariant * 1)(m.TunerVariant(0, 1, 8, 3))
+    _, one_ms = timed_steps(lambda: lib.ofi_amd_tuner_model_grid(plan, one, 1, d_cost.data_ptr(),
+                                                                 d_choice.data_ptr(), stream),
+                            args.steps, args.warmup, torch)
+    out = {"grids_per_launch": nv, "cells_per_grid": cells, "points_per_grid": points,
+           "model_ms": model_ms, "model_cells_per_s": nv * cells / model_ms * 1e3,
+           "model_single_grid_ms": one_ms, "region_ms": region_ms,
+           "region_points_per_s": nv * points / region_ms * 1e3}
+    if not args.skip_cpu:
+        # the scalar restatement looping the same grid in C, one core, ~2 s each
+        import _oracle
+        cost = np.zeros(cells, dtype=np.float64)
+        choice = np.zeros(points * 2, dtype=np.int8)
+        rchoice = np.zeros(points * 3, dtype=np.int32)
+        axes = (_oracle.ptr(colls), len(colls), _oracle.ptr(sizes), len(sizes), _oracle.ptr(nodes),
+                len(nodes), _oracle.ptr(ppn), len(ppn))
+        grids, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < 2.0:
+            oracle.oracle_model_grid(grids % 2, 1 + grids // 2, 8, 3, *axes, _oracle.ptr(algos), len(algos),
+                                     _oracle.ptr(cost), _oracle.ptr(choice))
+            grids += 1
+        out["cpu_model_cells_per_s"] = grids * cells / (time.perf_counter() - t0)
+        grids, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < 2.0:
+            oracle.oracle_region_grid(grids % 4, *axes, _oracle.ptr(rchoice))
+            grids += 1
+        out["cpu_region_points_per_s"] = grids * points / (time.perf_counter() - t0)
+        out["cpu_cores"] = 1
+        out["model_speedup_vs_cpu_core"] = out["model_cells_per_s"] / out["cpu_model_cells_per_s"]
+        out["region_speedup_vs_cpu_core"] = out["region_points_per_s"] / out["cpu_region_points_per_s"]
+    lib.ofi_amd_tuner_plan_destroy(plan)
+    return out
+
+
+def bench_gin(lib, oracle, torch, np, args):
+    import _gpu
+    import _oracle
+    import aws_ofi_nccl_amd as m
+    nctx, cap, ops = 256, 4096, args.gin_ops
+    out = {"contexts": nctx, "ring_capacity": cap, "ops_per_context": ops}
+    for mode, key in ((0, "drain"), (2, "drain_and_derive_wire")):
+        rings = ctypes.c_void_p()
+        m.check(lib.ofi_amd_gin_rings_create(nctx, cap, ctypes.byref(rings)), "rings_create")
+        comms = (m.GinComm * nctx)()
+        for c in range(nctx):
+            lib.ofi_amd_gin_comm_init(ctypes.byref(comms[c]), c % 1024, 4, 131072, 64, 1)
+        mrs = _oracle.default_mrs(m.GinMr)
+        stats = m.GinProxyStats()
+        t0 = time.perf_counter()
+        m.check(lib.ofi_amd_gin_produce_seeded(rings, SEED, ops, 1, 64, 1, 1, 0, _gpu.stream()), "produce")
+        rc = lib.ofi_amd_gin_proxy_drain(rings, ops, mode, None, ctypes.cast(comms, ctypes.c_void_p),
+                                         ctypes.cast(mrs, ctypes.c_void_p), None, 20000, ctypes.byref(stats))
+        torch.cuda.synchronize()
+        secs = time.perf_counter() - t0
+        if rc != 0 or lib.ofi_amd_gin_producer_status(rings) != 0:
+            raise RuntimeError("gin drain rc=%d" % rc)
+        out[key] = {"descriptors": stats.descriptors, "seconds": secs,
+                    "descs_per_s": stats.descriptors / secs,
+                    "host_link_gbs": stats.descriptors * 68 / secs / 1e9,
+                    "consumer_ns_per_desc": secs / stats.descriptors * 1e9,
+                    "checksum": "%016x" % stats.checksum, "rdma_writes": stats.writes}
+        lib.ofi_amd_gin_rings_destroy(rings)
+    if not args.skip_cpu:
+        # oracle: generate + fold the same stream on one core, on a bounded sample of the ops
+        sample = min(ops, 40000)
+        omrs = _oracle.default_mrs()
+        t0 = time.perf_counter()
+        ck = oracle.oracle_gin_stream_checksum(SEED, nctx, sample, 1, 64, 1, 1, 0, 4, 131072, 64, 1, omrs)
+        s0 = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        oracle.oracle_gin_stream_checksum(SEED, nctx, sample, 1, 64, 1, 1, 1, 4, 131072, 64, 1, omrs)
+        s1 = time.perf_counter() - t0
+        out["cpu_generate_and_fold_descs_per_s"] = nctx * sample / s0
+        out["cpu_generate_derive_fold_descs_per_s"] = nctx * sample / s1
+        out["cpu_cores"] = 1
+        out["cpu_sample"] = "%d ops per context" % sample
+        if sample == ops:
+            out["parity_ok"] = out["drain"]["checksum"] == "%016x" % ck
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--gin-ops", type=int, default=1_000_000, help="GIN ops per context")
+    ap.add_argument("--skip-extra", action="store_true", help="only the bounce-copy step")
+    ap.add_argument("--skip-cpu", action="store_true", help="no CPU baselines")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU only: this path has no collective or sharded leg "
+              "(run with --gpus 1)", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+    import _oracle
+    import aws_ofi_nccl_amd as m
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the hot path has no CPU implementation)", file=sys.stderr)
+        return 1
+    lib = m.load()
+    m.check(lib.ofi_amd_gpu_init(), "ofi_amd_gpu_init")
+    oracle = _oracle.load_oracle()
+    torch.cuda.init()
+
+    log("bounce copy")
+    bounce, cpu = bench_bounce(lib, oracle, torch, np, args)
+    extra = {}
+    if not args.skip_extra:
+        for name, fn in (("striping", bench_sched), ("tuner", bench_tuner), ("gin", bench_gin)):
+            log(name)
+            extra[name] = fn(lib, oracle, torch, np, args)
+
+    traffic = None
+    prof = os.path.join(ROOT, "profiles", "bounce_scatter_traffic.json")
+    if os.path.exists(prof):
+        traffic = json.load(open(prof)).get("hbm_bytes_per_launch")
+    line = {
+        "metric": "GIN puts/sec + bounce-copy GB/s on 1 MI355X (% of HBM/host-link peak)",
+        "value": bounce["gbs_wall"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": bounce["ms_wall"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "bounce copy: 65536 eager buffers, len uniform 0..8192 B, packed source "
+                               "-> seeded 64 B-aligned offsets in a 2 GiB HBM arena, 4 B flush read each",
+                   "buffers": bounce["buffers"], "payload_bytes": bounce["payload_bytes"],
+                   "arena_bytes": 2 << 30},
+        "roofline": {"bound": "hbm", "achieved": bounce["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": bounce["gbs"] / HBM_PEAK_GBS, "traffic": traffic,
+                     "kernel": "bounce_scatter_kernel", "kernel_ms": bounce["ms_kernel"],
+                     "algorithmic_bytes_per_launch": bounce["algo_bytes"],
+                     "device_copy_GBps_same_payload": bounce["device_copy_gbs"]},
+        "cpu_baseline": cpu,
+        "parity_ok": bounce["parity_ok"],
+        "gin_puts_per_s": extra.get("gin", {}).get("drain", {}).get("descs_per_s"),
+        "extra": extra,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

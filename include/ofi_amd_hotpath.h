@@ -226,7 +226,7 @@ typedef struct {
 	uint32_t more; /* FI_MORE */
 } ofi_amd_gin_write_t;
 
-/* Everything iputSignal derives from one descriptor (192 bytes). */
+/* Everything iputSignal derives from one descriptor (224 bytes). */
 typedef struct {
 	uint32_t seq;
 	uint32_t nseg;

@@ -97,6 +97,10 @@ int oracle_mpsc_pop(oracle_mpsc_t *r, void *entry);        /* 1 popped, 0 empty 
 /* For tests: place both cursors at `pos` (sequence words re-seeded accordingly). */
 void oracle_mpsc_set_positions(oracle_mpsc_t *r, uint32_t pos);
 
+/* Threaded self-check (producers x per_producer pushes, caller consumes): 0 = all
+ * of per-producer FIFO, no loss, no duplicate held. */
+int oracle_mpsc_stress(uint32_t capacity, uint32_t producers, uint32_t per_producer);
+
 typedef struct oracle_spsc oracle_spsc_t;
 oracle_spsc_t *oracle_spsc_create(uint32_t capacity, uint32_t payload_bytes);
 void oracle_spsc_destroy(oracle_spsc_t *r);
@@ -142,7 +146,7 @@ typedef struct {
 	uint32_t more; /* FI_MORE set */
 } oracle_gin_write_t;
 
-/* Everything iputSignal derives from one descriptor. 192 bytes. */
+/* Everything iputSignal derives from one descriptor. 224 bytes. */
 typedef struct {
 	uint32_t seq;
 	uint32_t nseg;
@@ -190,6 +194,13 @@ void oracle_gin_comm_init(oracle_gin_comm_t *c, uint32_t comm_id, uint32_t num_r
 int oracle_gin_iput_signal(oracle_gin_comm_t *c, const oracle_gin_mr_t *mrs,
 			   const oracle_gin_desc_t *d, oracle_gin_wire_t *out);
 
+uint64_t oracle_gin_fold(uint64_t h, const uint64_t *w, int n);
+uint64_t oracle_gin_stream_checksum(uint64_t seed, uint32_t n_contexts, uint64_t ops,
+				    uint32_t peer_rank, uint32_t signal_every, uint32_t signal_op,
+				    uint32_t aggregate_mask, int with_wire, uint32_t num_rails,
+				    uint64_t min_stripe, uint64_t max_small, uint32_t ack_model,
+				    const oracle_gin_mr_t *mrs);
+
 /* ------------------------------------------------------------------- tuner */
 
 enum { ORACLE_PLAT_P5_P5E = 0, ORACLE_PLAT_P5EN = 1, ORACLE_PLAT_P6 = 2, ORACLE_PLAT_P6_B300 = 3 };
@@ -222,6 +233,17 @@ int oracle_region_polys(int platform, uint64_t num_ranks, uint64_t num_nodes, in
 int oracle_region_chunk_size(int platform, int coll, uint64_t size, int algo, int proto,
 			     uint64_t num_ranks, uint64_t num_nodes, uint64_t *chunk);
 uint64_t oracle_chunk_tree_ll128(uint64_t message_size, int nchannels, int log2_nnodes);
+
+/* Whole-grid loops over the functions above.  point = ((coll*n_sizes + size)*n_nodes +
+ * node)*n_ppn + ppn; cost[point*n_algos*3 + a*3 + proto]; choice[point*2 + {algo, proto}];
+ * region choice[point*3 + {algo, proto, nchannels}]. */
+void oracle_model_grid(int platform, int pipe_ops, int num_channels, int net_comp_overhead,
+		       const int32_t *colls, uint32_t n_colls, const uint64_t *sizes, uint32_t n_sizes,
+		       const uint64_t *nodes, uint32_t n_nodes, const uint32_t *ppn, uint32_t n_ppn,
+		       const int32_t *algos, uint32_t n_algos, double *cost, int8_t *choice);
+void oracle_region_grid(int platform, const int32_t *colls, uint32_t n_colls, const uint64_t *sizes,
+			uint32_t n_sizes, const uint64_t *nodes, uint32_t n_nodes, const uint32_t *ppn,
+			uint32_t n_ppn, int32_t *choice);
 
 #ifdef __cplusplus
 }

@@ -257,3 +257,52 @@ int oracle_gin_iput_signal(oracle_gin_comm_t *c, const oracle_gin_mr_t *mrs,
 	}
 	return 0;
 }
+
+/* ---- stream checksum (defined by this project): order-sensitive per context ---- */
+
+static uint64_t rotl64(uint64_t x, int k) { return (x << k) | (x >> (64 - k)); }
+
+uint64_t oracle_gin_fold(uint64_t h, const uint64_t *w, int n)
+{
+	static const uint64_t K[8] = {
+		0x9E3779B97F4A7C15ull, 0xBF58476D1CE4E5B9ull, 0x94D049BB133111EBull, 0xD6E8FEB86659FD93ull,
+		0xCA5A826395121157ull, 0x2545F4914F6CDD1Dull, 0xA0761D6478BD642Full, 0xE7037ED1A0B428DBull,
+	};
+	uint64_t x = 0;
+	for (int k = 0; k < n; k++) {
+		x += (w[k] + (uint64_t)(k + 1)) * K[k & 7];
+	}
+	return (rotl64(h, 5) ^ x) * 0x100000001B3ull;
+}
+
+/* Sum over contexts of the per-context hash of the seeded descriptor stream
+ * (with_wire = 0) or of descriptors interleaved with the wire records iputSignal
+ * derives from them (with_wire = 1; comm c uses comm_id c % 1024). */
+uint64_t oracle_gin_stream_checksum(uint64_t seed, uint32_t n_contexts, uint64_t ops,
+				    uint32_t peer_rank, uint32_t signal_every, uint32_t signal_op,
+				    uint32_t aggregate_mask, int with_wire, uint32_t num_rails,
+				    uint64_t min_stripe, uint64_t max_small, uint32_t ack_model,
+				    const oracle_gin_mr_t *mrs)
+{
+	uint64_t total = 0;
+	for (uint32_t c = 0; c < n_contexts; c++) {
+		uint64_t h = 0x9E3779B97F4A7C15ull ^ c;
+		oracle_gin_comm_t comm;
+		oracle_gin_comm_init(&comm, c % 1024u, num_rails, min_stripe, max_small, ack_model);
+		for (uint64_t i = 0; i < ops; i++) {
+			oracle_gin_desc_t d;
+			oracle_gin_gen_desc(seed, c, i, peer_rank, signal_every, signal_op,
+					    aggregate_mask, &d);
+			h = oracle_gin_fold(h, (const uint64_t *)&d, 8);
+			if (with_wire) {
+				oracle_gin_wire_t w;
+				if (oracle_gin_iput_signal(&comm, mrs, &d, &w) != 0) {
+					return 0;
+				}
+				h = oracle_gin_fold(h, (const uint64_t *)&w, (int)(sizeof(w) / 8));
+			}
+		}
+		total += h;
+	}
+	return total;
+}

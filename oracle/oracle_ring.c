@@ -178,3 +178,74 @@ int oracle_spsc_pop(oracle_spsc_t *r, void *entry)
 	atomic_store_explicit(&r->tail, (t + 1) % r->capacity, memory_order_release);
 	return 1;
 }
+
+/* ---- threaded self-check, the scenario of tests/unit/mpsc_ring.cpp:118-189 ----
+ * `producers` threads push (id << 28 | counter); the calling thread pops and checks
+ * per-producer FIFO, no loss, no duplicate.  Returns 0 when every property held. */
+#include <pthread.h>
+
+struct stress_arg {
+	oracle_mpsc_t *ring;
+	uint32_t id;
+	uint32_t count;
+};
+
+static void *stress_producer(void *p)
+{
+	struct stress_arg *a = (struct stress_arg *)p;
+	uint32_t i = 0;
+	while (i < a->count) {
+		uint32_t v = (a->id << 28) | i;
+		if (oracle_mpsc_push(a->ring, &v)) {
+			++i;
+		}
+	}
+	return NULL;
+}
+
+int oracle_mpsc_stress(uint32_t capacity, uint32_t producers, uint32_t per_producer)
+{
+	if (producers == 0 || producers > 15 || per_producer >= (1u << 28)) {
+		return -22;
+	}
+	oracle_mpsc_t *ring = oracle_mpsc_create(capacity, sizeof(uint32_t));
+	if (!ring) {
+		return -12;
+	}
+	pthread_t th[15];
+	struct stress_arg args[15];
+	uint32_t next_expected[15] = { 0 };
+	int bad = 0;
+
+	for (uint32_t p = 0; p < producers; p++) {
+		args[p].ring = ring;
+		args[p].id = p;
+		args[p].count = per_producer;
+		pthread_create(&th[p], NULL, stress_producer, &args[p]);
+	}
+	uint64_t total = 0, want = (uint64_t)producers * per_producer;
+	while (total < want) {
+		uint32_t v;
+		if (oracle_mpsc_pop(ring, &v)) {
+			uint32_t p = v >> 28, c = v & ((1u << 28) - 1);
+			if (p >= producers || c != next_expected[p]) {
+				bad = 1;
+			} else {
+				next_expected[p] = c + 1;
+			}
+			++total;
+		}
+	}
+	for (uint32_t p = 0; p < producers; p++) {
+		pthread_join(th[p], NULL);
+		if (next_expected[p] != per_producer) {
+			bad = 1;
+		}
+	}
+	uint32_t v;
+	if (oracle_mpsc_pop(ring, &v)) {
+		bad = 1; /* must be empty */
+	}
+	oracle_mpsc_destroy(ring);
+	return bad;
+}

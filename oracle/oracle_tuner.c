@@ -571,3 +571,66 @@ int oracle_region_chunk_size(int platform, int coll, uint64_t size, int algo, in
 	}
 	return 0;
 }
+
+/* ---- whole-grid loops (the scalar baseline the batched kernels are timed against) ----
+ * Layouts as the product's grid entry points: point = ((coll*n_sizes + size)*n_nodes +
+ * node)*n_ppn + ppn; cost[point*n_algos*3 + a*3 + proto]; choice[point*2 + {0,1}];
+ * region choice[point*3 + {algo, proto, nchannels}] (int32, nchannels -1 when left alone). */
+void oracle_model_grid(int platform, int pipe_ops, int num_channels, int net_comp_overhead,
+		       const int32_t *colls, uint32_t n_colls, const uint64_t *sizes, uint32_t n_sizes,
+		       const uint64_t *nodes, uint32_t n_nodes, const uint32_t *ppn, uint32_t n_ppn,
+		       const int32_t *algos, uint32_t n_algos, double *cost, int8_t *choice)
+{
+	uint64_t point = 0;
+	const int modelled = platform == ORACLE_PLAT_P5_P5E || platform == ORACLE_PLAT_P5EN;
+	for (uint32_t c = 0; c < n_colls; c++) {
+		for (uint32_t s = 0; s < n_sizes; s++) {
+			for (uint32_t n = 0; n < n_nodes; n++) {
+				for (uint32_t q = 0; q < n_ppn; q++, point++) {
+					uint64_t R = nodes[n] * ppn[q];
+					if (cost) {
+						double *row = cost + point * n_algos * 3;
+						for (uint32_t a = 0; a < n_algos; a++) {
+							for (int pr = 0; pr < 3; pr++) {
+								row[a * 3 + pr] = modelled ? (double)oracle_model_cost(
+									platform, colls[c], algos[a], pr, pipe_ops, sizes[s],
+									R, nodes[n], num_channels, net_comp_overhead) : -1.0;
+							}
+						}
+					}
+					if (choice) {
+						int al = -1, pr = -1;
+						if (modelled) {
+							oracle_model_decide(platform, colls[c], pipe_ops, sizes[s], R,
+									    nodes[n], num_channels, net_comp_overhead,
+									    &al, &pr);
+						}
+						choice[point * 2] = (int8_t)al;
+						choice[point * 2 + 1] = (int8_t)pr;
+					}
+				}
+			}
+		}
+	}
+}
+
+void oracle_region_grid(int platform, const int32_t *colls, uint32_t n_colls, const uint64_t *sizes,
+			uint32_t n_sizes, const uint64_t *nodes, uint32_t n_nodes, const uint32_t *ppn,
+			uint32_t n_ppn, int32_t *choice)
+{
+	uint64_t point = 0;
+	for (uint32_t c = 0; c < n_colls; c++) {
+		for (uint32_t s = 0; s < n_sizes; s++) {
+			for (uint32_t n = 0; n < n_nodes; n++) {
+				for (uint32_t q = 0; q < n_ppn; q++, point++) {
+					int al, pr, ch = -1;
+					oracle_region_decide(platform, colls[c], sizes[s], nodes[n] * ppn[q],
+							     nodes[n], &al, &pr, &ch);
+					choice[point * 3] = al;
+					choice[point * 3 + 1] = pr;
+					choice[point * 3 + 2] = ch;
+				}
+			}
+		}
+	}
+}

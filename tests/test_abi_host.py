@@ -1,0 +1,136 @@
+"""CPU-side checks of the product library: it loads, exports every symbol the header declares,
+refuses GPU work without a GPU (no silent CPU path), and its host-side logic -- the per-op
+scheduler call and the proxy's iputSignal derivation -- matches the oracle bit for bit."""
+import ctypes
+import errno
+import os
+import re
+
+import numpy as np
+import pytest
+
+import _oracle
+import aws_ofi_nccl_amd as m
+from aws_ofi_nccl_amd import synthetic
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "ofi_amd_hotpath.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ofi_amd_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(lib):
+    names = declared_symbols()
+    assert len(names) >= 45
+    raw = ctypes.CDLL(m.LIB_PATH)
+    for name in names:
+        assert hasattr(raw, name), "header declares %s but the library lacks it" % name
+    # and the Python prototypes cover the same set
+    assert sorted(m.PROTOTYPES) == names
+
+
+def test_struct_sizes_match_the_header():
+    assert ctypes.sizeof(m.XferInfo) == 24          # nccl_net_ofi_xfer_info_t
+    assert ctypes.sizeof(m.SchedState) == 32
+    assert ctypes.sizeof(m.GinDesc) == 64
+    assert ctypes.sizeof(m.GinWire) == 224
+    assert ctypes.sizeof(m.GinMr) == 56             # gin_remote_mr is 56 bytes in the reference too
+    assert ctypes.sizeof(m.TunerVariant) == 16
+
+
+def test_gpu_entry_points_fail_loudly_without_a_gpu(lib):
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    enodev = -errno.ENODEV
+    assert lib.ofi_amd_gpu_init() == enodev
+    p = ctypes.c_void_p()
+    assert lib.ofi_amd_gpu_mem_alloc(ctypes.byref(p), 64) == enodev
+    assert lib.ofi_amd_bounce_scatter(1, 1, 64, 1, 1, 1, 1, None, None) == enodev
+    assert lib.ofi_amd_flush_read(1, 1, 1, 1, None) == enodev
+    assert lib.ofi_amd_sched_batch(1, 1, 1, 128, 1, 1, None) == enodev
+    assert lib.ofi_amd_gin_rings_create(4, 256, ctypes.byref(p)) == enodev
+    colls, sizes, nodes, ppn, algos = synthetic.tuner_axes()
+    assert lib.ofi_amd_tuner_plan_create(colls.ctypes.data, 3, sizes.ctypes.data, 140,
+                                         nodes.ctypes.data, 11, ppn.ctypes.data, 4,
+                                         algos.ctypes.data, 3, ctypes.byref(p)) == enodev
+    assert lib.ofi_amd_devcopy_register(1, 64, ctypes.byref(p)) == enodev
+    assert lib.ofi_amd_gpu_flush_gpudirect_rdma_writes() == -errno.EPERM   # as the ROCm reference
+    assert lib.ofi_amd_gpu_have_gdr_support_attr() == 0
+
+
+def test_wire_encoders_match_oracle(lib, oracle):
+    rng = np.random.default_rng(3)
+    for _ in range(3000):
+        comm, seq = int(rng.integers(0, 1024)), int(rng.integers(0, 8192))
+        nseg, ack, rx = int(rng.integers(0, 16)), int(rng.integers(0, 2)), int(rng.integers(0, 16384))
+        assert lib.ofi_amd_gin_imm(comm, seq, nseg, ack) == oracle.oracle_gin_imm(comm, seq, nseg, ack)
+        assert lib.ofi_amd_gin_meta_header(comm, seq, nseg, ack) == \
+            oracle.oracle_gin_meta_header(comm, seq, nseg, ack)
+        assert lib.ofi_amd_gin_ack_msg(comm, rx) == oracle.oracle_gin_ack_msg(comm, rx)
+
+
+@pytest.mark.parametrize("rails,min_stripe,max_small", [(4, 131072, 64), (4, 4096, 64), (3, 100000, 64),
+                                                        (2, 8192, 0), (1, 131072, 64)])
+def test_host_scheduler_matches_oracle(lib, oracle, rails, min_stripe, max_small):
+    sizes = synthetic.stripe_sizes(rails * 7 + min_stripe, 20000)
+    num, xf, ost = _oracle.sched_batch(oracle, sizes, rails, min_stripe, max_small, (1 % rails, 0))
+    st = m.SchedState(1 % rails, 0, max_small, min_stripe, rails, 0)
+    x = (m.XferInfo * 4)()
+    for i, s in enumerate(sizes):
+        n = lib.ofi_amd_sched_get_schedule(ctypes.byref(st), int(s), 128, x)
+        assert n == num[i]
+        for k in range(n):
+            assert (x[k].rail_id, x[k].pad0, x[k].pad1, x[k].offset, x[k].msg_size) == (
+                int(xf[i, k, 0]) & 0xFFFF, 0, 0, int(xf[i, k, 1]), int(xf[i, k, 2]))
+    assert (st.rr_small_counter, st.rr_counter) == (ost.rr_small_counter, ost.rr_counter)
+    bad = m.SchedState(0, 0, 64, 0, 4, 0)
+    assert lib.ofi_amd_sched_get_schedule(ctypes.byref(bad), 100, 128, x) == -errno.EINVAL
+
+
+@pytest.mark.parametrize("ack_model,agg_mask,signal_op,rails", [(1, 1, 1, 4), (1, 0, 2, 4), (0, 1, 1, 2),
+                                                                 (1, 1, 2, 3)])
+def test_proxy_derivation_matches_oracle(lib, oracle, ack_model, agg_mask, signal_op, rails):
+    """ofi_amd_gin_iput_signal (product host code) against oracle_gin_iput_signal over a seeded
+    stream: every field of every wire record, and the whole comm state after each op."""
+    omrs = _oracle.default_mrs()
+    pmrs = _oracle.default_mrs(m.GinMr)
+    oc, pc = _oracle.GinComm(), m.GinComm()
+    oracle.oracle_gin_comm_init(ctypes.byref(oc), 9, rails, 131072, 64, ack_model)
+    assert lib.ofi_amd_gin_comm_init(ctypes.byref(pc), 9, rails, 131072, 64, ack_model) == 0
+    od, ow, pw = _oracle.GinDesc(), _oracle.GinWire(), m.GinWire()
+    n = 12000 if ack_model else 9000
+    for i in range(n):
+        oracle.oracle_gin_gen_desc(1234, 6, i, 1, 64 if i % 2000 < 1500 else 3, signal_op, agg_mask,
+                                   ctypes.byref(od))
+        if i % 97 == 0:
+            od.size = 0                                # signal-only / empty ops now and then
+        pd = m.GinDesc.from_buffer_copy(bytes(od))
+        orc = oracle.oracle_gin_iput_signal(ctypes.byref(oc), omrs, ctypes.byref(od), ctypes.byref(ow))
+        prc = lib.ofi_amd_gin_iput_signal(ctypes.byref(pc), pmrs, ctypes.byref(pd), ctypes.byref(pw))
+        assert (orc, prc) in ((0, 0), (-11, -errno.EAGAIN))
+        assert bytes(ow) == bytes(pw), i
+        assert bytes(oc) == bytes(pc), i
+    if ack_model == 0:
+        assert prc == -errno.EAGAIN                    # window filled at 8192 outstanding
+        lib.ofi_amd_gin_apply_ack(ctypes.byref(pc), 100)
+        assert pc.tx_tail == 100
+        lib.ofi_amd_gin_apply_ack(ctypes.byref(pc), 50)          # older ACK: ignored
+        assert pc.tx_tail == 100
+        assert lib.ofi_amd_gin_iput_signal(ctypes.byref(pc), pmrs, ctypes.byref(pd), ctypes.byref(pw)) == 0
+
+
+def test_proxy_rejects_bad_arguments(lib):
+    c = m.GinComm()
+    assert lib.ofi_amd_gin_comm_init(ctypes.byref(c), 1024, 4, 131072, 64, 1) == -errno.EINVAL
+    assert lib.ofi_amd_gin_comm_init(ctypes.byref(c), 1, 5, 131072, 64, 1) == -errno.EINVAL
+    assert lib.ofi_amd_gin_comm_init(ctypes.byref(c), 1, 4, 0, 64, 1) == -errno.EINVAL
+    assert lib.ofi_amd_gin_comm_init(ctypes.byref(c), 1, 4, 131072, 64, 1) == 0
+    d = m.GinDesc(0, 0, 8, 0, 0, 1, 7, 0, 0, 0, 1, 2, 2)
+    w = m.GinWire()
+    assert lib.ofi_amd_gin_iput_signal(ctypes.byref(c), _oracle.default_mrs(m.GinMr), ctypes.byref(d),
+                                       ctypes.byref(w)) == -errno.EINVAL

@@ -1,0 +1,197 @@
+"""GPU parity: batched bounce copy + flush through the C ABI against the CPU oracle
+(destination bytes, untouched bytes and flush words bit-exact)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import _gpu
+import _oracle
+from aws_ofi_nccl_amd import synthetic
+
+pytestmark = pytest.mark.gpu
+
+
+def scatter(lib, src, arena_t, src_off, dst_off, length, flush=True):
+    n = len(length)
+    d_src = _gpu.to_dev(src)
+    d_so, d_do, d_len = _gpu.to_dev(src_off), _gpu.to_dev(dst_off), _gpu.to_dev(length)
+    d_flush = torch.full((max(n, 1),), -1, dtype=torch.int32, device="cuda")
+    rc = lib.ofi_amd_bounce_scatter(d_src.data_ptr(), arena_t.data_ptr(), arena_t.numel(),
+                                    d_so.data_ptr(), d_do.data_ptr(), d_len.data_ptr(), n,
+                                    d_flush.data_ptr() if flush else None, _gpu.stream())
+    assert rc == 0
+    _gpu.sync()
+    return _gpu.to_host(d_flush, np.uint32)[:n]
+
+
+def oracle_scatter(oracle, src, arena, src_off, dst_off, length):
+    flush = np.zeros(len(length), dtype=np.uint32)
+    oracle.oracle_bounce_scatter(_oracle.ptr(src), _oracle.ptr(arena), _oracle.ptr(src_off),
+                                 _oracle.ptr(dst_off), _oracle.ptr(length), len(length),
+                                 _oracle.ptr(flush))
+    return flush
+
+
+@pytest.mark.parametrize("n,arena_mib,seed", [(1, 1, 0), (7, 1, 1), (1000, 16, 2), (4099, 64, 3)])
+def test_parity_small(lib, oracle, gpu, n, arena_mib, seed):
+    w = synthetic.bounce_workload(seed, n=n, arena_bytes=arena_mib << 20)
+    src = synthetic.random_bytes(seed, w["src_bytes"] + 16)
+    want = np.full(w["arena_bytes"], 0xCC, dtype=np.uint8)       # pre-filled: catches stray writes
+    want_flush = oracle_scatter(oracle, src, want, w["src_off"], w["dst_off"], w["len"])
+    arena = torch.full((w["arena_bytes"],), 0xCC, dtype=torch.uint8, device="cuda")
+    flush = scatter(lib, src, arena, w["src_off"], w["dst_off"], w["len"])
+    assert np.array_equal(arena.cpu().numpy(), want)
+    assert np.array_equal(flush, want_flush)
+    assert _gpu.fetch_async_errors(lib) == 0
+
+
+def test_every_length_and_source_alignment(lib, oracle, gpu):
+    """Lengths 0..300 plus the sizes around the 1 KiB / 4 KiB trip boundaries and the 8 KiB
+    maximum, each at all 16 source byte alignments."""
+    lens = list(range(0, 301)) + [1008, 1023, 1024, 1025, 1039, 4080, 4095, 4096, 4097, 4111,
+                                  8176, 8191, 8192]
+    length = np.array([l for l in lens for _ in range(16)], dtype=np.uint32)
+    n = len(length)
+    align = np.tile(np.arange(16, dtype=np.uint64), len(lens))
+    slot = 8192 + 64
+    src_off = np.arange(n, dtype=np.uint64) * np.uint64(slot) + align
+    dst_off = np.random.default_rng(5).permutation(n).astype(np.uint64) * np.uint64(slot)
+    src = synthetic.random_bytes(5, n * slot + 64)
+    want = np.full(n * slot, 0x5A, dtype=np.uint8)
+    want_flush = oracle_scatter(oracle, src, want, src_off, dst_off, length)
+    arena = torch.full((n * slot,), 0x5A, dtype=torch.uint8, device="cuda")
+    flush = scatter(lib, src, arena, src_off, dst_off, length)
+    assert np.array_equal(arena.cpu().numpy(), want)
+    assert np.array_equal(flush, want_flush)
+
+
+def test_empty_batch_and_all_zero_lengths(lib, oracle, gpu):
+    arena = torch.full((4096,), 9, dtype=torch.uint8, device="cuda")
+    assert lib.ofi_amd_bounce_scatter(arena.data_ptr(), arena.data_ptr(), 4096, None, None, None, 0,
+                                      None, _gpu.stream()) == 0
+    src = np.arange(64, dtype=np.uint8)
+    flush = scatter(lib, src, arena, np.zeros(8, np.uint64), np.arange(8, dtype=np.uint64) * 64,
+                    np.zeros(8, np.uint32))
+    assert torch.all(arena == 9) and list(flush) == [0x09090909] * 8
+
+
+def test_without_flush_output(lib, oracle, gpu):
+    w = synthetic.bounce_workload(8, n=500, arena_bytes=8 << 20)
+    src = synthetic.random_bytes(8, w["src_bytes"] + 16)
+    want = np.zeros(w["arena_bytes"], dtype=np.uint8)
+    oracle_scatter(oracle, src, want, w["src_off"], w["dst_off"], w["len"])
+    arena = torch.zeros(w["arena_bytes"], dtype=torch.uint8, device="cuda")
+    scatter(lib, src, arena, w["src_off"], w["dst_off"], w["len"], flush=False)
+    assert np.array_equal(arena.cpu().numpy(), want)
+
+
+def test_flush_into_pinned_host_memory(lib, oracle, gpu):
+    w = synthetic.bounce_workload(9, n=300, arena_bytes=4 << 20)
+    src = synthetic.random_bytes(9, w["src_bytes"] + 16)
+    want = np.zeros(w["arena_bytes"], dtype=np.uint8)
+    want_flush = oracle_scatter(oracle, src, want, w["src_off"], w["dst_off"], w["len"])
+    host = ctypes.c_void_p()
+    assert lib.ofi_amd_gpu_host_alloc(ctypes.byref(host), 4 * 300) == 0
+    dev = ctypes.c_void_p()
+    assert lib.ofi_amd_gpu_host_get_device_pointer(ctypes.byref(dev), host) == 0
+    arena = torch.zeros(w["arena_bytes"], dtype=torch.uint8, device="cuda")
+    d_src = _gpu.to_dev(src)
+    d = [_gpu.to_dev(w[k]) for k in ("src_off", "dst_off", "len")]
+    assert lib.ofi_amd_bounce_scatter(d_src.data_ptr(), arena.data_ptr(), arena.numel(), d[0].data_ptr(),
+                                      d[1].data_ptr(), d[2].data_ptr(), 300, dev, _gpu.stream()) == 0
+    _gpu.sync()
+    got = np.ctypeslib.as_array(ctypes.cast(host, ctypes.POINTER(ctypes.c_uint32)), shape=(300,)).copy()
+    assert np.array_equal(got, want_flush)
+    # flush-only entry point re-reads the same words
+    d_flush = torch.zeros(300, dtype=torch.int32, device="cuda")
+    assert lib.ofi_amd_flush_read(arena.data_ptr(), d[1].data_ptr(), 300, d_flush.data_ptr(),
+                                  _gpu.stream()) == 0
+    _gpu.sync()
+    assert np.array_equal(_gpu.to_host(d_flush, np.uint32), want_flush)
+    assert lib.ofi_amd_gpu_host_free(host) == 0
+
+
+def test_out_of_range_destination_is_skipped_and_reported(lib, gpu):
+    arena = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+    src = np.full(256, 0xEE, dtype=np.uint8)
+    # buffer 0 fine, 1 misaligned, 2 runs past the end, 3 starts past the end
+    flush = scatter(lib, src, arena, np.zeros(4, np.uint64),
+                    np.array([0, 100, 4096 - 64, 8192], dtype=np.uint64),
+                    np.array([64, 64, 128, 8], dtype=np.uint32))
+    got = arena.cpu().numpy()
+    assert np.all(got[:64] == 0xEE) and not got[64:].any()
+    assert _gpu.fetch_async_errors(lib) & 1
+    assert _gpu.fetch_async_errors(lib) == 0          # fetch clears
+
+
+def test_full_size_configuration(lib, oracle, gpu):
+    """65,536 eager buffers of 0..8 KiB scattered over a 2 GiB arena."""
+    w = synthetic.bounce_workload(1234)
+    assert len(w["len"]) == 65536 and w["arena_bytes"] == 2 << 30
+    src = synthetic.random_bytes(1234, w["src_bytes"] + 16)
+    want = np.zeros(w["arena_bytes"], dtype=np.uint8)
+    want_flush = oracle_scatter(oracle, src, want, w["src_off"], w["dst_off"], w["len"])
+    arena = torch.zeros(w["arena_bytes"], dtype=torch.uint8, device="cuda")
+    flush = scatter(lib, src, arena, w["src_off"], w["dst_off"], w["len"])
+    assert np.array_equal(flush, want_flush)
+    want_t = torch.from_numpy(want).cuda()
+    assert torch.equal(arena, want_t)
+    # size-independent property: the arena's byte sum equals the sum of all payload bytes
+    assert int(arena.sum(dtype=torch.int64)) == int(src[:w["src_bytes"]].sum(dtype=np.int64))
+    # idempotence: running the batch again changes nothing
+    scatter(lib, src, arena, w["src_off"], w["dst_off"], w["len"])
+    assert torch.equal(arena, want_t)
+
+
+def test_device_copy_interface(lib, gpu):
+    """The patterns of tests/unit/gdrcopy.cpp:15-133 through the nccl_ofi_device_copy mirror."""
+    size = 2 << 20
+    buf = torch.zeros(size, dtype=torch.uint8, device="cuda")
+    h = ctypes.c_void_p()
+    assert lib.ofi_amd_devcopy_register(buf.data_ptr(), size, ctypes.byref(h)) == 0
+    a = np.full(size, ord("A"), dtype=np.uint8)
+    assert lib.ofi_amd_devcopy_to_device(a.ctypes.data, h, 0, size) == 0
+    back = np.zeros(size, dtype=np.uint8)
+    assert lib.ofi_amd_devcopy_from_device(h, 0, back.ctypes.data, size) == 0
+    assert np.all(back == ord("A"))
+    for i in range(10):
+        b = np.array([ord("a") + i], dtype=np.uint8)
+        assert lib.ofi_amd_devcopy_to_device(b.ctypes.data, h, i, 1) == 0
+    for i in range(10):
+        b = np.zeros(1, dtype=np.uint8)
+        assert lib.ofi_amd_devcopy_from_device(h, i, b.ctypes.data, 1) == 0
+        assert b[0] == ord("a") + i
+    assert bytes(buf[:12].cpu().numpy()) == b"abcdefghijAA"
+    assert lib.ofi_amd_devcopy_to_device(a.ctypes.data, h, size - 4, 8) < 0     # past the region
+    assert lib.ofi_amd_devcopy_forced_pcie_copy() == 0
+    assert lib.ofi_amd_devcopy_deregister(h) == 0
+    host = np.zeros(16, dtype=np.uint8)
+    assert lib.ofi_amd_devcopy_register(host.ctypes.data, 16, ctypes.byref(h)) < 0   # not device memory
+
+
+def test_gpu_glue(lib, gpu):
+    p = ctypes.c_void_p()
+    assert lib.ofi_amd_gpu_mem_alloc(ctypes.byref(p), 1 << 20) == 0
+    dev = ctypes.c_int(-5)
+    assert lib.ofi_amd_gpu_get_device_for_addr(p, ctypes.byref(dev)) == 0 and dev.value == 0
+    base, size = ctypes.c_void_p(), ctypes.c_size_t()
+    assert lib.ofi_amd_gpu_get_address_range(ctypes.c_void_p(p.value + 4096), ctypes.byref(base),
+                                             ctypes.byref(size)) == 0
+    assert base.value == p.value and size.value >= 1 << 20
+    is_host = ctypes.c_int(-1)
+    assert lib.ofi_amd_gpu_seg_is_host(p, ctypes.byref(is_host)) == 0 and is_host.value == 0
+    data = np.arange(256, dtype=np.uint8)
+    assert lib.ofi_amd_gpu_mem_copy_host_to_device(p, data.ctypes.data, 256) == 0
+    back = np.zeros(256, dtype=np.uint8)
+    assert lib.ofi_amd_gpu_mem_copy_device_to_host(back.ctypes.data, p, 256) == 0
+    assert np.array_equal(back, data)
+    assert lib.ofi_amd_gpu_mem_free(p) == 0
+    cur = ctypes.c_int(-1)
+    assert lib.ofi_amd_gpu_get_current_device(ctypes.byref(cur)) == 0 and cur.value == 0
+    assert lib.ofi_amd_gpu_set_current_device(0) == 0
+    assert lib.ofi_amd_gpu_have_dma_buf_attr() in (0, 1)
+    host = np.zeros(8, dtype=np.uint8)
+    assert lib.ofi_amd_gpu_seg_is_host(host.ctypes.data, ctypes.byref(is_host)) == 0 and is_host.value == 1
+    assert lib.ofi_amd_gpu_get_device_for_addr(host.ctypes.data, ctypes.byref(dev)) < 0 and dev.value == -1

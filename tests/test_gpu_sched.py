@@ -1,0 +1,129 @@
+"""GPU parity: batched rail striping through the C ABI against the CPU oracle
+(stripe counts, (rail, offset, length) triples, padding and final counters bit-exact)."""
+import ctypes
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import _gpu
+import _oracle
+import aws_ofi_nccl_amd as m
+from aws_ofi_nccl_amd import synthetic
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "scheduler_kat.json")
+
+
+def dev_state(rails, min_stripe, max_small, seeds):
+    st = m.SchedState(seeds[0], seeds[1], max_small, min_stripe, rails, 0)
+    return _gpu.to_dev(np.frombuffer(bytes(st), dtype=np.uint8).copy())
+
+
+def read_state(d_state):
+    return m.SchedState.from_buffer_copy(d_state.cpu().numpy().tobytes())
+
+
+def gpu_batch(lib, d_state, sizes, align=128):
+    n = len(sizes)
+    d_sizes = _gpu.to_dev(sizes) if n else torch.zeros(1, dtype=torch.int64, device="cuda")
+    d_num = torch.full((max(n, 1),), -1, dtype=torch.int32, device="cuda")
+    d_xf = torch.full((max(n, 1) * 12,), -1, dtype=torch.int64, device="cuda")
+    rc = lib.ofi_amd_sched_batch(d_state.data_ptr(), d_sizes.data_ptr(), n, align, d_num.data_ptr(),
+                                 d_xf.data_ptr(), _gpu.stream())
+    _gpu.sync()
+    return rc, _gpu.to_host(d_num, np.uint32)[:n], _gpu.to_host(d_xf, np.uint64)[:n * 12].reshape(n, 4, 3)
+
+
+def test_reference_known_answers_on_gpu(lib, gpu):
+    doc = json.load(open(GOLDEN))
+    sizes = np.array([c["size"] for c in doc["calls"]], dtype=np.uint64)
+    d_state = dev_state(doc["num_rails"], doc["min_stripe_size"], doc["max_small_msg_size"], (0, 0))
+    rc, num, xf = gpu_batch(lib, d_state, sizes, doc["align"])
+    assert rc == 0
+    for i, call in enumerate(doc["calls"]):
+        got = [(int(xf[i, k, 0]), int(xf[i, k, 1]), int(xf[i, k, 2])) for k in range(num[i])]
+        assert got == [tuple(t) for t in call["stripes"]], call["size"]
+
+
+@pytest.mark.parametrize("n", [1, 63, 64, 255, 256, 257, 1023, 1024, 1025, 4096, 100003])
+@pytest.mark.parametrize("rails,min_stripe,max_small,seeds", [(4, 131072, 64, (0, 0)),
+                                                              (3, 100000, 64, (2, 1)),
+                                                              (2, 4096, 0, (1, 1)),
+                                                              (1, 131072, 64, (0, 0)),
+                                                              (4, 4097, 1000, (3, 2))])
+def test_parity_random(lib, oracle, gpu, n, rails, min_stripe, max_small, seeds):
+    sizes = synthetic.stripe_sizes(n * 31 + rails, n)
+    sizes[::5] = sizes[::5] % np.uint64(200)                   # enough small messages
+    want_num, want_xf, ost = _oracle.sched_batch(oracle, sizes, rails, min_stripe, max_small, seeds)
+    d_state = dev_state(rails, min_stripe, max_small, seeds)
+    rc, num, xf = gpu_batch(lib, d_state, sizes)
+    assert rc == 0
+    assert np.array_equal(num, want_num)
+    assert np.array_equal(xf, want_xf)                          # includes zero padding and unused rows
+    st = read_state(d_state)
+    assert (st.rr_small_counter, st.rr_counter) == (ost.rr_small_counter, ost.rr_counter)
+    assert (st.max_small_msg_size, st.min_stripe_size, st.num_rails) == (max_small, min_stripe, rails)
+
+
+def test_chained_batches_carry_state(lib, oracle, gpu):
+    sizes = synthetic.stripe_sizes(77, 30000)
+    want_num, want_xf, ost = _oracle.sched_batch(oracle, sizes, 4, 131072, 64, (1, 2))
+    d_state = dev_state(4, 131072, 64, (1, 2))
+    cuts = [0, 1, 1000, 1001, 9999, 20480, 30000]
+    for a, b in zip(cuts[:-1], cuts[1:]):
+        rc, num, xf = gpu_batch(lib, d_state, sizes[a:b])
+        assert rc == 0
+        assert np.array_equal(num, want_num[a:b]) and np.array_equal(xf, want_xf[a:b])
+    st = read_state(d_state)
+    assert (st.rr_small_counter, st.rr_counter) == (ost.rr_small_counter, ost.rr_counter)
+
+
+def test_extreme_sizes(lib, oracle, gpu):
+    sizes = np.array([0, 1, 63, 64, (1 << 63) - 1, 1 << 63, (1 << 64) - 129, (1 << 64) - 1,
+                      131072, 131073, 393216, 393217], dtype=np.uint64)
+    want_num, want_xf, _ = _oracle.sched_batch(oracle, sizes)
+    rc, num, xf = gpu_batch(lib, dev_state(4, 131072, 64, (0, 0)), sizes)
+    assert rc == 0 and np.array_equal(num, want_num) and np.array_equal(xf, want_xf)
+
+
+def test_non_power_of_two_alignment(lib, oracle, gpu):
+    sizes = synthetic.stripe_sizes(5, 5000)
+    want_num, want_xf, _ = _oracle.sched_batch(oracle, sizes, 4, 131072, 64, (0, 0), align=96)
+    rc, num, xf = gpu_batch(lib, dev_state(4, 131072, 64, (0, 0)), sizes, align=96)
+    assert rc == 0 and np.array_equal(num, want_num) and np.array_equal(xf, want_xf)
+
+
+def test_bad_arguments(lib, gpu):
+    d_state = dev_state(4, 131072, 64, (0, 0))
+    rc, _, _ = gpu_batch(lib, d_state, np.zeros(0, np.uint64))
+    assert rc == 0                                              # empty batch
+    assert lib.ofi_amd_sched_batch(d_state.data_ptr(), None, 5, 128, None, None, None) < 0
+    assert lib.ofi_amd_sched_batch(d_state.data_ptr(), 1, 5, 0, 1, 1, None) < 0      # align 0
+    assert lib.ofi_amd_sched_batch(d_state.data_ptr(), 1, (1 << 28) + 1, 128, 1, 1, None) < 0
+    # unusable state on the device: the batch is left unwritten and the error word says why
+    for rails, min_stripe in [(5, 131072), (0, 131072), (4, 0)]:
+        bad = dev_state(rails, min_stripe, 64, (0, 0))
+        rc, num, xf = gpu_batch(lib, bad, np.arange(10, dtype=np.uint64))
+        assert rc == 0
+        assert np.all(num == 0xFFFFFFFF) and np.all(xf == np.uint64(0xFFFFFFFFFFFFFFFF))
+        assert _gpu.fetch_async_errors(lib) & 4
+
+
+def test_full_size_configuration(lib, oracle, gpu):
+    """1,000,000 messages log-uniform in [1 B, 256 MiB), 4 rails, default thresholds, seeded start rails."""
+    sizes = synthetic.stripe_sizes(2024, 1_000_000)
+    assert sizes.min() >= 1 and sizes.max() < (1 << 28)
+    want_num, want_xf, ost = _oracle.sched_batch(oracle, sizes, 4, 131072, 64, (1, 3))
+    d_state = dev_state(4, 131072, 64, (1, 3))
+    rc, num, xf = gpu_batch(lib, d_state, sizes)
+    assert rc == 0
+    assert np.array_equal(num, want_num)
+    assert np.array_equal(xf, want_xf)
+    st = read_state(d_state)
+    assert (st.rr_small_counter, st.rr_counter) == (ost.rr_small_counter, ost.rr_counter)
+    # invariants that hold at any size
+    assert np.array_equal(xf[:, :, 2].sum(axis=1), sizes)
+    assert set(np.unique(num)) <= {1, 2, 4}
