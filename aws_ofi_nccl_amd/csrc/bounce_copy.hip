@@ -7,13 +7,21 @@
  * visibility with a small read-back (rdma_flush_req::post, :2664-2713).  Here
  * one launch moves a whole batch.
  *
- * Work mapping: one 64-lane wavefront per buffer, four buffers per workgroup.
- * Destinations are 64-byte aligned, so every lane stores whole 16-byte words;
- * the packed source can start at any byte, so its 16-byte loads are unaligned
- * (gfx950 runs compute queues in unaligned access mode).  A wavefront covers
- * 4 KiB per trip: four independent loads per lane are issued before the four
- * stores, which keeps 4 x 1 KiB in flight per wave.  The sub-16-byte tail goes
- * out as single bytes so that nothing outside [dst, dst+len) is written.
+ * Work mapping: one 64-lane wavefront per buffer.  Destinations are 64-byte
+ * aligned, so every lane stores whole 16-byte words.  A wavefront covers up to
+ * 8 KiB (the eager limit) per trip: all eight loads of a lane are issued before
+ * its first store, so the whole buffer is in flight at once whatever its length.
+ * The table entry of the buffer is wave-uniform and is read through the scalar
+ * cache.
+ *
+ * The packed source can start at any byte.  16-byte loads from a 4-byte-aligned
+ * address run at full rate on gfx950, loads from an odd byte address do not
+ * (measured: about 15 % slower), so a source that is not 4-byte aligned is read
+ * as aligned dwords -- four plus the one that follows -- and each output dword
+ * is cut out of two neighbours with v_alignbyte_b32.  The fifth dword always
+ * contains at least one byte of the buffer, so nothing beyond the dword that
+ * holds the last source byte is read.  The sub-16-byte tail goes out as single
+ * bytes so that nothing outside [dst, dst+len) is written.
  *
  * Flush: the wave waits until its own stores have left the CU (they are
  * write-through to the L2 of its XCD), then lane 0 re-reads the first 4 bytes
@@ -25,19 +33,64 @@
 #include "common.hpp"
 #include "ofi_amd_hotpath.h"
 
+#ifndef OFI_BOUNCE_WAVES
+#define OFI_BOUNCE_WAVES 1 /* 64-thread workgroups measured fastest: finer-grained slot reuse */
+#endif
+
 namespace {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-struct __attribute__((packed, aligned(1))) unaligned_u32x4 {
+/* 16 bytes at a 4-byte-aligned address */
+struct __attribute__((packed, aligned(4))) dword_aligned_u32x4 {
 	u32x4 v;
 };
 
-constexpr int kWavesPerBlock = 4;
+constexpr int kWavesPerBlock = OFI_BOUNCE_WAVES;
 constexpr int kBlock = 64 * kWavesPerBlock;
+#ifndef OFI_BOUNCE_DEPTH
+#define OFI_BOUNCE_DEPTH 8
+#endif
+constexpr uint32_t kVecPerTrip = OFI_BOUNCE_DEPTH; /* 16-byte words per lane per trip: 8 KiB per wave */
 
-__device__ __forceinline__ u32x4 load16_unaligned(const uint8_t *p)
+__device__ __forceinline__ u32x4 load16_dword_aligned(const uint8_t *p)
 {
-	return reinterpret_cast<const unaligned_u32x4 *>(p)->v;
+	return reinterpret_cast<const dword_aligned_u32x4 *>(p)->v;
+}
+
+/* Copies nvec 16-byte words from s (4-byte aligned) + shift bytes to d (16-byte aligned).
+ * SHIFTED = false: shift is 0 and the source words are used as they are. */
+template <bool SHIFTED>
+__device__ __forceinline__ void copy_words(const uint8_t *__restrict__ s, uint8_t *__restrict__ d,
+					   uint32_t nvec, uint32_t shift, uint32_t lane)
+{
+	for (uint32_t base = 0; base < nvec; base += kVecPerTrip * 64u) {
+		u32x4 v[kVecPerTrip];
+		uint32_t x[kVecPerTrip];
+#pragma unroll
+		for (uint32_t k = 0; k < kVecPerTrip; k++) {
+			const uint32_t j = base + k * 64u + lane;
+			if (j < nvec) {
+				v[k] = load16_dword_aligned(s + ((uint64_t)j << 4));
+				if (SHIFTED) {
+					x[k] = *reinterpret_cast<const uint32_t *>(s + ((uint64_t)j << 4) + 16);
+				}
+			}
+		}
+#pragma unroll
+		for (uint32_t k = 0; k < kVecPerTrip; k++) {
+			const uint32_t j = base + k * 64u + lane;
+			if (j < nvec) {
+				u32x4 o = v[k];
+				if (SHIFTED) {
+					o.x = __builtin_amdgcn_alignbyte(v[k].y, v[k].x, shift);
+					o.y = __builtin_amdgcn_alignbyte(v[k].z, v[k].y, shift);
+					o.z = __builtin_amdgcn_alignbyte(v[k].w, v[k].z, shift);
+					o.w = __builtin_amdgcn_alignbyte(x[k], v[k].w, shift);
+				}
+				__builtin_nontemporal_store(o, reinterpret_cast<u32x4 *>(d + ((uint64_t)j << 4)));
+			}
+		}
+	}
 }
 
 __global__ __launch_bounds__(kBlock) void bounce_scatter_kernel(
@@ -47,13 +100,15 @@ __global__ __launch_bounds__(kBlock) void bounce_scatter_kernel(
 	uint32_t *__restrict__ err)
 {
 	const uint32_t lane = threadIdx.x & 63u;
-	const uint32_t buf = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+	const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const uint32_t buf = blockIdx.x * kWavesPerBlock + wave;
 	if (buf >= n) {
 		return;
 	}
 
 	const uint64_t doff = dst_off[buf];
 	const uint32_t bytes = len[buf];
+	const uint64_t soff = src_off[buf];
 	/* precondition check: skip (and report) instead of writing out of range */
 	if ((doff & 63u) != 0 || doff > arena_bytes || bytes > arena_bytes - doff) {
 		if (lane == 0) {
@@ -62,30 +117,26 @@ __global__ __launch_bounds__(kBlock) void bounce_scatter_kernel(
 		return;
 	}
 
-	const uint8_t *s = src + src_off[buf];
+	const uint8_t *s = src + soff;
 	uint8_t *d = arena + doff;
 	const uint32_t nvec = bytes >> 4;
-
-	/* 4 x 16 B per lane per trip */
-	uint32_t j = lane;
-	for (; j + 192u < nvec; j += 256u) {
-		u32x4 a = load16_unaligned(s + ((uint64_t)j << 4));
-		u32x4 b = load16_unaligned(s + ((uint64_t)(j + 64u) << 4));
-		u32x4 c = load16_unaligned(s + ((uint64_t)(j + 128u) << 4));
-		u32x4 e = load16_unaligned(s + ((uint64_t)(j + 192u) << 4));
-		__builtin_nontemporal_store(a, reinterpret_cast<u32x4 *>(d + ((uint64_t)j << 4)));
-		__builtin_nontemporal_store(b, reinterpret_cast<u32x4 *>(d + ((uint64_t)(j + 64u) << 4)));
-		__builtin_nontemporal_store(c, reinterpret_cast<u32x4 *>(d + ((uint64_t)(j + 128u) << 4)));
-		__builtin_nontemporal_store(e, reinterpret_cast<u32x4 *>(d + ((uint64_t)(j + 192u) << 4)));
-	}
-	for (; j < nvec; j += 64u) {
-		u32x4 a = load16_unaligned(s + ((uint64_t)j << 4));
-		__builtin_nontemporal_store(a, reinterpret_cast<u32x4 *>(d + ((uint64_t)j << 4)));
-	}
 	const uint32_t tail = bytes & 15u;
+
+	/* tail bytes first, so their latency overlaps the body */
+	uint8_t tail_byte = 0;
+	const uint64_t tail_at = ((uint64_t)nvec << 4) + lane;
 	if (lane < tail) {
-		const uint64_t o = ((uint64_t)nvec << 4) + lane;
-		d[o] = s[o];
+		tail_byte = s[tail_at];
+	}
+
+	const uint32_t shift = (uint32_t)(reinterpret_cast<uintptr_t>(s) & 3u);
+	if (shift == 0) {
+		copy_words<false>(s, d, nvec, 0, lane);
+	} else {
+		copy_words<true>(s - shift, d, nvec, shift, lane);
+	}
+	if (lane < tail) {
+		d[tail_at] = tail_byte;
 	}
 
 	if (flush != nullptr) {
