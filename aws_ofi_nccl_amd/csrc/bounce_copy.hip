@@ -47,6 +47,7 @@ struct __attribute__((packed, aligned(4))) dword_aligned_u32x4 {
 
 constexpr int kWavesPerBlock = OFI_BOUNCE_WAVES;
 constexpr int kBlock = 64 * kWavesPerBlock;
+constexpr uint32_t kXcds = 8;
 #ifndef OFI_BOUNCE_DEPTH
 #define OFI_BOUNCE_DEPTH 8
 #endif
@@ -101,7 +102,12 @@ __global__ __launch_bounds__(kBlock) void bounce_scatter_kernel(
 {
 	const uint32_t lane = threadIdx.x & 63u;
 	const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-	const uint32_t buf = blockIdx.x * kWavesPerBlock + wave;
+	/* Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give every
+	 * XCD one contiguous eighth of the batch, so that neighbouring buffers -- which share
+	 * a cache line of the packed source at their boundary -- meet in the same L2. */
+	const uint32_t per_xcd = gridDim.x / kXcds;
+	const uint32_t wg = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
+	const uint32_t buf = wg * kWavesPerBlock + wave;
 	if (buf >= n) {
 		return;
 	}
@@ -188,7 +194,8 @@ int ofi_amd_bounce_scatter(const void *d_src, void *d_arena, uint64_t arena_byte
 	if (!err) {
 		return -ENOMEM;
 	}
-	const uint32_t blocks = (n + kWavesPerBlock - 1) / kWavesPerBlock;
+	uint32_t blocks = (n + kWavesPerBlock - 1) / kWavesPerBlock;
+	blocks = (blocks + kXcds - 1) / kXcds * kXcds; /* whole rounds over the XCDs */
 	hipLaunchKernelGGL(bounce_scatter_kernel, dim3(blocks), dim3(kBlock), 0, as_stream(stream),
 			   static_cast<const uint8_t *>(d_src), static_cast<uint8_t *>(d_arena),
 			   arena_bytes, d_src_off, d_dst_off, d_len, n, d_flush, err);
