@@ -259,6 +259,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--gin-ops", type=int, default=1_000_000, help="GIN ops per context")
     ap.add_argument("--skip-extra", action="store_true", help="only the bounce-copy step")
+    ap.add_argument("--extra", default="striping,tuner,gin", help="which other paths to time")
     ap.add_argument("--skip-cpu", action="store_true", help="no CPU baselines")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -283,13 +284,15 @@ def main():
     extra = {}
     if not args.skip_extra:
         for name, fn in (("striping", bench_sched), ("tuner", bench_tuner), ("gin", bench_gin)):
+            if name not in args.extra.split(","):
+                continue
             log(name)
             extra[name] = fn(lib, oracle, torch, np, args)
 
-    traffic = None
-    prof = os.path.join(ROOT, "profiles", "bounce_scatter_traffic.json")
-    if os.path.exists(prof):
-        traffic = json.load(open(prof)).get("hbm_bytes_per_launch")
+    # HBM bytes per launch of bounce_scatter_kernel on this batch, from the rocprofv3 FETCH_SIZE /
+    # WRITE_SIZE runs summarised in profiles/bounce_scatter_kernel_65536buf_2GiB_arena.md
+    # (273,047.6 KiB read + 269,222.9 KiB written after scaling by the plain-copy factors)
+    traffic = 555285000 if bounce["buffers"] == 65536 else None
     line = {
         "metric": "GIN puts/sec + bounce-copy GB/s on 1 MI355X (% of HBM/host-link peak)",
         "value": bounce["gbs_wall"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
