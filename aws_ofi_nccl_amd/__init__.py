@@ -74,6 +74,58 @@ class GinProxyStats(ctypes.Structure):
                 ("checksum", c_u64), ("seconds", ctypes.c_double), ("empty_polls", c_u64)]
 
 
+class TunerQuery(ctypes.Structure):
+    """ofi_amd_tuner_query_t (64 bytes)"""
+    _fields_ = [("platform", c_i32), ("kind", c_i32), ("coll", c_i32), ("pipe_ops", c_i32),
+                ("num_channels", c_i32), ("net_comp_overhead", c_i32), ("algo", c_i32),
+                ("proto", c_i32), ("allowed_mask", c_u32), ("pad", c_u32), ("nbytes", c_u64),
+                ("num_ranks", c_u64), ("num_nodes", c_u64)]
+
+
+class TunerAnswer(ctypes.Structure):
+    """ofi_amd_tuner_answer_t (16 bytes)"""
+    _fields_ = [("algo", ctypes.c_int8), ("proto", ctypes.c_int8), ("nchannels", ctypes.c_int16),
+                ("pad", c_u32), ("chunk_size", c_u64)]
+
+
+class NcclTunerV2(ctypes.Structure):
+    """ncclTuner_v2_t"""
+    _fields_ = [("name", ctypes.c_char_p),
+                ("init", ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_size_t, ctypes.c_size_t, c_vp,
+                                          ctypes.POINTER(c_vp))),
+                ("getCollInfo", ctypes.CFUNCTYPE(ctypes.c_int, c_vp, ctypes.c_int, ctypes.c_size_t,
+                                                 ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                 ctypes.POINTER(ctypes.c_int),
+                                                 ctypes.POINTER(ctypes.c_int),
+                                                 ctypes.POINTER(ctypes.c_int))),
+                ("destroy", ctypes.CFUNCTYPE(ctypes.c_int, c_vp))]
+
+
+class NcclTunerV3(ctypes.Structure):
+    """ncclTuner_v3_t"""
+    _fields_ = [("name", ctypes.c_char_p),
+                ("init", ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_size_t, ctypes.c_size_t, c_vp,
+                                          ctypes.POINTER(c_vp))),
+                ("getCollInfo", ctypes.CFUNCTYPE(ctypes.c_int, c_vp, ctypes.c_int, ctypes.c_size_t,
+                                                 ctypes.c_int, c_vp, ctypes.c_int, ctypes.c_int,
+                                                 ctypes.POINTER(ctypes.c_int))),
+                ("destroy", ctypes.CFUNCTYPE(ctypes.c_int, c_vp))]
+
+
+class NcclTunerV6(ctypes.Structure):
+    """ncclTuner_v6_t"""
+    _fields_ = [("name", ctypes.c_char_p),
+                ("init", ctypes.CFUNCTYPE(ctypes.c_int, ctypes.POINTER(c_vp), c_u64, ctypes.c_size_t,
+                                          ctypes.c_size_t, c_vp, c_vp, c_vp)),
+                ("getCollInfo", ctypes.CFUNCTYPE(ctypes.c_int, c_vp, ctypes.c_int, ctypes.c_size_t,
+                                                 ctypes.c_int, c_vp, ctypes.c_int, ctypes.c_int,
+                                                 ctypes.c_int, ctypes.POINTER(ctypes.c_int))),
+                ("finalize", ctypes.CFUNCTYPE(ctypes.c_int, c_vp)),
+                ("getChunkSize", ctypes.CFUNCTYPE(ctypes.c_int, c_vp, ctypes.c_int, ctypes.c_size_t,
+                                                  ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                  ctypes.POINTER(ctypes.c_size_t)))]
+
+
 class TunerVariant(ctypes.Structure):
     _fields_ = [("platform", c_i32), ("pipe_ops", c_i32), ("num_channels", c_i32),
                 ("net_comp_overhead", c_i32)]
@@ -141,6 +193,7 @@ PROTOTYPES = {
     "ofi_amd_tuner_plan_cells": (c_u64, [c_vp]),
     "ofi_amd_tuner_model_grid": (ctypes.c_int, [c_vp, c_vp, c_u32, c_vp, c_vp, c_vp]),
     "ofi_amd_tuner_region_grid": (ctypes.c_int, [c_vp, c_vp, c_u32, c_vp, c_vp]),
+    "ofi_amd_tuner_query": (ctypes.c_int, [c_vp, c_u32, c_vp]),
 }
 
 

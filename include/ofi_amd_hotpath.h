@@ -350,6 +350,54 @@ int ofi_amd_tuner_model_grid(ofi_amd_tuner_plan_t *plan, const ofi_amd_tuner_var
 int ofi_amd_tuner_region_grid(ofi_amd_tuner_plan_t *plan, const int32_t *platforms,
 			      uint32_t n_platforms, int8_t *d_choice, void *stream);
 
+/*
+ * Point queries: a list of independent tuner questions answered in one launch.
+ * This is the form behind the plugin's per-collective calls
+ * (nccl_ofi_tuner_get_coll_info / _v2 / _v6 and nccl_ofi_tuner_get_chunk_size,
+ * src/tuner/nccl_ofi_tuner.cpp:162-272), which memoises the answers.
+ *   kind 0  region decision (region_get_coll_info_internal_v3 / _v2)
+ *   kind 1  model decision  (model_get_coll_info_internal_v3 / _v2)
+ *   kind 2  region chunk size for a given algo / proto (region_get_chunk_size_internal)
+ * allowed_mask bit (algo*3 + proto): for kind 0 a region with a clear bit is passed
+ * over (NCCL marked the cell -1, or it lies beyond numAlgo / numProto; v2: PAT, and NVLS
+ * tree without NVLS support); for kind 1 only the NVLS-tree/Simple bit is looked at.
+ */
+typedef struct {
+	int32_t platform;
+	int32_t kind;
+	int32_t coll;
+	int32_t pipe_ops;
+	int32_t num_channels;
+	int32_t net_comp_overhead;
+	int32_t algo;
+	int32_t proto;
+	uint32_t allowed_mask;
+	uint32_t pad;
+	uint64_t nbytes;
+	uint64_t num_ranks;
+	uint64_t num_nodes;
+} ofi_amd_tuner_query_t; /* 64 bytes */
+
+typedef struct {
+	int8_t algo;        /* -1: no decision, fall back to NCCL */
+	int8_t proto;
+	int16_t nchannels;  /* -1: left alone */
+	uint32_t pad;
+	uint64_t chunk_size; /* kind 2; 0: left alone */
+} ofi_amd_tuner_answer_t; /* 16 bytes */
+
+/* Synchronous: queries and answers are host arrays. */
+int ofi_amd_tuner_query(const ofi_amd_tuner_query_t *queries, uint32_t n,
+			ofi_amd_tuner_answer_t *answers);
+
+/*
+ * NCCL tuner plugin symbols, same names and struct layouts as the reference exports
+ * (src/tuner/nccl_ofi_tuner.cpp:185,242,274; nccl/tuner.h:46-87, tuner_v2.h, tuner_v6.h):
+ *   ncclTunerPlugin_v2, ncclTunerPlugin_v3, ncclTunerPlugin_v6
+ * They are data symbols of this library; their types are declared in
+ * aws_ofi_nccl_amd/csrc/nccl_tuner_abi.h.
+ */
+
 #ifdef __cplusplus
 }
 #endif

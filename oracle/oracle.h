@@ -214,6 +214,11 @@ void oracle_model_decide(int platform, int coll, int pipe_ops, uint64_t size,
 			 uint64_t num_ranks, uint64_t num_nodes, int num_channels,
 			 int net_comp_overhead, int *algo, int *proto);
 
+/* model_get_coll_info_internal_v2, :236-309 */
+void oracle_model_decide_v2(int platform, int coll, int pipe_ops, uint64_t size,
+			    uint64_t num_ranks, uint64_t num_nodes, int num_channels,
+			    int net_comp_overhead, int nvls_support, int *algo, int *proto);
+
 typedef struct { double x, y; } oracle_point_t;
 /* extend_region, src/tuner/nccl_ofi_regions.cpp:254-289 (linear in, linear out). */
 oracle_point_t oracle_region_extend(oracle_point_t a, oracle_point_t b, oracle_point_t z);
@@ -225,6 +230,10 @@ int oracle_region_inside(oracle_point_t p, const oracle_point_t *verts, size_t n
  * algo and proto are -1 on fall-back; nchannels is left alone unless overridden. */
 void oracle_region_decide(int platform, int coll, uint64_t size, uint64_t num_ranks,
 			  uint64_t num_nodes, int *algo, int *proto, int *nchannels);
+/* The same, skipping every region whose (algorithm*3 + protocol) bit is clear in allowed_mask. */
+void oracle_region_decide_masked(int platform, int coll, uint64_t size, uint64_t num_ranks,
+				 uint64_t num_nodes, uint32_t allowed_mask, int *algo, int *proto,
+				 int *nchannels);
 /* Number of polygons and log2-space vertices for one (platform, shape, coll):
  * used by tests to inspect the built table. Returns polygon count. */
 int oracle_region_polys(int platform, uint64_t num_ranks, uint64_t num_nodes, int coll,

@@ -113,6 +113,16 @@ void oracle_model_decide(int platform, int coll, int pipe_ops, uint64_t size,
 			 uint64_t num_ranks, uint64_t num_nodes, int num_channels,
 			 int net_comp_overhead, int *algo_out, int *proto_out)
 {
+	oracle_model_decide_v2(platform, coll, pipe_ops, size, num_ranks, num_nodes, num_channels,
+			       net_comp_overhead, 1, algo_out, proto_out);
+}
+
+/* model_get_coll_info_internal_v2, :236-309: as v3, but NVLS tree (and the P5 quirk
+ * that selects it) only when NCCL reports NVLS support. */
+void oracle_model_decide_v2(int platform, int coll, int pipe_ops, uint64_t size,
+			    uint64_t num_ranks, uint64_t num_nodes, int num_channels,
+			    int net_comp_overhead, int nvls_support, int *algo_out, int *proto_out)
+{
 	float lowest = FLT_MAX;
 	int chosen_algo = -1, chosen_proto = -1;
 
@@ -122,7 +132,7 @@ void oracle_model_decide(int platform, int coll, int pipe_ops, uint64_t size,
 		return;
 	}
 	if (platform == ORACLE_PLAT_P5_P5E) { /* :183-192 */
-		if (coll == FUNC_ALLREDUCE && num_nodes == 16 && num_ranks == 128 &&
+		if (coll == FUNC_ALLREDUCE && num_nodes == 16 && num_ranks == 128 && nvls_support &&
 		    size > 3ULL * 1024ULL * 1024ULL * 1024ULL &&
 		    size <= 5ULL * 1024ULL * 1024ULL * 1024ULL) {
 			*algo_out = ALGO_NVLS_TREE;
@@ -132,6 +142,9 @@ void oracle_model_decide(int platform, int coll, int pipe_ops, uint64_t size,
 	}
 	for (int algo = 0; algo < NUM_ALGOS; algo++) {
 		if (algo == ALGO_COLLNET_DIRECT || algo == ALGO_COLLNET_CHAIN || algo == ALGO_NVLS) {
+			continue;
+		}
+		if (!nvls_support && algo == ALGO_NVLS_TREE) { /* :279-280 */
 			continue;
 		}
 		for (int proto = 0; proto < NUM_PROTOS; proto++) {
@@ -469,9 +482,21 @@ static int best_nchannel_tree(uint64_t message_size, int log2_nnodes)
 	return best;
 }
 
-/* region_get_coll_info_internal_v3, :2070-2157 */
+/* region_get_coll_info_internal_v3, :2070-2157, on a table with no ignored cell */
 void oracle_region_decide(int platform, int coll, uint64_t size, uint64_t num_ranks,
 			  uint64_t num_nodes, int *algo_out, int *proto_out, int *nchannels)
+{
+	oracle_region_decide_masked(platform, coll, size, num_ranks, num_nodes, 0x1fffffu, algo_out,
+				    proto_out, nchannels);
+}
+
+/* The same with the skip rule spelled out: region i is passed over when bit
+ * (algorithm*3 + protocol) of allowed_mask is clear.  v3 clears the bits of cells NCCL
+ * marked -1 or that lie beyond numAlgo/numProto (:2109-2114); v2 clears PAT and, without
+ * NVLS support, NVLS tree (region_get_coll_info_internal_v2, :2029-2035). */
+void oracle_region_decide_masked(int platform, int coll, uint64_t size, uint64_t num_ranks,
+				 uint64_t num_nodes, uint32_t allowed_mask, int *algo_out,
+				 int *proto_out, int *nchannels)
 {
 	int in_out = -1;
 	int algorithm = -1, protocol = -1;
@@ -493,9 +518,12 @@ void oracle_region_decide(int platform, int coll, uint64_t size, uint64_t num_ra
 	for (int i = 0; i < np && in_out < 0; i++) {
 		oracle_point_t verts[MAX_VERTICES];
 		const int *poly = ofi_region_polys[ofi_region_sets[s][3] + i];
-		int nv = build_poly(s, i, verts);
 		algorithm = poly[0];
 		protocol = poly[1];
+		if (!((allowed_mask >> (algorithm * 3 + protocol)) & 1u)) {
+			continue;
+		}
+		int nv = build_poly(s, i, verts);
 		in_out = oracle_region_inside(p, verts, (size_t)nv);
 	}
 	if (in_out < 0) {

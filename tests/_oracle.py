@@ -105,6 +105,11 @@ _ORACLE_PROTOS = {
     "oracle_region_chunk_size": (c_int, [c_int, c_int, c_u64, c_int, c_int, c_u64, c_u64,
                                          ctypes.POINTER(c_u64)]),
     "oracle_chunk_tree_ll128": (c_u64, [c_u64, c_int, c_int]),
+    "oracle_model_decide_v2": (None, [c_int, c_int, c_int, c_u64, c_u64, c_u64, c_int, c_int, c_int,
+                                      ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
+    "oracle_region_decide_masked": (None, [c_int, c_int, c_u64, c_u64, c_u64, c_u32,
+                                           ctypes.POINTER(c_int), ctypes.POINTER(c_int),
+                                           ctypes.POINTER(c_int)]),
     "oracle_model_grid": (None, [c_int, c_int, c_int, c_int, c_vp, c_u32, c_vp, c_u32, c_vp, c_u32,
                                  c_vp, c_u32, c_vp, c_u32, c_vp, c_vp]),
     "oracle_region_grid": (None, [c_int, c_vp, c_u32, c_vp, c_u32, c_vp, c_u32, c_vp, c_u32, c_vp]),
