@@ -74,6 +74,22 @@ class GinProxyStats(ctypes.Structure):
                 ("checksum", c_u64), ("seconds", ctypes.c_double), ("empty_polls", c_u64)]
 
 
+class GinSignalWork(ctypes.Structure):
+    """ofi_amd_gin_signal_work_t (32 bytes)"""
+    _fields_ = [("base", c_u64), ("offset", c_u64), ("value", c_u64), ("peer", c_u32),
+                ("gate_seq", ctypes.c_uint16), ("run_len", ctypes.c_uint16)]
+
+
+class GinAck(ctypes.Structure):
+    """ofi_amd_gin_ack_t (16 bytes)"""
+    _fields_ = [("peer", c_u32), ("rx_consumed", c_u32), ("msg", c_u64)]
+
+
+class GinSignalRegion(ctypes.Structure):
+    """ofi_amd_gin_signal_region_t"""
+    _fields_ = [("base", c_u64), ("size", c_u64), ("d_counters", c_vp)]
+
+
 class TunerQuery(ctypes.Structure):
     """ofi_amd_tuner_query_t (64 bytes)"""
     _fields_ = [("platform", c_i32), ("kind", c_i32), ("coll", c_i32), ("pipe_ops", c_i32),
@@ -186,6 +202,16 @@ PROTOTYPES = {
     "ofi_amd_gin_ack_msg": (c_u64, [c_u32, c_u32]),
     "ofi_amd_gin_proxy_drain": (ctypes.c_int, [c_vp, c_u64, ctypes.c_int, c_vp, c_vp, c_vp, c_vp,
                                                c_u32, ctypes.POINTER(GinProxyStats)]),
+    "ofi_amd_gin_rx_create": (ctypes.c_int, [c_u32, ctypes.POINTER(c_u32), ctypes.POINTER(c_vp)]),
+    "ofi_amd_gin_rx_destroy": (ctypes.c_int, [c_vp]),
+    "ofi_amd_gin_rx_write_completion": (ctypes.c_int, [c_vp, c_u32, c_u32]),
+    "ofi_amd_gin_rx_metadata": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(c_u64)]),
+    "ofi_amd_gin_rx_take_work": (c_u32, [c_vp, ctypes.POINTER(GinSignalWork), c_u32]),
+    "ofi_amd_gin_rx_take_acks": (c_u32, [c_vp, ctypes.POINTER(GinAck), c_u32]),
+    "ofi_amd_gin_rx_cursors": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(c_u32),
+                                              ctypes.POINTER(c_u32)]),
+    "ofi_amd_gin_signal_apply": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(GinSignalRegion),
+                                                c_u32, c_vp, c_vp]),
     "ofi_amd_tuner_plan_create": (ctypes.c_int, [c_vp, c_u32, c_vp, c_u32, c_vp, c_u32, c_vp,
                                                  c_u32, c_vp, c_u32, ctypes.POINTER(c_vp)]),
     "ofi_amd_tuner_plan_destroy": (ctypes.c_int, [c_vp]),

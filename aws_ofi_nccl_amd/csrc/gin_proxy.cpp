@@ -92,12 +92,18 @@ int ofi_amd_gin_comm_init(ofi_amd_gin_comm_t *c, uint32_t comm_id, uint32_t num_
 	return 0;
 }
 
-/* apply_rx_consumed, include/rdma/gin/nccl_ofi_gin.h:535-543 */
+/* handle_ack_completion, src/rdma/gin/nccl_ofi_gin.cpp:1843-1869, with apply_rx_consumed,
+ * include/rdma/gin/nccl_ofi_gin.h:535-543 */
 void ofi_amd_gin_apply_ack(ofi_amd_gin_comm_t *c, uint32_t wire_rx_consumed)
 {
-	const uint32_t delta = cursor_delta(wire_rx_consumed, c->tx_tail);
+	const uint32_t rx = wire_rx_consumed & kCursorMask;
+	const uint32_t delta = cursor_delta(rx, c->tx_tail);
 	if (delta > 0 && delta <= kCursorHalf) {
-		c->tx_tail = wire_rx_consumed & kCursorMask;
+		c->tx_tail = rx;
+	}
+	if (c->has_pending_ack_request &&
+	    cursor_delta(rx, c->last_ack_requested_seq) <= kCursorHalf) {
+		c->has_pending_ack_request = 0;
 	}
 }
 

@@ -1,0 +1,87 @@
+/*
+ * Signal delivery on the GPU: a batch of folded signal work items becomes one launch of
+ * 64-bit device-scope atomic adds on the counters in HBM.
+ *
+ * The reference updates each counter from a CPU worker thread through GDRCopy -- a PCIe
+ * read and a PCIe write per slot (apply_signal_work, src/rdma/gin/nccl_ofi_gin.cpp:
+ * 1193-1256) -- and therefore folds a batch by slot first to save round trips
+ * (apply_and_complete, :1425-1479).  With the adds executed next to the memory the fold
+ * is unnecessary for speed and, additions being commutative, for the result: N items on
+ * one slot leave it at the same value as the reference's single +sum write.
+ */
+#include "common.hpp"
+#include "ofi_amd_hotpath.h"
+
+namespace {
+
+constexpr uint32_t kMaxRegions = 16;
+
+struct regions_t {
+	uint64_t base[kMaxRegions];
+	uint64_t size[kMaxRegions];
+	uint64_t *counters[kMaxRegions];
+	uint32_t n;
+};
+
+__global__ __launch_bounds__(256) void gin_signal_apply_kernel(
+	const ofi_amd_gin_signal_work_t *__restrict__ work, uint32_t n, regions_t regions,
+	uint32_t *__restrict__ rejected)
+{
+	const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+	if (i >= n) {
+		return;
+	}
+	const ofi_amd_gin_signal_work_t w = work[i];
+	uint64_t *slot = nullptr;
+	for (uint32_t r = 0; r < regions.n; r++) {
+		if (w.base == regions.base[r] && w.offset <= regions.size[r] &&
+		    regions.size[r] - w.offset >= 8) {
+			slot = regions.counters[r] + (w.offset >> 3);
+			break;
+		}
+	}
+	if (slot == nullptr || (w.offset & 7u) != 0) {
+		if (rejected) {
+			atomicAdd(rejected, 1u);
+		}
+		return;
+	}
+	/* relaxed: ordering against the payload is the put-before-signal protocol's business
+	 * (the reference uses a relaxed fetch_add on its host path for the same reason, :1209) */
+	__hip_atomic_fetch_add(slot, w.value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+} // namespace
+
+using namespace ofi_amd;
+
+extern "C" int ofi_amd_gin_signal_apply(const ofi_amd_gin_signal_work_t *d_work, uint32_t n,
+					const ofi_amd_gin_signal_region_t *regions, uint32_t n_regions,
+					uint32_t *d_rejected, void *stream)
+{
+	int rc = require_device();
+	if (rc != 0) {
+		return rc;
+	}
+	if (n == 0) {
+		return 0;
+	}
+	if (!d_work || !regions || n_regions == 0 || n_regions > kMaxRegions) {
+		return -EINVAL;
+	}
+	regions_t r;
+	r.n = n_regions;
+	for (uint32_t i = 0; i < kMaxRegions; i++) {
+		const bool live = i < n_regions;
+		if (live && (!regions[i].d_counters || (reinterpret_cast<uintptr_t>(regions[i].d_counters) & 7u))) {
+			return -EINVAL;
+		}
+		r.base[i] = live ? regions[i].base : 0;
+		r.size[i] = live ? regions[i].size : 0;
+		r.counters[i] = live ? static_cast<uint64_t *>(regions[i].d_counters) : nullptr;
+	}
+	hipLaunchKernelGGL(gin_signal_apply_kernel, dim3((n + 255u) / 256u), dim3(256), 0, as_stream(stream),
+			   d_work, n, r, d_rejected);
+	OFI_AMD_HIP_TRY(hipGetLastError());
+	return 0;
+}

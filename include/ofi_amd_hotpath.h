@@ -295,6 +295,70 @@ int ofi_amd_gin_proxy_drain(ofi_amd_gin_rings_t *rings, uint64_t ops_per_context
 			    const ofi_amd_gin_mr_t *mrs, ofi_amd_gin_wire_t *out_wire,
 			    uint32_t timeout_ms, ofi_amd_gin_proxy_stats_t *stats);
 
+/* ---- receiver side: completions -> in-order retire -> signal counters in HBM ---- */
+
+/* One folded signal delivery: add `value` to the 8-byte counter at base + offset
+ * (gin_signal_work_entry, include/rdma/gin/nccl_ofi_gin.h:257-299, reduced to what the
+ * update needs).  32 bytes. */
+typedef struct {
+	uint64_t base;     /* signal_base_address: the VA the initiator knows the signal MR by */
+	uint64_t offset;
+	uint64_t value;
+	uint32_t peer;
+	uint16_t gate_seq; /* sequence number of the last op folded in */
+	uint16_t run_len;  /* number of consecutive ops folded in */
+} ofi_amd_gin_signal_work_t;
+
+/* Standalone ACK to send back (gin_ack_msg_t in `msg`). */
+typedef struct {
+	uint32_t peer;
+	uint32_t rx_consumed;
+	uint64_t msg;
+} ofi_amd_gin_ack_t;
+
+typedef struct ofi_amd_gin_rx ofi_amd_gin_rx_t;
+
+/*
+ * Receiver state of one put-comm for n_peers initiators (peer_comm_ids[p] = the comm id
+ * peer p expects in ACKs).  Feed it the completions the CQ delivers, in arrival order:
+ * handle_signal_write_completion / handle_signal_metadata_completion,
+ * src/rdma/gin/nccl_ofi_gin.cpp:1792-1924.  Ops retire strictly in sequence order per
+ * peer; consecutive ready signals to the same (base, offset) fold into one work item
+ * (retire_completed_peer_iput_ops, :1622-1790); an ACK is queued when a retired op asked
+ * for one.  The hand-off of a work item is synchronous here (the reference's closing-path
+ * behaviour, :1298-1304), so the output depends only on the arrival order.
+ */
+int ofi_amd_gin_rx_create(uint32_t n_peers, const uint32_t *peer_comm_ids, ofi_amd_gin_rx_t **out);
+int ofi_amd_gin_rx_destroy(ofi_amd_gin_rx_t *rx);
+int ofi_amd_gin_rx_write_completion(ofi_amd_gin_rx_t *rx, uint32_t peer, uint32_t imm);
+int ofi_amd_gin_rx_metadata(ofi_amd_gin_rx_t *rx, uint32_t peer, const uint64_t meta[4]);
+/* Move queued work items / ACKs out (returns how many were written). */
+uint32_t ofi_amd_gin_rx_take_work(ofi_amd_gin_rx_t *rx, ofi_amd_gin_signal_work_t *out, uint32_t cap);
+uint32_t ofi_amd_gin_rx_take_acks(ofi_amd_gin_rx_t *rx, ofi_amd_gin_ack_t *out, uint32_t cap);
+int ofi_amd_gin_rx_cursors(const ofi_amd_gin_rx_t *rx, uint32_t peer, uint32_t *rx_consumed,
+			   uint32_t *next_seq);
+
+/* A registered signal region: initiators address it as `base`; its counters live at
+ * d_counters (device memory), `size` bytes. */
+typedef struct {
+	uint64_t base;
+	uint64_t size;
+	void *d_counters;
+} ofi_amd_gin_signal_region_t;
+
+/*
+ * Applies a batch of work items to the signal counters in HBM, replacing the reference's
+ * GDRCopy read-modify-write over PCIe (apply_signal_work, nccl_ofi_gin.cpp:1193-1256) and
+ * its per-batch same-slot fold (apply_and_complete, :1425-1479): one thread per item, one
+ * 64-bit device-scope atomic add each, so items hitting one slot combine in the L2.
+ * d_work is device-accessible (pinned host or HBM); regions is a host array (<= 16).
+ * Items that match no region or are misaligned are skipped and counted in *d_rejected
+ * (device-accessible u32, may be NULL).
+ */
+int ofi_amd_gin_signal_apply(const ofi_amd_gin_signal_work_t *d_work, uint32_t n,
+			     const ofi_amd_gin_signal_region_t *regions, uint32_t n_regions,
+			     uint32_t *d_rejected, void *stream);
+
 /* ======================================================================
  * 5. Tuner: batched cost model and region lookup.
  *    Model: nccl_ofi_tuner_compute_cost + model_get_coll_info_internal_v3,

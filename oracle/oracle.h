@@ -18,6 +18,13 @@
  *   gin iputSignal   state machine (window, pin, FI_MORE flags): PARITY UNPINNED
  *                    beyond the encoders above -- the reference has no
  *                    wire-level test for it and its source does not build here
+ *   gin receiver     end values of tests/functional/rma.cpp (64 put-signals -> 64)
+ *                    and rma_multiseg_signal.cpp (two slots, each its count)
+ *                    under arbitrary arrival orders; hand-derived fold runs;
+ *                    exactly-once in-order delivery; ACK cursor + encoding.  The
+ *                    work-item / ACK streams themselves: PARITY UNPINNED (no
+ *                    reference test observes them; source does not build here)
+ *   gin signal apply per-slot sums against a plain scatter-add (mod 2^64)
  *   region geometry  ~70 points + 4 extend_region cases of
  *                    tests/unit/region_based_tuner.cpp
  *   region tables    re-parsed from the reference source text and compared
@@ -193,6 +200,38 @@ void oracle_gin_comm_init(oracle_gin_comm_t *c, uint32_t comm_id, uint32_t num_r
  * -11 (window full and no ACK can arrive). */
 int oracle_gin_iput_signal(oracle_gin_comm_t *c, const oracle_gin_mr_t *mrs,
 			   const oracle_gin_desc_t *d, oracle_gin_wire_t *out);
+void oracle_gin_apply_ack(oracle_gin_comm_t *c, uint32_t wire_rx_consumed);
+
+/* ---- receiver side (oracle_gin_rx.c) ---- */
+
+/* One folded signal delivery: +value on the 8-byte counter at base + offset. 32 bytes. */
+typedef struct {
+	uint64_t base;
+	uint64_t offset;
+	uint64_t value;
+	uint32_t peer;
+	uint16_t gate_seq; /* sequence number of the run's last op */
+	uint16_t run_len;  /* ops folded into this item */
+} oracle_gin_signal_work_t;
+
+typedef struct {
+	uint32_t peer;
+	uint32_t rx_consumed;
+	uint64_t msg; /* gin_ack_msg_t */
+} oracle_gin_ack_t;
+
+typedef struct oracle_gin_rx oracle_gin_rx_t;
+oracle_gin_rx_t *oracle_gin_rx_create(uint32_t n_peers, const uint32_t *peer_comm_ids);
+void oracle_gin_rx_destroy(oracle_gin_rx_t *rx);
+/* a write-with-immediate completion / a 32-byte metadata message from `peer` */
+int oracle_gin_rx_write(oracle_gin_rx_t *rx, uint32_t peer, uint32_t imm);
+int oracle_gin_rx_metadata(oracle_gin_rx_t *rx, uint32_t peer, const uint64_t meta[4]);
+uint32_t oracle_gin_rx_take_work(oracle_gin_rx_t *rx, oracle_gin_signal_work_t *out, uint32_t cap);
+uint32_t oracle_gin_rx_take_acks(oracle_gin_rx_t *rx, oracle_gin_ack_t *out, uint32_t cap);
+void oracle_gin_rx_cursors(const oracle_gin_rx_t *rx, uint32_t peer, uint32_t *rx_consumed,
+			   uint32_t *next_seq);
+int oracle_gin_signal_apply(const oracle_gin_signal_work_t *batch, uint32_t n, const uint64_t *bases,
+			    const uint64_t *sizes, uint64_t *const *counters, uint32_t n_regions);
 
 uint64_t oracle_gin_fold(uint64_t h, const uint64_t *w, int n);
 uint64_t oracle_gin_stream_checksum(uint64_t seed, uint32_t n_contexts, uint64_t ops,

@@ -258,6 +258,23 @@ int oracle_gin_iput_signal(oracle_gin_comm_t *c, const oracle_gin_mr_t *mrs,
 	return 0;
 }
 
+/* handle_ack_completion, src/rdma/gin/nccl_ofi_gin.cpp:1843-1869, with apply_rx_consumed,
+ * include/rdma/gin/nccl_ofi_gin.h:535-543: a wire cursor moves the tail forward only, and
+ * by at most half the cursor space; a pending ACK request is satisfied by any cursor at or
+ * past the op that asked. */
+void oracle_gin_apply_ack(oracle_gin_comm_t *c, uint32_t wire_rx_consumed)
+{
+	const uint32_t half = (RX_CONSUMED_MASK + 1) / 2;
+	uint32_t rx = wire_rx_consumed & RX_CONSUMED_MASK;
+	uint32_t delta = cursor_delta(rx, c->tx_tail);
+	if (delta > 0 && delta <= half) {
+		c->tx_tail = rx;
+	}
+	if (c->has_pending_ack_request && cursor_delta(rx, c->last_ack_requested_seq) <= half) {
+		c->has_pending_ack_request = 0;
+	}
+}
+
 /* ---- stream checksum (defined by this project): order-sensitive per context ---- */
 
 static uint64_t rotl64(uint64_t x, int k) { return (x << k) | (x >> (64 - k)); }

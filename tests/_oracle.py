@@ -58,6 +58,15 @@ class GinComm(ctypes.Structure):
                 ("ack_model", c_u32), ("pad", c_u32)]
 
 
+class GinSignalWork(ctypes.Structure):
+    _fields_ = [("base", c_u64), ("offset", c_u64), ("value", c_u64), ("peer", c_u32),
+                ("gate_seq", ctypes.c_uint16), ("run_len", ctypes.c_uint16)]
+
+
+class GinAck(ctypes.Structure):
+    _fields_ = [("peer", c_u32), ("rx_consumed", c_u32), ("msg", c_u64)]
+
+
 class Point(ctypes.Structure):
     _fields_ = [("x", ctypes.c_double), ("y", ctypes.c_double)]
 
@@ -87,6 +96,16 @@ _ORACLE_PROTOS = {
     "oracle_gin_comm_init": (None, [ctypes.POINTER(GinComm), c_u32, c_u32, c_u64, c_u64, c_u32]),
     "oracle_gin_iput_signal": (c_int, [ctypes.POINTER(GinComm), ctypes.POINTER(GinMr),
                                        ctypes.POINTER(GinDesc), ctypes.POINTER(GinWire)]),
+    "oracle_gin_apply_ack": (None, [ctypes.POINTER(GinComm), c_u32]),
+    "oracle_gin_rx_create": (c_vp, [c_u32, ctypes.POINTER(c_u32)]),
+    "oracle_gin_rx_destroy": (None, [c_vp]),
+    "oracle_gin_rx_write": (c_int, [c_vp, c_u32, c_u32]),
+    "oracle_gin_rx_metadata": (c_int, [c_vp, c_u32, ctypes.POINTER(c_u64)]),
+    "oracle_gin_rx_take_work": (c_u32, [c_vp, ctypes.POINTER(GinSignalWork), c_u32]),
+    "oracle_gin_rx_take_acks": (c_u32, [c_vp, ctypes.POINTER(GinAck), c_u32]),
+    "oracle_gin_rx_cursors": (None, [c_vp, c_u32, ctypes.POINTER(c_u32), ctypes.POINTER(c_u32)]),
+    "oracle_gin_signal_apply": (c_int, [ctypes.POINTER(GinSignalWork), c_u32, ctypes.POINTER(c_u64),
+                                        ctypes.POINTER(c_u64), ctypes.POINTER(c_vp), c_u32]),
     "oracle_gin_fold": (c_u64, [c_u64, c_vp, c_int]),
     "oracle_gin_stream_checksum": (c_u64, [c_u64, c_u32, c_u64, c_u32, c_u32, c_u32, c_u32, c_int,
                                            c_u32, c_u64, c_u64, c_u32, ctypes.POINTER(GinMr)]),

@@ -1,0 +1,188 @@
+"""GIN signal delivery on the GPU: work items produced by the receiver become atomic adds on
+counters in HBM; the counters must end bit-exact where the oracle's batch-wise
+read-modify-write path (and a plain scatter-add) leaves them."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import _gin_rx as G
+import _gpu
+import _oracle
+import aws_ofi_nccl_amd as m
+
+pytestmark = pytest.mark.gpu
+
+SIG_BASE = 0x7F0000000000
+c_u32 = ctypes.c_uint32
+
+
+def work_array(items):
+    """[(base, offset, value, peer, gate_seq, run_len)] -> packed bytes of ofi_amd_gin_signal_work_t"""
+    dt = np.dtype([("base", "<u8"), ("offset", "<u8"), ("value", "<u8"), ("peer", "<u4"),
+                   ("gate_seq", "<u2"), ("run_len", "<u2")])
+    assert dt.itemsize == ctypes.sizeof(m.GinSignalWork) == 32
+    a = np.zeros(len(items), dtype=dt)
+    for i, it in enumerate(items):
+        a[i] = it
+    return a
+
+
+def oracle_apply(oracle, work, regions, batch=64):
+    """The reference-shaped path: batches of 64 work items, folded per slot, one r-m-w each."""
+    n_r = len(regions)
+    bases = (ctypes.c_uint64 * n_r)(*[b for b, _c in regions])
+    sizes = (ctypes.c_uint64 * n_r)(*[c.nbytes for _b, c in regions])
+    ptrs = (ctypes.c_void_p * n_r)(*[c.ctypes.data for _b, c in regions])
+    raw = work.tobytes()
+    for lo in range(0, len(work), batch):
+        n = min(batch, len(work) - lo)
+        buf = (_oracle.GinSignalWork * n).from_buffer_copy(raw[32 * lo:32 * (lo + n)])
+        assert oracle.oracle_gin_signal_apply(buf, n, bases, sizes, ptrs, n_r) > 0
+
+
+def gpu_apply(lib, work, dev_regions, rejected=None):
+    d_work = _gpu.to_dev(work.view(np.uint8))
+    regs = (m.GinSignalRegion * len(dev_regions))()
+    for i, (base, t) in enumerate(dev_regions):
+        regs[i] = m.GinSignalRegion(base, t.numel() * 8, t.data_ptr())
+    rc = lib.ofi_amd_gin_signal_apply(ctypes.c_void_p(d_work.data_ptr()), len(work), regs,
+                                      len(dev_regions),
+                                      ctypes.c_void_p(rejected.data_ptr()) if rejected is not None else None,
+                                      _gpu.stream())
+    _gpu.sync()
+    return rc
+
+
+def test_receiver_stream_to_counters(lib, oracle, gpu):
+    """Sender wire records -> reordered completions -> product receiver -> GPU counters."""
+    rng = np.random.default_rng(41)
+    slots = 512
+    ops = []
+    for i in range(7000):
+        size = int(2 ** rng.uniform(3, 20))
+        if i % 3 == 0:
+            ops.append((size, G.INC, 0, 8 * ((i // 64) % slots)))
+        elif i % 3 == 1:
+            ops.append((size, G.ADD, int(rng.integers(0, 1 << 64, dtype=np.uint64)),
+                        8 * int(rng.integers(0, slots))))
+        else:
+            ops.append((size, 0, 0, 0))
+    wire = G.sender_ops(oracle, ops, ack_model=0)
+    ev = G.reorder(G.events_of(wire), rng, 30)
+    prx = ctypes.c_void_p()
+    assert lib.ofi_amd_gin_rx_create(1, None, ctypes.byref(prx)) == 0
+    G.feed((lib.ofi_amd_gin_rx_write_completion, lib.ofi_amd_gin_rx_metadata), prx, 0, ev)
+    items = G.take_all(lib.ofi_amd_gin_rx_take_work, prx, m.GinSignalWork)
+    assert lib.ofi_amd_gin_rx_destroy(prx) == 0
+    assert sum(it[5] for it in items) == sum(1 for o in ops if o[1])
+
+    work = work_array(items)
+    start = rng.integers(0, 1 << 64, slots, dtype=np.uint64)
+    host = start.copy()
+    oracle_apply(oracle, work, [(SIG_BASE, host)])
+    # straight from the ops, without receiver or folding
+    want = [int(x) for x in start]
+    for _size, sop, val, off in ops:
+        if sop:
+            want[off // 8] = (want[off // 8] + (1 if sop == G.INC else val)) % (1 << 64)
+    assert [int(x) for x in host] == want
+
+    d_cnt = _gpu.to_dev(start)
+    assert gpu_apply(lib, work, [(SIG_BASE, d_cnt)]) == 0
+    assert np.array_equal(_gpu.to_host(d_cnt, np.uint64), host)
+
+
+@pytest.mark.parametrize("n,slots", [(1, 1), (63, 2), (100000, 8), (1 << 20, 512), (300000, 1 << 16)])
+def test_contended_slots_bit_exact(lib, oracle, gpu, n, slots):
+    rng = np.random.default_rng(n + slots)
+    vals = rng.integers(0, 1 << 64, n, dtype=np.uint64)
+    idx = rng.integers(0, slots, n)
+    dt_items = np.zeros(n, dtype=work_array([]).dtype)
+    dt_items["base"] = SIG_BASE
+    dt_items["offset"] = 8 * idx.astype(np.uint64)
+    dt_items["value"] = vals
+    dt_items["run_len"] = 1
+    start = rng.integers(0, 1 << 64, slots, dtype=np.uint64)
+    want = start.copy()
+    with np.errstate(over="ignore"):
+        np.add.at(want, idx, vals)
+    if n <= 100000:
+        host = start.copy()
+        oracle_apply(oracle, dt_items, [(SIG_BASE, host)])
+        assert np.array_equal(host, want)
+    d_cnt = _gpu.to_dev(start)
+    assert gpu_apply(lib, dt_items, [(SIG_BASE, d_cnt)]) == 0
+    assert np.array_equal(_gpu.to_host(d_cnt, np.uint64), want)
+    # a second batch accumulates on top
+    assert gpu_apply(lib, dt_items, [(SIG_BASE, d_cnt)]) == 0
+    with np.errstate(over="ignore"):
+        np.add.at(want, idx, vals)
+    assert np.array_equal(_gpu.to_host(d_cnt, np.uint64), want)
+
+
+def test_several_regions_and_rejects(lib, oracle, gpu):
+    rng = np.random.default_rng(43)
+    bases = [SIG_BASE + (i << 32) for i in range(16)]
+    sizes = [int(rng.integers(1, 200)) for _ in bases]
+    host = [np.zeros(s, dtype=np.uint64) for s in sizes]
+    items, n_bad = [], 0
+    for i in range(20000):
+        r = int(rng.integers(0, 16))
+        kind = rng.random()
+        if kind < 0.9:
+            s = int(rng.integers(0, sizes[r]))
+            v = int(rng.integers(0, 1 << 64, dtype=np.uint64))
+            items.append((bases[r], 8 * s, v, 0, i & 0x1FFF, 1))
+            host[r][s] = np.uint64((int(host[r][s]) + v) % (1 << 64))
+        elif kind < 0.94:
+            items.append((bases[r] + 8, 0, 1, 0, 0, 1)); n_bad += 1          # unknown base
+        elif kind < 0.97:
+            items.append((bases[r], 8 * sizes[r], 1, 0, 0, 1)); n_bad += 1   # one past the end
+        else:
+            items.append((bases[r], 4, 1, 0, 0, 1)); n_bad += 1              # misaligned
+    work = work_array(items)
+    dev = [(b, torch.zeros(s + 1, dtype=torch.int64, device="cuda")) for b, s in zip(bases, sizes)]
+    # the extra trailing word per region is a canary: declared size excludes it
+    regs = [(b, t[:-1]) for b, t in dev]
+    rejected = torch.zeros(1, dtype=torch.int32, device="cuda")
+    assert gpu_apply(lib, work, regs, rejected) == 0
+    assert int(rejected.item()) == n_bad and n_bad > 500
+    for (b, t), h in zip(dev, host):
+        got = _gpu.to_host(t, np.uint64)
+        assert np.array_equal(got[:-1], h)
+        assert got[-1] == 0
+
+
+def test_work_items_in_pinned_host_memory(lib, oracle, gpu):
+    """The proxy writes work items into pinned host memory and launches straight from there."""
+    n = 5000
+    rng = np.random.default_rng(44)
+    work = work_array([(SIG_BASE, 8 * int(rng.integers(0, 32)), int(rng.integers(0, 1 << 62)), 0,
+                        i & 0x1FFF, 1) for i in range(n)])
+    pinned = torch.empty(work.nbytes, dtype=torch.uint8, pin_memory=True)
+    pinned.numpy()[:] = work.view(np.uint8)
+    d_cnt = torch.zeros(32, dtype=torch.int64, device="cuda")
+    regs = (m.GinSignalRegion * 1)(m.GinSignalRegion(SIG_BASE, 256, d_cnt.data_ptr()))
+    assert lib.ofi_amd_gin_signal_apply(ctypes.c_void_p(pinned.data_ptr()), n, regs, 1, None,
+                                        _gpu.stream()) == 0
+    _gpu.sync()
+    want = np.zeros(32, dtype=np.uint64)
+    np.add.at(want, (work["offset"] // 8).astype(np.int64), work["value"])
+    assert np.array_equal(_gpu.to_host(d_cnt, np.uint64), want)
+
+
+def test_bad_arguments(lib, gpu):
+    d_cnt = torch.zeros(8, dtype=torch.int64, device="cuda")
+    regs = (m.GinSignalRegion * 1)(m.GinSignalRegion(SIG_BASE, 64, d_cnt.data_ptr()))
+    d_work = torch.zeros(32, dtype=torch.uint8, device="cuda")
+    p = ctypes.c_void_p(d_work.data_ptr())
+    assert lib.ofi_amd_gin_signal_apply(p, 0, regs, 1, None, _gpu.stream()) == 0
+    assert lib.ofi_amd_gin_signal_apply(None, 1, regs, 1, None, _gpu.stream()) == -22
+    assert lib.ofi_amd_gin_signal_apply(p, 1, None, 1, None, _gpu.stream()) == -22
+    assert lib.ofi_amd_gin_signal_apply(p, 1, regs, 0, None, _gpu.stream()) == -22
+    assert lib.ofi_amd_gin_signal_apply(p, 1, regs, 17, None, _gpu.stream()) == -22
+    odd = (m.GinSignalRegion * 1)(m.GinSignalRegion(SIG_BASE, 64, d_cnt.data_ptr() + 4))
+    assert lib.ofi_amd_gin_signal_apply(p, 1, odd, 1, None, _gpu.stream()) == -22
+    _gpu.sync()

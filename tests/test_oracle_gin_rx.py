@@ -1,0 +1,340 @@
+"""GIN receiver side: reassembly, in-order retire with same-slot folding, ACKs, and the
+signal counter update.
+
+The reference's own tests for this path are functional and check end values only
+(tests/functional/rma.cpp: 64 put-signals leave the counter at 64;
+rma_multiseg_signal.cpp: each of two slots reaches its count), so the work-item and ACK
+streams are pinned here by those end values for arbitrary arrival orders, by hand-derived
+arrival orders whose folding follows from the retire rules
+(src/rdma/gin/nccl_ofi_gin.cpp:1622-1790), and by invariants of in-order delivery.  The
+product's host receiver must then agree with the oracle event for event."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import _gin_rx as G
+import _oracle
+from _oracle import GinAck, GinSignalWork
+
+SIG_BASE = 0x7F0000000000
+c_u32 = ctypes.c_uint32
+
+
+def oracle_rx(oracle, n_peers=1, comm_ids=None):
+    ids = (c_u32 * n_peers)(*(comm_ids or [7 + p for p in range(n_peers)]))
+    rx = oracle.oracle_gin_rx_create(n_peers, ids)
+    assert rx
+    return rx
+
+
+def oracle_api(oracle):
+    return (oracle.oracle_gin_rx_write, oracle.oracle_gin_rx_metadata)
+
+
+def run_oracle(oracle, events, peer=0, n_peers=1):
+    rx = oracle_rx(oracle, n_peers)
+    G.feed(oracle_api(oracle), rx, peer, events)
+    work = G.take_all(oracle.oracle_gin_rx_take_work, rx, GinSignalWork)
+    acks = G.take_all(oracle.oracle_gin_rx_take_acks, rx, GinAck)
+    cons, nxt = c_u32(), c_u32()
+    oracle.oracle_gin_rx_cursors(rx, peer, ctypes.byref(cons), ctypes.byref(nxt))
+    oracle.oracle_gin_rx_destroy(rx)
+    return work, acks, cons.value, nxt.value
+
+
+def signals(n, slot=0, size=4096):
+    return [(size, G.INC, 0, 8 * slot)] * n
+
+
+# ---- end values the reference's functional tests check ----
+
+@pytest.mark.parametrize("lookahead", [0, 1, 7, 63])
+def test_sixty_four_put_signals_leave_sixty_four(oracle, lookahead):
+    wire = G.sender_ops(oracle, signals(64, size=42))
+    ev = G.reorder(G.events_of(wire), np.random.default_rng(lookahead), lookahead)
+    work, _acks, cons, nxt = run_oracle(oracle, ev)
+    assert int(G.slot_sums(work, 4, SIG_BASE)[0]) == 64
+    assert cons == 64 and nxt == 64
+    assert sum(w[5] for w in work) == 64
+
+
+def test_two_slots_each_reach_their_count(oracle):
+    # multi-rail payloads (4 segments + metadata) to two different slots, interleaved
+    ops = []
+    for i in range(32):
+        ops.append((1 << 20, G.INC, 0, 0))
+        ops.append((1 << 20, G.INC, 0, 8 * 300))
+    wire = G.sender_ops(oracle, ops)
+    assert all(nw == 4 for _imm, nw, _m, _a, _s in wire)
+    ev = G.reorder(G.events_of(wire), np.random.default_rng(3), 9)
+    work, _acks, cons, _nxt = run_oracle(oracle, ev)
+    sums = G.slot_sums(work, 512, SIG_BASE)
+    assert int(sums[0]) == 32 and int(sums[300]) == 32 and int(sums.sum()) == 64
+    assert cons == 64
+
+
+# ---- arrival orders whose outcome follows from the retire rules ----
+
+def test_in_order_arrival_never_folds(oracle):
+    wire = G.sender_ops(oracle, signals(20))
+    work, _a, _c, _n = run_oracle(oracle, G.events_of(wire))
+    assert [w[5] for w in work] == [1] * 20
+    assert [w[4] for w in work] == list(range(20))
+
+
+def test_reversed_arrival_folds_the_whole_run(oracle):
+    wire = G.sender_ops(oracle, signals(20))
+    ev = G.events_of(wire)
+    by_op = [[e for e in ev if e[0] == k] for k in range(20)]
+    rev = [e for k in reversed(range(20)) for e in by_op[k]]
+    work, _a, cons, _n = run_oracle(oracle, rev)
+    assert len(work) == 1
+    base, off, val, peer, gate, run = work[0]
+    assert (base, off, val, peer, gate, run) == (SIG_BASE, 0, 20, 0, 19, 20)
+    assert cons == 20
+
+
+def test_fold_stops_where_the_slot_changes(oracle):
+    # slots A A B A A A, delivered last-first: runs [A x2] [B] [A x3]
+    ops = [(256, G.ADD, 5, 0), (256, G.ADD, 6, 0), (256, G.ADD, 7, 8), (256, G.ADD, 1, 0),
+           (256, G.ADD, 2, 0), (256, G.ADD, 3, 0)]
+    wire = G.sender_ops(oracle, ops)
+    ev = G.events_of(wire)
+    rev = [e for k in reversed(range(6)) for e in ev if e[0] == k]
+    work, _a, _c, _n = run_oracle(oracle, rev)
+    assert [(w[1], w[2], w[4], w[5]) for w in work] == [(0, 11, 1, 2), (8, 7, 2, 1), (0, 6, 5, 3)]
+
+
+def test_plain_put_between_signals_breaks_the_run(oracle):
+    ops = [(256, G.INC, 0, 0), (256, 0, 0, 0), (256, G.INC, 0, 0)]
+    wire = G.sender_ops(oracle, ops)
+    assert wire[1][2] is None
+    ev = G.events_of(wire)
+    rev = [e for k in reversed(range(3)) for e in ev if e[0] == k]
+    work, _a, cons, nxt = run_oracle(oracle, rev)
+    assert [(w[2], w[4], w[5]) for w in work] == [(1, 0, 1), (1, 2, 1)]
+    assert cons == 3 and nxt == 3
+
+
+def test_nothing_is_delivered_past_a_missing_segment(oracle):
+    wire = G.sender_ops(oracle, [(1 << 20, G.INC, 0, 0)] + signals(5))
+    ev = G.events_of(wire)
+    held = ev[0]                       # one payload segment of op 0 is late
+    work, _a, cons, _n = run_oracle(oracle, ev[1:])
+    assert work == [] and cons == 0
+    work, _a, cons, _n = run_oracle(oracle, ev[1:] + [held])
+    assert sum(w[5] for w in work) == 6 and cons == 6
+    assert work[0][5] == 6             # all six were ready: one folded delivery
+
+
+def test_signal_only_and_add_values(oracle):
+    ops = [(0, G.ADD, 1 << 63, 16), (0, G.ADD, 1 << 63, 16), (0, G.ADD, 9, 16)]
+    wire = G.sender_ops(oracle, ops)
+    assert all(nw == 0 and m is not None for _i, nw, m, _a, _s in wire)
+    work, _a, _c, _n = run_oracle(oracle, G.events_of(wire))
+    assert int(G.slot_sums(work, 4, SIG_BASE)[2]) == 9      # 2^63 + 2^63 wraps to 0
+
+
+# ---- invariants under random traffic ----
+
+def random_ops(rng, n, slots=8):
+    ops = []
+    for _ in range(n):
+        size = int(2 ** rng.uniform(0, 21)) if rng.random() < 0.9 else 0
+        kind = rng.random()
+        if kind < 0.45 or size == 0:
+            sop = G.INC if rng.random() < 0.5 else G.ADD
+            ops.append((size, sop, int(rng.integers(0, 1 << 40)), 8 * int(rng.integers(0, slots))))
+        else:
+            ops.append((size, 0, 0, 0))
+    return ops
+
+
+@pytest.mark.parametrize("seed,lookahead", [(1, 0), (2, 3), (3, 40), (4, 700)])
+def test_in_order_delivery_invariants(oracle, seed, lookahead):
+    rng = np.random.default_rng(seed)
+    ops = random_ops(rng, 6000)
+    wire = G.sender_ops(oracle, ops)
+    ev = G.reorder(G.events_of(wire), rng, lookahead)
+    work, acks, cons, nxt = run_oracle(oracle, ev)
+    assert cons == len(ops) and nxt == len(ops) % 8192
+    sig_seqs = [s for (_i, _nw, m, _a, s) in wire if m is not None]
+    covered = []
+    for base, off, val, _peer, gate, run in work:
+        covered += [(gate - run + 1 + j) % 8192 for j in range(run)]
+    # every signal op delivered exactly once, in sequence order (a run may not skip a put)
+    assert covered == sig_seqs
+    # the end state equals a straight per-slot sum over the ops
+    want = np.zeros(8, dtype=np.uint64)
+    for size, sop, val, off in ops:
+        if sop:
+            want[off // 8] += np.uint64(1 if sop == G.INC else val)
+    assert np.array_equal(G.slot_sums(work, 8, SIG_BASE), want)
+    # folded values are sums of their ops
+    k = 0
+    values = [1 if sop == G.INC else val for (_s, sop, val, _o) in ops if sop]
+    for _b, _o, val, _p, _g, run in work:
+        assert val == sum(values[k:k + run]) % (1 << 64)
+        k += run
+
+
+def test_ack_carries_the_cursor_and_decodes_with_reference_bitfields(oracle, ref):
+    # past 4096 outstanding the sender asks for an ACK every 65th op (model 0: no ACK arrives)
+    ops = signals(4400, size=8)
+    wire = G.sender_ops(oracle, ops, ack_model=0)
+    asked = [k for k, w in enumerate(wire) if w[3]]
+    assert asked and asked[0] == 4096 + 64
+    work, acks, cons, _n = run_oracle(oracle, G.events_of(wire))
+    assert [a[1] for a in acks] == [k + 1 for k in asked]     # in-order arrival: one ACK per ask
+    for peer, rx_consumed, msg in acks:
+        assert msg == ref.ref_gin_ack(7, rx_consumed)
+        assert msg == oracle.oracle_gin_ack_msg(7, rx_consumed)
+
+
+def test_closed_loop_never_stalls(oracle):
+    """Sender and receiver wired back to back for four trips round the 13-bit sequence
+    space: the ACKs the receiver produces keep the sender's window open."""
+    rx = oracle_rx(oracle, 1, [5])
+    api = oracle_api(oracle)
+    rng = np.random.default_rng(11)
+    ackbuf = (GinAck * 64)()
+    workbuf = (GinSignalWork * 4096)()
+    c = _oracle.GinComm()
+    oracle.oracle_gin_comm_init(ctypes.byref(c), 5, 4, 131072, 64, 0)
+    mrs = G.make_mrs(SIG_BASE)
+    total = 4 * 8192 + 123
+    pending, n_acks, max_out, delivered = [], 0, 0, 0
+    for k in range(total):
+        d = _oracle.GinDesc(0, 0, 8, 0, 0, 1, G.INC, 0, 0, 0, 1, 2, 2)
+        w = _oracle.GinWire()
+        rc = oracle.oracle_gin_iput_signal(ctypes.byref(c), mrs, ctypes.byref(d), ctypes.byref(w))
+        assert rc == 0, "window closed at op %d" % k
+        pending.append((int(w.imm), int(w.num_writes), [int(x) for x in w.meta], int(w.ack_req),
+                        int(w.seq)))
+        max_out = max(max_out, (c.tx_head - c.tx_tail) & 0x3FFF)
+        if len(pending) < 5000 and k != total - 1:
+            continue
+        # the receiver lags: it sees a burst, out of order within the burst
+        G.feed(api, rx, 0, G.reorder(G.events_of(pending), rng, 50))
+        pending = []
+        for i in range(oracle.oracle_gin_rx_take_acks(rx, ackbuf, 64)):
+            oracle.oracle_gin_apply_ack(ctypes.byref(c), ackbuf[i].rx_consumed)
+            n_acks += 1
+        n = oracle.oracle_gin_rx_take_work(rx, workbuf, 4096)
+        while n:
+            delivered += sum(workbuf[i].run_len for i in range(n))
+            n = oracle.oracle_gin_rx_take_work(rx, workbuf, 4096)
+    assert delivered == total
+    assert n_acks > 0 and 4096 < max_out <= 8192
+    cons, nxt = c_u32(), c_u32()
+    oracle.oracle_gin_rx_cursors(rx, 0, ctypes.byref(cons), ctypes.byref(nxt))
+    assert cons.value == total % 16384 and nxt.value == total % 8192
+    oracle.oracle_gin_rx_destroy(rx)
+
+
+# ---- the counter update ----
+
+def test_batch_apply_matches_a_plain_scatter_add(oracle):
+    rng = np.random.default_rng(5)
+    n, slots = 64, 16
+    bases = (ctypes.c_uint64 * 2)(SIG_BASE, SIG_BASE + (1 << 30))
+    sizes = (ctypes.c_uint64 * 2)(8 * slots, 8 * slots)
+    c0 = rng.integers(0, 1 << 63, slots, dtype=np.uint64)
+    c1 = rng.integers(0, 1 << 63, slots, dtype=np.uint64)
+    want = [c0.copy(), c1.copy()]
+    batch = (GinSignalWork * n)()
+    for i in range(n):
+        r = int(rng.integers(0, 2))
+        s = int(rng.integers(0, slots if i % 2 else 3))
+        v = int(rng.integers(0, 1 << 64, dtype=np.uint64))
+        batch[i] = GinSignalWork(bases[r], 8 * s, v, 0, i, 1)
+        want[r][s] = np.uint64((int(want[r][s]) + v) % (1 << 64))
+    ptrs = (ctypes.c_void_p * 2)(c0.ctypes.data, c1.ctypes.data)
+    rmw = oracle.oracle_gin_signal_apply(batch, n, bases, sizes, ptrs, 2)
+    distinct = len({(batch[i].base, batch[i].offset) for i in range(n)})
+    assert rmw == distinct               # one read-modify-write per slot touched
+    assert np.array_equal(c0, want[0]) and np.array_equal(c1, want[1])
+
+
+def test_batch_apply_rejects_unknown_region_and_misaligned_offset(oracle):
+    bases = (ctypes.c_uint64 * 1)(SIG_BASE)
+    sizes = (ctypes.c_uint64 * 1)(64)
+    c0 = np.zeros(8, dtype=np.uint64)
+    ptrs = (ctypes.c_void_p * 1)(c0.ctypes.data)
+    for bad in (GinSignalWork(SIG_BASE + 8, 0, 1, 0, 0, 1), GinSignalWork(SIG_BASE, 64, 1, 0, 0, 1),
+                GinSignalWork(SIG_BASE, 4, 1, 0, 0, 1)):
+        batch = (GinSignalWork * 1)(bad)
+        assert oracle.oracle_gin_signal_apply(batch, 1, bases, sizes, ptrs, 1) == -22
+    assert not c0.any()
+
+
+# ---- the product's host receiver against the oracle ----
+
+def product_api(lib):
+    return (lib.ofi_amd_gin_rx_write_completion, lib.ofi_amd_gin_rx_metadata)
+
+
+@pytest.mark.parametrize("seed,lookahead,ack_model", [(21, 0, 1), (22, 5, 1), (23, 90, 0),
+                                                      (24, 2000, 0)])
+def test_product_receiver_matches_oracle(lib, oracle, seed, lookahead, ack_model):
+    import aws_ofi_nccl_amd as m
+    rng = np.random.default_rng(seed)
+    n_peers = 3
+    ids = (c_u32 * n_peers)(11, 12, 1023)
+    orx = oracle.oracle_gin_rx_create(n_peers, ids)
+    prx = ctypes.c_void_p()
+    assert lib.ofi_amd_gin_rx_create(n_peers, ids, ctypes.byref(prx)) == 0
+    for peer in range(n_peers):
+        ops = random_ops(rng, 8000 if ack_model == 0 else 3000, slots=4)
+        wire = G.sender_ops(oracle, ops, comm_id=int(ids[peer]), ack_model=ack_model)
+        ev = G.reorder(G.events_of(wire), rng, lookahead)
+        G.feed(oracle_api(oracle), orx, peer, ev)
+        G.feed(product_api(lib), prx, peer, ev)
+        oc, on, pc, pn = c_u32(), c_u32(), c_u32(), c_u32()
+        oracle.oracle_gin_rx_cursors(orx, peer, ctypes.byref(oc), ctypes.byref(on))
+        assert lib.ofi_amd_gin_rx_cursors(prx, peer, ctypes.byref(pc), ctypes.byref(pn)) == 0
+        assert (oc.value, on.value) == (pc.value, pn.value) == (len(ops) % 16384, len(ops) % 8192)
+    ow = G.take_all(oracle.oracle_gin_rx_take_work, orx, GinSignalWork)
+    pw = G.take_all(lib.ofi_amd_gin_rx_take_work, prx, m.GinSignalWork)
+    oa = G.take_all(oracle.oracle_gin_rx_take_acks, orx, GinAck)
+    pa = G.take_all(lib.ofi_amd_gin_rx_take_acks, prx, m.GinAck)
+    assert len(ow) > 1000 and ow == pw
+    assert oa == pa
+    if ack_model == 0:
+        assert len(oa) > 0
+    oracle.oracle_gin_rx_destroy(orx)
+    assert lib.ofi_amd_gin_rx_destroy(prx) == 0
+
+
+def test_product_apply_ack_matches_oracle(lib, oracle):
+    import aws_ofi_nccl_amd as m
+    rng = np.random.default_rng(31)
+    oc, pc = _oracle.GinComm(), m.GinComm()
+    oracle.oracle_gin_comm_init(ctypes.byref(oc), 3, 4, 131072, 64, 0)
+    assert lib.ofi_amd_gin_comm_init(ctypes.byref(pc), 3, 4, 131072, 64, 0) == 0
+    for _ in range(20000):
+        head = int(rng.integers(0, 1 << 14))
+        tail = (head - int(rng.integers(0, 8193))) & 0x3FFF
+        for c in (oc, pc):
+            c.tx_head, c.tx_tail = head, tail
+            c.last_ack_requested_seq = (head - 1) & 0x3FFF
+            c.has_pending_ack_request = 1
+        wire = int(rng.integers(0, 1 << 14))
+        oracle.oracle_gin_apply_ack(ctypes.byref(oc), wire)
+        lib.ofi_amd_gin_apply_ack(ctypes.byref(pc), wire)
+        assert (oc.tx_tail, oc.has_pending_ack_request) == (pc.tx_tail, pc.has_pending_ack_request)
+        moved = (wire - tail) & 0x3FFF
+        assert oc.tx_tail == (wire if 0 < moved <= 8192 else tail)
+
+
+def test_product_receiver_bad_arguments(lib):
+    prx = ctypes.c_void_p()
+    assert lib.ofi_amd_gin_rx_create(0, None, ctypes.byref(prx)) == -22
+    assert lib.ofi_amd_gin_rx_create(1, None, None) == -22
+    assert lib.ofi_amd_gin_rx_create(2, None, ctypes.byref(prx)) == 0
+    assert lib.ofi_amd_gin_rx_write_completion(prx, 2, 0) == -22
+    ack_as_meta = (ctypes.c_uint64 * 4)(1, 0, 0, 0)          # msg_type 1 is an ACK, not metadata
+    assert lib.ofi_amd_gin_rx_metadata(prx, 0, ack_as_meta) == -22
+    assert lib.ofi_amd_gin_rx_destroy(prx) == 0
+    assert lib.ofi_amd_gin_rx_destroy(None) == -22
