@@ -62,6 +62,11 @@ constexpr int kWavesPerBlock = OFI_BOUNCE_WAVES;
 constexpr int kBlock = 64 * kWavesPerBlock;
 constexpr uint32_t kXcds = 8;
 constexpr uint32_t kGroup = OFI_BOUNCE_GROUP;
+#ifndef OFI_BOUNCE_LDS
+#define OFI_BOUNCE_LDS 0
+#endif
+/* Unused LDS requested per workgroup: caps the workgroups resident on a CU (160 KiB each). */
+constexpr uint32_t kLdsPerBlock = OFI_BOUNCE_LDS;
 constexpr uint32_t kRows = 8;              /* rows of 64 x 16 bytes per trip: 8 KiB per wave */
 constexpr uint32_t kTripVec = kRows * 64u; /* 16-byte words per trip */
 
@@ -236,7 +241,7 @@ int ofi_amd_bounce_scatter(const void *d_src, void *d_arena, uint64_t arena_byte
 	uint32_t blocks = (n + kWavesPerBlock - 1) / kWavesPerBlock;
 	const uint32_t round = kXcds * kGroup; /* whole rounds over the XCDs */
 	blocks = (blocks + round - 1) / round * round;
-	hipLaunchKernelGGL(bounce_scatter_kernel, dim3(blocks), dim3(kBlock), 0, as_stream(stream),
+	hipLaunchKernelGGL(bounce_scatter_kernel, dim3(blocks), dim3(kBlock), kLdsPerBlock, as_stream(stream),
 			   static_cast<const uint8_t *>(d_src), static_cast<uint8_t *>(d_arena),
 			   arena_bytes, d_src_off, d_dst_off, d_len, n, d_flush, err);
 	OFI_AMD_HIP_TRY(hipGetLastError());
