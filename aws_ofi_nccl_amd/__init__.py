@@ -90,6 +90,39 @@ class GinSignalRegion(ctypes.Structure):
     _fields_ = [("base", c_u64), ("size", c_u64), ("d_counters", c_vp)]
 
 
+class EagerHdr(ctypes.Structure):
+    """ofi_amd_eager_hdr_t (8 bytes)"""
+    _fields_ = [("eager_offset", ctypes.c_uint8), ("prev_batch_count", ctypes.c_uint8),
+                ("eager_seq", ctypes.c_uint16), ("tag", c_i32)]
+
+
+class CtrlEntry(ctypes.Structure):
+    """ofi_amd_ctrl_entry_t (64 bytes)"""
+    _fields_ = [("buff_offset", c_u64), ("mr_key", c_u64 * 4), ("buff_len", c_u32),
+                ("tag", ctypes.c_int16), ("flags", ctypes.c_uint16), ("num_recvs", ctypes.c_uint16),
+                ("recv_idx", ctypes.c_uint8), ("entry_used", ctypes.c_uint8),
+                ("pad", ctypes.c_uint8 * 10), ("msg_seq_num", ctypes.c_uint16)]
+
+
+class CtrlMsg(ctypes.Structure):
+    """ofi_amd_ctrl_msg_t (512 bytes)"""
+    _fields_ = [("entries", CtrlEntry * 8)]
+
+
+class EagerEntry(ctypes.Structure):
+    """ofi_amd_eager_entry_t (24 bytes)"""
+    _fields_ = [("eager_offset", ctypes.c_uint8), ("prev_batch_count", ctypes.c_uint8),
+                ("eager_seq", ctypes.c_uint16), ("msg_seq_num", ctypes.c_uint16),
+                ("pad", ctypes.c_uint16), ("tag", c_i32), ("recv_len", c_u32), ("cookie", c_u64)]
+
+
+class EagerTx(ctypes.Structure):
+    """ofi_amd_eager_tx_t"""
+    _fields_ = [("eager_seq_next", ctypes.c_uint16), ("cur_eager_seq", ctypes.c_uint16),
+                ("eager_offset_next", ctypes.c_uint8), ("prev_eager_batch_count", ctypes.c_uint8),
+                ("pad", ctypes.c_uint16)]
+
+
 class TunerQuery(ctypes.Structure):
     """ofi_amd_tuner_query_t (64 bytes)"""
     _fields_ = [("platform", c_i32), ("kind", c_i32), ("coll", c_i32), ("pipe_ops", c_i32),
@@ -176,6 +209,8 @@ PROTOTYPES = {
                                                   ctypes.POINTER(XferInfo)]),
     "ofi_amd_bounce_scatter": (ctypes.c_int, [c_vp, c_vp, c_u64, c_vp, c_vp, c_vp, c_u32, c_vp,
                                               c_vp]),
+    "ofi_amd_eager_copy_batch": (ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_u32, c_vp, c_vp,
+                                                c_vp]),
     "ofi_amd_flush_read": (ctypes.c_int, [c_vp, c_vp, c_u32, c_vp, c_vp]),
     "ofi_amd_devcopy_register": (ctypes.c_int, [c_vp, ctypes.c_size_t, ctypes.POINTER(c_vp)]),
     "ofi_amd_devcopy_to_device": (ctypes.c_int, [c_vp, c_vp, ctypes.c_size_t, ctypes.c_size_t]),
@@ -212,6 +247,31 @@ PROTOTYPES = {
                                               ctypes.POINTER(c_u32)]),
     "ofi_amd_gin_signal_apply": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(GinSignalRegion),
                                                 c_u32, c_vp, c_vp]),
+    "ofi_amd_rdma_imm": (c_u32, [c_u32, c_u32, c_u32, c_u32]),
+    "ofi_amd_rdma_imm_decode": (None, [c_u32] + [ctypes.POINTER(c_u32)] * 4),
+    "ofi_amd_ctrl_mailbox_slot": (c_u32, [ctypes.c_uint16]),
+    "ofi_amd_ctrl_msg_fill": (ctypes.c_int, [ctypes.POINTER(CtrlMsg), ctypes.c_uint16, ctypes.c_uint16,
+                                             ctypes.POINTER(c_u64), ctypes.POINTER(c_u32),
+                                             ctypes.POINTER(ctypes.c_int), ctypes.POINTER(c_u64), c_u32,
+                                             ctypes.c_int]),
+    "ofi_amd_ctrl_msg_ready": (ctypes.c_int, [ctypes.POINTER(CtrlMsg), ctypes.c_uint16, ctypes.c_int,
+                                              ctypes.c_int]),
+    "ofi_amd_ctrl_msg_find_tag": (ctypes.c_int, [ctypes.POINTER(CtrlMsg), ctypes.c_int]),
+    "ofi_amd_seq_before": (ctypes.c_int, [ctypes.c_uint16, ctypes.c_uint16]),
+    "ofi_amd_eager_seq_before": (ctypes.c_int, [ctypes.c_uint16, ctypes.c_uint16]),
+    "ofi_amd_eager_entry_less": (ctypes.c_int, [ctypes.POINTER(EagerEntry), ctypes.POINTER(EagerEntry)]),
+    "ofi_amd_eager_entry_can_process": (ctypes.c_int, [ctypes.c_int, ctypes.c_uint16, ctypes.c_uint8,
+                                                       ctypes.POINTER(EagerEntry)]),
+    "ofi_amd_eager_rxq_create": (ctypes.c_int, [ctypes.POINTER(c_vp)]),
+    "ofi_amd_eager_rxq_destroy": (ctypes.c_int, [c_vp]),
+    "ofi_amd_eager_rxq_insert": (ctypes.c_int, [c_vp, ctypes.POINTER(EagerEntry)]),
+    "ofi_amd_eager_rxq_drain": (c_u32, [c_vp, ctypes.POINTER(EagerEntry), c_u32]),
+    "ofi_amd_eager_rxq_pending": (c_u32, [c_vp]),
+    "ofi_amd_eager_rxq_peek": (c_u32, [c_vp, ctypes.POINTER(EagerEntry), c_u32]),
+    "ofi_amd_eager_tx_init": (None, [ctypes.POINTER(EagerTx)]),
+    "ofi_amd_eager_tx_assign": (None, [ctypes.POINTER(EagerTx), c_i32, ctypes.POINTER(EagerHdr)]),
+    "ofi_amd_eager_tx_advance": (None, [ctypes.POINTER(EagerTx)]),
+    "ofi_amd_eager_fits": (ctypes.c_int, [c_u64, ctypes.c_int64]),
     "ofi_amd_tuner_plan_create": (ctypes.c_int, [c_vp, c_u32, c_vp, c_u32, c_vp, c_u32, c_vp,
                                                  c_u32, c_vp, c_u32, ctypes.POINTER(c_vp)]),
     "ofi_amd_tuner_plan_destroy": (ctypes.c_int, [c_vp]),

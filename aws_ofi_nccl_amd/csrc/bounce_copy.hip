@@ -198,6 +198,73 @@ __global__ __launch_bounds__(kBlock) void bounce_scatter_kernel(
 	}
 }
 
+/*
+ * The same copy for eager arrivals as they sit in rx buffers: an 8-byte header, then the
+ * payload, which goes to a receive buffer at any alignment, truncated to that buffer's
+ * length (rdma_eager_copy_req::post, src/nccl_ofi_rdma.cpp:2729-2776).  The bytes in front
+ * of the first 16-byte boundary of the destination go out singly; from there on it is the
+ * aligned-destination copy above, with whatever source alignment that leaves.
+ */
+__global__ __launch_bounds__(kBlock) void eager_copy_kernel(
+	const uint8_t *__restrict__ rx_base, const uint64_t *__restrict__ rx_off,
+	const uint32_t *__restrict__ recv_len, uint8_t *__restrict__ dst_base,
+	const uint64_t *__restrict__ dst_off, const uint32_t *__restrict__ dst_len, uint32_t n,
+	uint32_t *__restrict__ copied, uint32_t *__restrict__ flush)
+{
+	const uint32_t lane = threadIdx.x & 63u;
+	const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const uint32_t xcd = blockIdx.x % kXcds;
+	const uint32_t turn = blockIdx.x / kXcds;
+	const uint32_t wg = ((turn / kGroup) * kXcds + xcd) * kGroup + turn % kGroup;
+	const uint32_t buf = wg * kWavesPerBlock + wave;
+	if (buf >= n) {
+		return;
+	}
+	const uint8_t *s = rx_base + rx_off[buf] + 8u; /* skip nccl_ofi_eager_msg_header_t */
+	uint8_t *d = dst_base + dst_off[buf];
+	const uint32_t bytes = min(recv_len[buf], dst_len[buf]);
+	if (copied != nullptr && lane == 0) {
+		copied[buf] = bytes;
+	}
+
+	if (bytes != 0) {
+		const uint32_t head = min(bytes, (16u - (uint32_t)(reinterpret_cast<uintptr_t>(d) & 15u)) & 15u);
+		/* lanes without a head byte re-copy byte 0: same value, same place */
+		const uint32_t head_at = min(lane, max(head, 1u) - 1u);
+		const uint8_t head_byte = s[head_at];
+		const uint32_t rem = bytes - head;
+		if (rem != 0) {
+			const uint8_t *s2 = s + head;
+			uint8_t *d2 = d + head;
+			const uint32_t nvec = rem >> 4;
+			const uint32_t tail_at = min((nvec << 4) + lane, rem - 1u);
+			const uint8_t tail_byte = s2[tail_at];
+			const uint32_t shift = (uint32_t)(reinterpret_cast<uintptr_t>(s2) & 3u);
+			if (shift == 0) {
+				copy_words<false>(s2, d2, nvec, 0, lane);
+			} else {
+				copy_words<true>(s2 - shift, d2, nvec, shift, lane);
+			}
+			d2[tail_at] = tail_byte;
+		}
+		d[head_at] = head_byte;
+	}
+
+	if (flush != nullptr) {
+		__builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+		if (lane == 0) {
+			/* the first min(4, bytes) destination bytes, little-endian */
+			uint32_t word = 0;
+			for (uint32_t b = 0; b < min(bytes, 4u); b++) {
+				word |= (uint32_t)__hip_atomic_load(d + b, __ATOMIC_RELAXED,
+								    __HIP_MEMORY_SCOPE_WORKGROUP)
+					<< (8u * b);
+			}
+			flush[buf] = word;
+		}
+	}
+}
+
 __global__ __launch_bounds__(256) void flush_read_kernel(const uint8_t *__restrict__ arena,
 							 const uint64_t *__restrict__ dst_off,
 							 uint32_t n, uint32_t *__restrict__ flush)
@@ -244,6 +311,30 @@ int ofi_amd_bounce_scatter(const void *d_src, void *d_arena, uint64_t arena_byte
 	hipLaunchKernelGGL(bounce_scatter_kernel, dim3(blocks), dim3(kBlock), kLdsPerBlock, as_stream(stream),
 			   static_cast<const uint8_t *>(d_src), static_cast<uint8_t *>(d_arena),
 			   arena_bytes, d_src_off, d_dst_off, d_len, n, d_flush, err);
+	OFI_AMD_HIP_TRY(hipGetLastError());
+	return 0;
+}
+
+int ofi_amd_eager_copy_batch(const void *rx_base, const uint64_t *d_rx_off, const uint32_t *d_recv_len,
+			     void *dst_base, const uint64_t *d_dst_off, const uint32_t *d_dst_len,
+			     uint32_t n, uint32_t *d_copied, uint32_t *d_flush, void *stream)
+{
+	int rc = require_device();
+	if (rc != 0) {
+		return rc;
+	}
+	if (n == 0) {
+		return 0;
+	}
+	if (!rx_base || !d_rx_off || !d_recv_len || !d_dst_off || !d_dst_len || n > (1u << 30)) {
+		return -EINVAL;
+	}
+	uint32_t blocks = (n + kWavesPerBlock - 1) / kWavesPerBlock;
+	const uint32_t round = kXcds * kGroup;
+	blocks = (blocks + round - 1) / round * round;
+	hipLaunchKernelGGL(eager_copy_kernel, dim3(blocks), dim3(kBlock), 0, as_stream(stream),
+			   static_cast<const uint8_t *>(rx_base), d_rx_off, d_recv_len,
+			   static_cast<uint8_t *>(dst_base), d_dst_off, d_dst_len, n, d_copied, d_flush);
 	OFI_AMD_HIP_TRY(hipGetLastError());
 	return 0;
 }

@@ -134,6 +134,21 @@ int ofi_amd_bounce_scatter(const void *d_src, void *d_arena, uint64_t arena_byte
 			   const uint64_t *d_src_off, const uint64_t *d_dst_off,
 			   const uint32_t *d_len, uint32_t n, uint32_t *d_flush, void *stream);
 
+/*
+ * Eager arrivals as they sit in rx buffers: buffer i starts at rx_base + d_rx_off[i] with
+ * the 8-byte nccl_ofi_eager_msg_header_t (include/nccl_ofi_rdma.h:217-228) followed by
+ * d_recv_len[i] payload bytes.  Copies min(d_recv_len[i], d_dst_len[i]) payload bytes to
+ * dst_base + d_dst_off[i] -- any alignment; dst_base may be NULL with absolute addresses in
+ * d_dst_off -- as rdma_eager_copy_req::post does one fi_read at a time
+ * (src/nccl_ofi_rdma.cpp:2729-2776; truncation :2738-2743; zero length copies nothing,
+ * :753-762).  rx_base is any device-accessible memory (pinned host rx buffers or HBM).
+ * d_copied[i] (optional) receives the byte count; d_flush[i] (optional) the first
+ * min(4, count) destination bytes, little-endian, read back after the copy.
+ */
+int ofi_amd_eager_copy_batch(const void *rx_base, const uint64_t *d_rx_off, const uint32_t *d_recv_len,
+			     void *dst_base, const uint64_t *d_dst_off, const uint32_t *d_dst_len,
+			     uint32_t n, uint32_t *d_copied, uint32_t *d_flush, void *stream);
+
 /* Flush only: d_flush[i] = 4 bytes at d_arena + d_dst_off[i], read with
  * device-scope acquire semantics (the C5 read-back without a copy). */
 int ofi_amd_flush_read(const void *d_arena, const uint64_t *d_dst_off, uint32_t n,

@@ -34,6 +34,12 @@
  *                    protocol-ratio identities; exact fp32 bit pattern of the
  *                    reference binary: PARITY UNPINNED (not buildable here)
  *   bounce copy      memcpy semantics; patterns of tests/unit/gdrcopy.cpp:15-133
+ *   eager copy       memcpy semantics with truncation (a plain numpy slice copy)
+ *   rdma wire items  known answers of tests/unit/ctrl_msg.cpp (tag search, ready bit,
+ *                    full groups, sorted insert 1-7, chain decisions, wrap
+ *                    regression) and the static_asserts of include/nccl_ofi_rdma.h
+ *                    (8 / 64 / 512 / 560 bytes); sender numbering -> reordered
+ *                    delivery -> chain drain returns send order
  */
 #ifndef ORACLE_H_
 #define ORACLE_H_
@@ -292,6 +298,84 @@ void oracle_model_grid(int platform, int pipe_ops, int num_channels, int net_com
 void oracle_region_grid(int platform, const int32_t *colls, uint32_t n_colls, const uint64_t *sizes,
 			uint32_t n_sizes, const uint64_t *nodes, uint32_t n_nodes, const uint32_t *ppn,
 			uint32_t n_ppn, int32_t *choice);
+
+/* ------------------------------------------------- RDMA wire formats (oracle_wire.c) */
+
+/* nccl_ofi_eager_msg_header_t, include/nccl_ofi_rdma.h:217-228 */
+typedef struct {
+	uint8_t eager_offset;
+	uint8_t prev_batch_count;
+	uint16_t eager_seq;
+	int32_t tag;
+} oracle_eager_hdr_t;
+
+/* nccl_net_ofi_ctrl_msg_entry_t / nccl_net_ofi_ctrl_msg_t, :235-290 */
+typedef struct {
+	uint64_t buff_offset;
+	uint64_t mr_key[4];
+	uint32_t buff_len;
+	int16_t tag;
+	uint16_t flags;
+	uint16_t num_recvs;
+	uint8_t recv_idx;
+	uint8_t entry_used;
+	uint8_t pad[10];
+	uint16_t msg_seq_num;
+} oracle_ctrl_entry_t;
+
+typedef struct {
+	oracle_ctrl_entry_t entries[8];
+} oracle_ctrl_msg_t;
+
+/* the ordering fields of nccl_ofi_recv_eager_entry_t, :650-663 */
+typedef struct {
+	uint8_t eager_offset;
+	uint8_t prev_batch_count;
+	uint16_t eager_seq;
+	uint16_t msg_seq_num;
+	uint16_t pad;
+	int32_t tag;
+	uint32_t recv_len;
+	uint64_t cookie;
+} oracle_eager_entry_t;
+
+typedef struct {
+	uint16_t eager_seq_next;
+	uint16_t cur_eager_seq;
+	uint8_t eager_offset_next;
+	uint8_t prev_eager_batch_count;
+	uint16_t pad;
+} oracle_eager_tx_t;
+
+uint32_t oracle_rdma_imm(uint32_t comm_id, uint32_t seq, uint32_t recv_idx, uint32_t nseg);
+void oracle_rdma_imm_decode(uint32_t imm, uint32_t *comm_id, uint32_t *seq, uint32_t *recv_idx,
+			    uint32_t *nseg);
+uint32_t oracle_ctrl_mailbox_slot(uint16_t msg_seq_num);
+int oracle_ctrl_msg_fill(oracle_ctrl_msg_t *mailbox, uint16_t msg_seq_num, uint16_t num_recvs,
+			 const uint64_t *buff_offsets, const uint32_t *sizes, const int *tags,
+			 const uint64_t *mr_keys, uint32_t num_rails, int recv_completion_optional);
+int oracle_ctrl_msg_ready(const oracle_ctrl_msg_t *mailbox, uint16_t seq_num, int tag,
+			  int ignore_tag_match);
+int oracle_ctrl_msg_find_tag(const oracle_ctrl_msg_t *msg, int tag);
+int oracle_seq_before(uint16_t a, uint16_t b);
+int oracle_eager_seq_before(uint16_t a, uint16_t b);
+int oracle_eager_entry_less(const oracle_eager_entry_t *a, const oracle_eager_entry_t *b);
+int oracle_eager_entry_can_process(int has_processed, uint16_t last_eager_seq, uint8_t last_offset,
+				   const oracle_eager_entry_t *entry);
+typedef struct oracle_eager_rxq oracle_eager_rxq_t;
+oracle_eager_rxq_t *oracle_eager_rxq_create(void);
+void oracle_eager_rxq_destroy(oracle_eager_rxq_t *q);
+int oracle_eager_rxq_insert(oracle_eager_rxq_t *q, const oracle_eager_entry_t *e);
+uint32_t oracle_eager_rxq_drain(oracle_eager_rxq_t *q, oracle_eager_entry_t *out, uint32_t cap);
+uint32_t oracle_eager_rxq_pending(const oracle_eager_rxq_t *q);
+uint32_t oracle_eager_rxq_peek(const oracle_eager_rxq_t *q, oracle_eager_entry_t *out, uint32_t cap);
+void oracle_eager_tx_init(oracle_eager_tx_t *tx);
+void oracle_eager_tx_assign(oracle_eager_tx_t *tx, int32_t tag, oracle_eager_hdr_t *hdr);
+void oracle_eager_tx_advance(oracle_eager_tx_t *tx);
+int oracle_eager_fits(uint64_t size, int64_t eager_send_size);
+void oracle_eager_copy_batch(const uint8_t *rx_base, const uint64_t *rx_off, const uint32_t *recv_len,
+			     uint8_t *dst_base, const uint64_t *dst_off, const uint32_t *dst_len, uint32_t n,
+			     uint32_t *copied);
 
 #ifdef __cplusplus
 }

@@ -67,6 +67,34 @@ class GinAck(ctypes.Structure):
     _fields_ = [("peer", c_u32), ("rx_consumed", c_u32), ("msg", c_u64)]
 
 
+class EagerHdr(ctypes.Structure):
+    _fields_ = [("eager_offset", ctypes.c_uint8), ("prev_batch_count", ctypes.c_uint8),
+                ("eager_seq", ctypes.c_uint16), ("tag", c_i32)]
+
+
+class CtrlEntry(ctypes.Structure):
+    _fields_ = [("buff_offset", c_u64), ("mr_key", c_u64 * 4), ("buff_len", c_u32),
+                ("tag", ctypes.c_int16), ("flags", ctypes.c_uint16), ("num_recvs", ctypes.c_uint16),
+                ("recv_idx", ctypes.c_uint8), ("entry_used", ctypes.c_uint8),
+                ("pad", ctypes.c_uint8 * 10), ("msg_seq_num", ctypes.c_uint16)]
+
+
+class CtrlMsg(ctypes.Structure):
+    _fields_ = [("entries", CtrlEntry * 8)]
+
+
+class EagerEntry(ctypes.Structure):
+    _fields_ = [("eager_offset", ctypes.c_uint8), ("prev_batch_count", ctypes.c_uint8),
+                ("eager_seq", ctypes.c_uint16), ("msg_seq_num", ctypes.c_uint16),
+                ("pad", ctypes.c_uint16), ("tag", c_i32), ("recv_len", c_u32), ("cookie", c_u64)]
+
+
+class EagerTx(ctypes.Structure):
+    _fields_ = [("eager_seq_next", ctypes.c_uint16), ("cur_eager_seq", ctypes.c_uint16),
+                ("eager_offset_next", ctypes.c_uint8), ("prev_eager_batch_count", ctypes.c_uint8),
+                ("pad", ctypes.c_uint16)]
+
+
 class Point(ctypes.Structure):
     _fields_ = [("x", ctypes.c_double), ("y", ctypes.c_double)]
 
@@ -107,6 +135,30 @@ _ORACLE_PROTOS = {
     "oracle_gin_signal_apply": (c_int, [ctypes.POINTER(GinSignalWork), c_u32, ctypes.POINTER(c_u64),
                                         ctypes.POINTER(c_u64), ctypes.POINTER(c_vp), c_u32]),
     "oracle_gin_fold": (c_u64, [c_u64, c_vp, c_int]),
+    "oracle_rdma_imm": (c_u32, [c_u32, c_u32, c_u32, c_u32]),
+    "oracle_rdma_imm_decode": (None, [c_u32] + [ctypes.POINTER(c_u32)] * 4),
+    "oracle_ctrl_mailbox_slot": (c_u32, [ctypes.c_uint16]),
+    "oracle_ctrl_msg_fill": (c_int, [ctypes.POINTER(CtrlMsg), ctypes.c_uint16, ctypes.c_uint16,
+                                     ctypes.POINTER(c_u64), ctypes.POINTER(c_u32), ctypes.POINTER(c_int),
+                                     ctypes.POINTER(c_u64), c_u32, c_int]),
+    "oracle_ctrl_msg_ready": (c_int, [ctypes.POINTER(CtrlMsg), ctypes.c_uint16, c_int, c_int]),
+    "oracle_ctrl_msg_find_tag": (c_int, [ctypes.POINTER(CtrlMsg), c_int]),
+    "oracle_seq_before": (c_int, [ctypes.c_uint16, ctypes.c_uint16]),
+    "oracle_eager_seq_before": (c_int, [ctypes.c_uint16, ctypes.c_uint16]),
+    "oracle_eager_entry_less": (c_int, [ctypes.POINTER(EagerEntry), ctypes.POINTER(EagerEntry)]),
+    "oracle_eager_entry_can_process": (c_int, [c_int, ctypes.c_uint16, ctypes.c_uint8,
+                                               ctypes.POINTER(EagerEntry)]),
+    "oracle_eager_rxq_create": (c_vp, []),
+    "oracle_eager_rxq_destroy": (None, [c_vp]),
+    "oracle_eager_rxq_insert": (c_int, [c_vp, ctypes.POINTER(EagerEntry)]),
+    "oracle_eager_rxq_drain": (c_u32, [c_vp, ctypes.POINTER(EagerEntry), c_u32]),
+    "oracle_eager_rxq_pending": (c_u32, [c_vp]),
+    "oracle_eager_rxq_peek": (c_u32, [c_vp, ctypes.POINTER(EagerEntry), c_u32]),
+    "oracle_eager_tx_init": (None, [ctypes.POINTER(EagerTx)]),
+    "oracle_eager_tx_assign": (None, [ctypes.POINTER(EagerTx), c_i32, ctypes.POINTER(EagerHdr)]),
+    "oracle_eager_tx_advance": (None, [ctypes.POINTER(EagerTx)]),
+    "oracle_eager_fits": (c_int, [c_u64, ctypes.c_int64]),
+    "oracle_eager_copy_batch": (None, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_u32, c_vp]),
     "oracle_gin_stream_checksum": (c_u64, [c_u64, c_u32, c_u64, c_u32, c_u32, c_u32, c_u32, c_int,
                                            c_u32, c_u64, c_u64, c_u32, ctypes.POINTER(GinMr)]),
     "oracle_model_cost": (ctypes.c_float, [c_int, c_int, c_int, c_int, c_int, c_u64, c_u64, c_u64,

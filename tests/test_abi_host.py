@@ -14,13 +14,16 @@ import aws_ofi_nccl_amd as m
 from aws_ofi_nccl_amd import synthetic
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "ofi_amd_hotpath.h")
+HEADERS = [os.path.join(ROOT, "include", h) for h in ("ofi_amd_hotpath.h", "ofi_amd_wire.h")]
 
 
 def declared_symbols():
-    text = open(HEADER).read()
-    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(ofi_amd_\w+)\s*\(", text)))
+    names = set()
+    for header in HEADERS:
+        text = open(header).read()
+        text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+        names |= set(re.findall(r"\b(ofi_amd_\w+)\s*\(", text))
+    return sorted(names)
 
 
 def test_library_exports_every_declared_symbol(lib):
