@@ -291,8 +291,8 @@ def main():
 
     # HBM bytes per launch of bounce_scatter_kernel on this batch, from the rocprofv3 FETCH_SIZE /
     # WRITE_SIZE runs summarised in profiles/bounce_scatter_kernel_65536buf_2GiB_arena.md
-    # (273,047.6 KiB read + 269,222.9 KiB written after scaling by the plain-copy factors)
-    traffic = 555285000 if bounce["buffers"] == 65536 else None
+    # (273,371.4 KiB read + 266,846.6 KiB written after scaling by the plain-copy factors)
+    traffic = 553183000 if bounce["buffers"] == 65536 else None
     line = {
         "metric": "GIN puts/sec + bounce-copy GB/s on 1 MI355X (% of HBM/host-link peak)",
         "value": bounce["gbs_wall"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
