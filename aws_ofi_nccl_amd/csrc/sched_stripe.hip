@@ -10,13 +10,20 @@
  *   small_rail_i = (rr_small + #{j < i : size_j <  max_small}) mod R
  *   start_rail_i = (rr      + sum{j < i : size_j >= max_small} n_j) mod R
  *
- * Three launches on one stream:
- *   1. stripe_count_kernel  per-tile totals of (small count, stripe count)
- *   2. stripe_scan_kernel   one workgroup scans the tile totals, seeds them with
- *                           the counters in *state, writes the new counters back
+ * Launches on one stream:
+ *   1. stripe_count_kernel  per-tile totals of (small count, stripe count), each
+ *                           reduced mod R (only the residues matter); snapshots the
+ *                           two counters of *state as the batch's seed
+ *   2. stripe_scan_kernel   (batches of more than kInlineTiles tiles only) one
+ *                           workgroup scans the tile totals and writes the new
+ *                           counters back
  *   3. stripe_emit_kernel   re-reads the tile, scans inside the workgroup with
  *                           wavefront shuffles, builds the 96-byte stripe rows in
- *                           LDS and writes them out as coalesced 16-byte stores
+ *                           LDS and writes them out as coalesced 16-byte stores.
+ *                           Up to kInlineTiles tiles every workgroup sums the
+ *                           totals of the tiles before it by itself (at most 16 KiB
+ *                           from L2) instead of waiting for a scan launch, and the
+ *                           last workgroup writes the new counters back.
  *
  * HBM traffic per message: 8 B read twice + 4 B + 96 B written.
  */
@@ -34,6 +41,8 @@ constexpr uint32_t kPasses = 4;
 constexpr uint32_t kTile = kThreads * kPasses; /* messages per workgroup */
 constexpr uint32_t kScanThreads = 1024;
 constexpr uint64_t kMaxBatch = 1ull << 28;
+/* residues are < 4, so packed 16-bit sums over this many tiles cannot overflow */
+constexpr uint32_t kInlineTiles = 4096;
 
 struct params_t {
 	uint64_t max_small;
@@ -124,12 +133,19 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, uint32_t lan
 
 __global__ __launch_bounds__(kThreads) void stripe_count_kernel(
 	const uint64_t *__restrict__ sizes, uint32_t n, const ofi_amd_sched_state_t *__restrict__ state,
-	uint64_t align, uint32_t *__restrict__ tile_totals)
+	uint64_t align, uint32_t *__restrict__ tile_totals, uint32_t *__restrict__ seed0,
+	uint32_t *__restrict__ err)
 {
 	__shared__ uint32_t wave_sum[kThreads / 64];
 	params_t p;
 	if (!load_params(state, align, p)) {
+		if (blockIdx.x == 0 && threadIdx.x == 0) {
+			atomicOr(err, ofi_amd::ASYNC_ERR_SCHED_STATE);
+		}
 		return;
+	}
+	if (blockIdx.x == 0 && threadIdx.x == 0) {
+		*seed0 = ((state->rr_small_counter % p.num_rails) << 16) | (state->rr_counter % p.num_rails);
 	}
 	const uint32_t base = blockIdx.x * kTile;
 	uint32_t acc = 0;
@@ -150,7 +166,8 @@ __global__ __launch_bounds__(kThreads) void stripe_count_kernel(
 	}
 	__syncthreads();
 	if (threadIdx.x == 0) {
-		tile_totals[blockIdx.x] = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
+		const uint32_t t = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
+		tile_totals[blockIdx.x] = (((t >> 16) % p.num_rails) << 16) | ((t & 0xffffu) % p.num_rails);
 	}
 }
 
@@ -212,10 +229,13 @@ __global__ __launch_bounds__(kScanThreads) void stripe_scan_kernel(
 	}
 }
 
+/* INLINE: tile_prefix holds the per-tile totals (residues) and *seed0 the batch's seed;
+ * otherwise tile_prefix holds each tile's finished seed. */
+template <bool INLINE>
 __global__ __launch_bounds__(kThreads) void stripe_emit_kernel(
-	const uint64_t *__restrict__ sizes, uint32_t n, const ofi_amd_sched_state_t *__restrict__ state,
-	uint64_t align, const uint32_t *__restrict__ tile_prefix, uint32_t *__restrict__ num_xfers,
-	u32x4 *__restrict__ xfers)
+	const uint64_t *__restrict__ sizes, uint32_t n, ofi_amd_sched_state_t *__restrict__ state,
+	uint64_t align, const uint32_t *__restrict__ tile_prefix, const uint32_t *__restrict__ seed0,
+	uint32_t *__restrict__ num_xfers, u32x4 *__restrict__ xfers)
 {
 	params_t p;
 	if (!load_params(state, align, p)) {
@@ -228,7 +248,27 @@ __global__ __launch_bounds__(kThreads) void stripe_emit_kernel(
 	const uint32_t base = blockIdx.x * kTile;
 	const uint32_t R = p.num_rails;
 
-	uint32_t seed = tile_prefix[blockIdx.x];
+	uint32_t seed;
+	if (INLINE) {
+		/* sum of the totals of the tiles before this one (packed halves, no overflow) */
+		uint32_t acc = 0;
+		for (uint32_t t = threadIdx.x; t < blockIdx.x; t += kThreads) {
+			acc += tile_prefix[t];
+		}
+#pragma unroll
+		for (uint32_t d = 32; d > 0; d >>= 1) {
+			acc += __shfl_xor(acc, d, 64);
+		}
+		if (lane == 0) {
+			wave_sum[wave] = acc;
+		}
+		__syncthreads();
+		acc = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3] + *seed0;
+		__syncthreads();
+		seed = (((acc >> 16) % R) << 16) | ((acc & 0xffffu) % R);
+	} else {
+		seed = tile_prefix[blockIdx.x];
+	}
 	uint32_t carry_small = seed >> 16, carry_big = seed & 0xffffu; /* both < R */
 
 	for (uint32_t pass = 0; pass < kPasses; pass++) {
@@ -309,13 +349,19 @@ __global__ __launch_bounds__(kThreads) void stripe_emit_kernel(
 		carry_big = (carry_big + (tot & 0xffffu)) % R;
 		__syncthreads();
 	}
+	if (INLINE && blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
+		/* the carries after the last tile are the counters the next batch starts from;
+		 * nobody reads them any more in this launch (the seed was snapshotted) */
+		state->rr_small_counter = carry_small;
+		state->rr_counter = carry_big;
+	}
 }
 
 /* Per-process scratch for tile totals / prefixes, grown on demand. */
 struct workspace_t {
 	std::mutex lock;
 	uint32_t *totals = nullptr;
-	uint32_t *prefix = nullptr;
+	uint32_t *prefix = nullptr; /* prefix[capacity] is the seed word */
 	uint32_t tiles = 0;
 };
 workspace_t g_ws;
@@ -350,14 +396,14 @@ int ofi_amd_sched_batch(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes,
 	}
 
 	const uint32_t tiles = (uint32_t)((n + kTile - 1) / kTile);
-	uint32_t *totals, *prefix;
+	uint32_t *totals, *prefix, *seed0;
 	{
 		std::lock_guard<std::mutex> g(g_ws.lock);
 		if (tiles > g_ws.tiles) {
 			uint32_t want = tiles < 4096 ? 4096 : tiles;
 			uint32_t *a = nullptr, *b = nullptr;
 			OFI_AMD_HIP_TRY(hipMalloc((void **)&a, sizeof(uint32_t) * want));
-			if (hipMalloc((void **)&b, sizeof(uint32_t) * want) != hipSuccess) {
+			if (hipMalloc((void **)&b, sizeof(uint32_t) * (want + 1)) != hipSuccess) {
 				(void)hipFree(a);
 				return -ENOMEM;
 			}
@@ -371,16 +417,23 @@ int ofi_amd_sched_batch(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes,
 		}
 		totals = g_ws.totals;
 		prefix = g_ws.prefix;
+		seed0 = g_ws.prefix + g_ws.tiles;
 	}
 
 	hipStream_t s = as_stream(stream);
 	hipLaunchKernelGGL(stripe_count_kernel, dim3(tiles), dim3(kThreads), 0, s, d_sizes,
-			   (uint32_t)n, d_state, align, totals);
-	hipLaunchKernelGGL(stripe_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, totals, tiles,
-			   d_state, prefix, err);
-	hipLaunchKernelGGL(stripe_emit_kernel, dim3(tiles), dim3(kThreads), 0, s, d_sizes,
-			   (uint32_t)n, d_state, align, prefix, d_num_xfers,
-			   reinterpret_cast<u32x4 *>(d_xfers));
+			   (uint32_t)n, d_state, align, totals, seed0, err);
+	if (tiles <= kInlineTiles) {
+		hipLaunchKernelGGL(stripe_emit_kernel<true>, dim3(tiles), dim3(kThreads), 0, s, d_sizes,
+				   (uint32_t)n, d_state, align, totals, seed0, d_num_xfers,
+				   reinterpret_cast<u32x4 *>(d_xfers));
+	} else {
+		hipLaunchKernelGGL(stripe_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, totals, tiles,
+				   d_state, prefix, err);
+		hipLaunchKernelGGL(stripe_emit_kernel<false>, dim3(tiles), dim3(kThreads), 0, s, d_sizes,
+				   (uint32_t)n, d_state, align, prefix, seed0, d_num_xfers,
+				   reinterpret_cast<u32x4 *>(d_xfers));
+	}
 	OFI_AMD_HIP_TRY(hipGetLastError());
 	return 0;
 }

@@ -112,6 +112,22 @@ def test_bad_arguments(lib, gpu):
         assert _gpu.fetch_async_errors(lib) & 4
 
 
+@pytest.mark.parametrize("rails,seeds", [(4, (3, 2)), (3, (1, 2))])
+def test_batches_beyond_the_inline_prefix_limit(lib, oracle, gpu, rails, seeds):
+    """More than 4096 tiles of 1024 messages: the tile seeds come from the separate scan launch;
+    one tile below and one above the limit must chain exactly like the small form."""
+    for n in (4096 * 1024, 4096 * 1024 + 1, 5_000_011):
+        sizes = synthetic.stripe_sizes(n + rails, n)
+        want_num, want_xf, ost = _oracle.sched_batch(oracle, sizes, rails, 131072, 64, seeds)
+        d_state = dev_state(rails, 131072, 64, seeds)
+        rc, num, xf = gpu_batch(lib, d_state, sizes)
+        assert rc == 0
+        assert np.array_equal(num, want_num)
+        assert np.array_equal(xf, want_xf)
+        st = read_state(d_state)
+        assert (st.rr_small_counter, st.rr_counter) == (ost.rr_small_counter, ost.rr_counter)
+
+
 def test_full_size_configuration(lib, oracle, gpu):
     """1,000,000 messages log-uniform in [1 B, 256 MiB), 4 rails, default thresholds, seeded start rails."""
     sizes = synthetic.stripe_sizes(2024, 1_000_000)
