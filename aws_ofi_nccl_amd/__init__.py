@@ -237,6 +237,8 @@ PROTOTYPES = {
     "ofi_amd_gin_ack_msg": (c_u64, [c_u32, c_u32]),
     "ofi_amd_gin_proxy_drain": (ctypes.c_int, [c_vp, c_u64, ctypes.c_int, c_vp, c_vp, c_vp, c_vp,
                                                c_u32, ctypes.POINTER(GinProxyStats)]),
+    "ofi_amd_gin_proxy_drain_mt": (ctypes.c_int, [c_vp, c_u64, ctypes.c_int, c_vp, c_vp, c_vp, c_vp,
+                                                  c_u32, c_u32, ctypes.POINTER(GinProxyStats)]),
     "ofi_amd_gin_rx_create": (ctypes.c_int, [c_u32, ctypes.POINTER(c_u32), ctypes.POINTER(c_vp)]),
     "ofi_amd_gin_rx_destroy": (ctypes.c_int, [c_vp]),
     "ofi_amd_gin_rx_write_completion": (ctypes.c_int, [c_vp, c_u32, c_u32]),

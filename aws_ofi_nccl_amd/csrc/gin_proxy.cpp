@@ -10,6 +10,8 @@
  */
 #include <cerrno>
 #include <chrono>
+#include <thread>
+#include <vector>
 #include <cstring>
 
 #include "gin_rings.hpp"
@@ -274,16 +276,15 @@ int ofi_amd_gin_ring_pop(ofi_amd_gin_rings_t *r, uint32_t context, ofi_amd_gin_d
 	return 1;
 }
 
-int ofi_amd_gin_proxy_drain(ofi_amd_gin_rings_t *r, uint64_t ops_per_context, int mode,
-			    ofi_amd_gin_desc_t *out_desc, ofi_amd_gin_comm_t *comms,
-			    const ofi_amd_gin_mr_t *mrs, ofi_amd_gin_wire_t *out_wire,
-			    uint32_t timeout_ms, ofi_amd_gin_proxy_stats_t *stats)
+/* One proxy thread's share: contexts [c_begin, c_end). */
+static int drain_contexts(ofi_amd_gin_rings_t *r, uint32_t c_begin, uint32_t c_end,
+			  uint64_t ops_per_context, int mode, ofi_amd_gin_desc_t *out_desc,
+			  ofi_amd_gin_comm_t *comms, const ofi_amd_gin_mr_t *mrs,
+			  ofi_amd_gin_wire_t *out_wire, uint32_t timeout_ms,
+			  ofi_amd_gin_proxy_stats_t *stats)
 {
-	if (!r || mode < 0 || mode > 2 || (mode == 1 && !out_desc) || (mode == 2 && (!comms || !mrs))) {
-		return -EINVAL;
-	}
 	using clock = std::chrono::steady_clock;
-	const uint32_t nctx = r->n_contexts, cap = r->capacity, mask = cap - 1;
+	const uint32_t nctx = c_end - c_begin, cap = r->capacity, mask = cap - 1;
 	const uint32_t burst = cap / 2 < 1024 ? cap / 2 : 1024;
 
 	uint64_t *done = new (std::nothrow) uint64_t[nctx]();
@@ -293,8 +294,8 @@ int ofi_amd_gin_proxy_drain(ofi_amd_gin_rings_t *r, uint64_t ops_per_context, in
 		delete[] hash;
 		return -ENOMEM;
 	}
-	for (uint32_t c = 0; c < nctx; c++) {
-		hash[c] = 0x9E3779B97F4A7C15ull ^ c;
+	for (uint32_t k = 0; k < nctx; k++) {
+		hash[k] = 0x9E3779B97F4A7C15ull ^ (c_begin + k);
 	}
 
 	ofi_amd_gin_proxy_stats_t st;
@@ -307,22 +308,23 @@ int ofi_amd_gin_proxy_drain(ofi_amd_gin_rings_t *r, uint64_t ops_per_context, in
 
 	while (remaining > 0) {
 		bool progressed = false;
-		for (uint32_t c = 0; c < nctx; c++) {
-			if (done[c] >= ops_per_context) {
+		for (uint32_t k = 0; k < nctx; k++) {
+			if (done[k] >= ops_per_context) {
 				continue;
 			}
+			const uint32_t c = c_begin + k;
 			uint32_t *seq = r->sequences + (size_t)c * cap;
 			const ofi_amd_gin_desc_t *rec = r->records + (size_t)c * cap;
 			const uint32_t start = r->dequeue_pos[c];
 			uint32_t pos = start;
-			uint64_t want = ops_per_context - done[c];
+			uint64_t want = ops_per_context - done[k];
 			uint32_t limit = want < burst ? (uint32_t)want : burst;
-			uint64_t h = hash[c];
+			uint64_t h = hash[k];
 
 			while (pos - start < limit &&
 			       __atomic_load_n(&seq[pos & mask], __ATOMIC_ACQUIRE) == pos + 1) {
 				const ofi_amd_gin_desc_t *d = &rec[pos & mask];
-				const uint64_t i = done[c] + (pos - start);
+				const uint64_t i = done[k] + (pos - start);
 				h = fold_words(h, reinterpret_cast<const uint64_t *>(d), 8);
 				st.signals += d->signal_op != 0;
 				if (mode == 1) {
@@ -350,10 +352,10 @@ int ofi_amd_gin_proxy_drain(ofi_amd_gin_rings_t *r, uint64_t ops_per_context, in
 					__atomic_store_n(&seq[p & mask], p + cap, __ATOMIC_RELEASE);
 				}
 				r->dequeue_pos[c] = pos;
-				done[c] += pos - start;
+				done[k] += pos - start;
 				remaining -= pos - start;
 				st.descriptors += pos - start;
-				hash[c] = h;
+				hash[k] = h;
 				progressed = true;
 			} else {
 				st.empty_polls++;
@@ -379,15 +381,75 @@ int ofi_amd_gin_proxy_drain(ofi_amd_gin_rings_t *r, uint64_t ops_per_context, in
 		}
 	}
 	st.seconds = std::chrono::duration<double>(clock::now() - t0).count();
-	for (uint32_t c = 0; c < nctx; c++) {
-		st.checksum += hash[c];
+	for (uint32_t k = 0; k < nctx; k++) {
+		st.checksum += hash[k];
 	}
-	if (stats) {
-		*stats = st;
-	}
+	*stats = st;
 	delete[] done;
 	delete[] hash;
 	return rc;
+}
+
+int ofi_amd_gin_proxy_drain_mt(ofi_amd_gin_rings_t *r, uint64_t ops_per_context, int mode,
+			       ofi_amd_gin_desc_t *out_desc, ofi_amd_gin_comm_t *comms,
+			       const ofi_amd_gin_mr_t *mrs, ofi_amd_gin_wire_t *out_wire,
+			       uint32_t timeout_ms, uint32_t n_threads, ofi_amd_gin_proxy_stats_t *stats)
+{
+	if (!r || mode < 0 || mode > 2 || (mode == 1 && !out_desc) || (mode == 2 && (!comms || !mrs)) ||
+	    n_threads < 1 || n_threads > 64) {
+		return -EINVAL;
+	}
+	const uint32_t nctx = r->n_contexts;
+	const uint32_t workers = n_threads < nctx ? n_threads : nctx;
+	std::vector<ofi_amd_gin_proxy_stats_t> part(workers);
+	std::vector<int> rcs(workers, 0);
+	const auto t0 = std::chrono::steady_clock::now();
+	auto share = [&](uint32_t w) {
+		/* contiguous ranges of contexts, sizes differing by at most one */
+		const uint32_t lo = (uint32_t)((uint64_t)nctx * w / workers);
+		const uint32_t hi = (uint32_t)((uint64_t)nctx * (w + 1) / workers);
+		rcs[w] = drain_contexts(r, lo, hi, ops_per_context, mode, out_desc, comms, mrs, out_wire,
+					timeout_ms, &part[w]);
+	};
+	try {
+		std::vector<std::thread> threads;
+		for (uint32_t w = 1; w < workers; w++) {
+			threads.emplace_back(share, w);
+		}
+		share(0); /* the calling thread is a proxy thread too */
+		for (auto &t : threads) {
+			t.join();
+		}
+	} catch (...) {
+		return -ENOMEM;
+	}
+	ofi_amd_gin_proxy_stats_t st;
+	std::memset(&st, 0, sizeof(st));
+	int rc = 0;
+	for (uint32_t w = 0; w < workers; w++) {
+		st.descriptors += part[w].descriptors;
+		st.signals += part[w].signals;
+		st.writes += part[w].writes;
+		st.checksum += part[w].checksum;
+		st.empty_polls += part[w].empty_polls;
+		if (rcs[w] != 0 && rc == 0) {
+			rc = rcs[w];
+		}
+	}
+	st.seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+	if (stats) {
+		*stats = st;
+	}
+	return rc;
+}
+
+int ofi_amd_gin_proxy_drain(ofi_amd_gin_rings_t *r, uint64_t ops_per_context, int mode,
+			    ofi_amd_gin_desc_t *out_desc, ofi_amd_gin_comm_t *comms,
+			    const ofi_amd_gin_mr_t *mrs, ofi_amd_gin_wire_t *out_wire,
+			    uint32_t timeout_ms, ofi_amd_gin_proxy_stats_t *stats)
+{
+	return ofi_amd_gin_proxy_drain_mt(r, ops_per_context, mode, out_desc, comms, mrs, out_wire,
+					  timeout_ms, 1, stats);
 }
 
 } /* extern "C" */

@@ -211,7 +211,9 @@ def bench_gin(lib, oracle, torch, np, args):
     import aws_ofi_nccl_amd as m
     nctx, cap, ops = 256, 4096, args.gin_ops
     out = {"contexts": nctx, "ring_capacity": cap, "ops_per_context": ops}
-    for mode, key in ((0, "drain"), (2, "drain_and_derive_wire")):
+    # NCCL runs up to NCCL_GIN_MAX_CONNECTIONS = 4 GIN proxy threads (nccl/net.h:38)
+    for mode, threads, key in ((0, 1, "drain"), (2, 1, "drain_and_derive_wire"),
+                               (2, 4, "drain_and_derive_wire_4_proxy_threads")):
         rings = ctypes.c_void_p()
         m.check(lib.ofi_amd_gin_rings_create(nctx, cap, ctypes.byref(rings)), "rings_create")
         comms = (m.GinComm * nctx)()
@@ -221,8 +223,9 @@ def bench_gin(lib, oracle, torch, np, args):
         stats = m.GinProxyStats()
         t0 = time.perf_counter()
         m.check(lib.ofi_amd_gin_produce_seeded(rings, SEED, ops, 1, 64, 1, 1, 0, _gpu.stream()), "produce")
-        rc = lib.ofi_amd_gin_proxy_drain(rings, ops, mode, None, ctypes.cast(comms, ctypes.c_void_p),
-                                         ctypes.cast(mrs, ctypes.c_void_p), None, 20000, ctypes.byref(stats))
+        rc = lib.ofi_amd_gin_proxy_drain_mt(rings, ops, mode, None, ctypes.cast(comms, ctypes.c_void_p),
+                                            ctypes.cast(mrs, ctypes.c_void_p), None, 20000, threads,
+                                            ctypes.byref(stats))
         torch.cuda.synchronize()
         secs = time.perf_counter() - t0
         if rc != 0 or lib.ofi_amd_gin_producer_status(rings) != 0:
@@ -230,7 +233,7 @@ def bench_gin(lib, oracle, torch, np, args):
         out[key] = {"descriptors": stats.descriptors, "seconds": secs,
                     "descs_per_s": stats.descriptors / secs,
                     "host_link_gbs": stats.descriptors * 68 / secs / 1e9,
-                    "consumer_ns_per_desc": secs / stats.descriptors * 1e9,
+                    "consumer_ns_per_desc": secs / stats.descriptors * 1e9, "proxy_threads": threads,
                     "checksum": "%016x" % stats.checksum, "rdma_writes": stats.writes}
         lib.ofi_amd_gin_rings_destroy(rings)
     if not args.skip_cpu:
@@ -249,6 +252,8 @@ def bench_gin(lib, oracle, torch, np, args):
         out["cpu_sample"] = "%d ops per context" % sample
         if sample == ops:
             out["parity_ok"] = out["drain"]["checksum"] == "%016x" % ck
+    out["derive_checksums_agree_across_thread_counts"] = (
+        out["drain_and_derive_wire"]["checksum"] == out["drain_and_derive_wire_4_proxy_threads"]["checksum"])
     return out
 
 

@@ -310,6 +310,17 @@ int ofi_amd_gin_proxy_drain(ofi_amd_gin_rings_t *rings, uint64_t ops_per_context
 			    const ofi_amd_gin_mr_t *mrs, ofi_amd_gin_wire_t *out_wire,
 			    uint32_t timeout_ms, ofi_amd_gin_proxy_stats_t *stats);
 
+/*
+ * The same loop on n_threads proxy threads (the caller's included), each owning a contiguous
+ * range of contexts -- NCCL runs up to NCCL_GIN_MAX_CONNECTIONS = 4 GIN proxy threads
+ * (nccl/net.h:38).  Contexts are independent (own ring, own comm state), so the per-context
+ * results, and the checksum summed over contexts, do not depend on n_threads.  1..64.
+ */
+int ofi_amd_gin_proxy_drain_mt(ofi_amd_gin_rings_t *rings, uint64_t ops_per_context, int mode,
+			       ofi_amd_gin_desc_t *out_desc, ofi_amd_gin_comm_t *comms,
+			       const ofi_amd_gin_mr_t *mrs, ofi_amd_gin_wire_t *out_wire,
+			       uint32_t timeout_ms, uint32_t n_threads, ofi_amd_gin_proxy_stats_t *stats);
+
 /* ---- receiver side: completions -> in-order retire -> signal counters in HBM ---- */
 
 /* One folded signal delivery: add `value` to the 8-byte counter at base + offset

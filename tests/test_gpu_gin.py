@@ -122,6 +122,37 @@ def test_wire_records_bit_exact(lib, oracle, gpu, signal_every, signal_op, agg_m
     lib.ofi_amd_gin_rings_destroy(rings)
 
 
+def test_proxy_thread_count_does_not_change_the_result(lib, oracle, gpu):
+    """Several proxy threads, each owning a range of contexts: wire records, per-context comm
+    state and the checksum equal the single-thread run (and so the oracle's)."""
+    nctx, cap, ops = 13, 512, 6000
+    omrs, pmrs = _oracle.default_mrs(), _oracle.default_mrs(m.GinMr)
+    want_ck = oracle.oracle_gin_stream_checksum(SEED, nctx, ops, 1, 5, 2, 1, 1, 4, 131072, 64, 1, omrs)
+    results = []
+    for threads in (1, 3, 4, 32):
+        rings = make_rings(lib, nctx, cap)
+        comms = (m.GinComm * nctx)()
+        for c in range(nctx):
+            assert lib.ofi_amd_gin_comm_init(ctypes.byref(comms[c]), c, 4, 131072, 64, 1) == 0
+        wires = (m.GinWire * (nctx * ops))()
+        stats = m.GinProxyStats()
+        assert lib.ofi_amd_gin_produce_seeded(rings, SEED, ops, 1, 5, 2, 1, 0, _gpu.stream()) == 0
+        rc = lib.ofi_amd_gin_proxy_drain_mt(rings, ops, 2, None, ctypes.cast(comms, ctypes.c_void_p),
+                                            ctypes.cast(pmrs, ctypes.c_void_p),
+                                            ctypes.cast(wires, ctypes.c_void_p), 10000, threads,
+                                            ctypes.byref(stats))
+        _gpu.sync()
+        assert rc == 0 and lib.ofi_amd_gin_producer_status(rings) == 0
+        assert stats.descriptors == nctx * ops and stats.checksum == want_ck
+        results.append((bytes(wires), bytes(comms), stats.writes, stats.signals))
+        lib.ofi_amd_gin_rings_destroy(rings)
+    assert all(r == results[0] for r in results[1:])
+    rings = make_rings(lib, 2, 256)
+    assert lib.ofi_amd_gin_proxy_drain_mt(rings, 0, 0, None, None, None, None, 10, 0, None) == -22
+    assert lib.ofi_amd_gin_proxy_drain_mt(rings, 0, 0, None, None, None, None, 10, 65, None) == -22
+    lib.ofi_amd_gin_rings_destroy(rings)
+
+
 def test_configured_shape_checksum(lib, oracle, gpu):
     """256 contexts, 4096-entry rings, put-signal every 64th op; 20,000 ops per context here
     (the benchmark runs the full 1,000,000).  Checked through the order-sensitive checksum."""
