@@ -35,6 +35,11 @@ def ref():
 @pytest.fixture(scope="session")
 def lib():
     """The product C-ABI library.  Missing library = failure, never a fallback."""
+    # The tests use torch for device buffers, and this torch wheel bundles its own HIP/HSA
+    # runtime.  A process can drive the GPU through one runtime only: whichever of two is
+    # initialised second sees no device.  Loading torch first makes the library bind to the
+    # runtime already in the process (same soname) instead of bringing /opt/rocm's.
+    import torch  # noqa: F401
     import aws_ofi_nccl_amd as m
     if not os.path.exists(m.LIB_PATH):
         from aws_ofi_nccl_amd import build
