@@ -211,6 +211,9 @@ PROTOTYPES = {
                                               c_vp]),
     "ofi_amd_eager_copy_batch": (ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_u32, c_vp, c_vp,
                                                 c_vp]),
+    "ofi_amd_flush_buffer_fill": (ctypes.c_int, [c_vp, c_u64, c_vp]),
+    "ofi_amd_flush_post": (ctypes.c_int, [c_vp, c_vp, c_u32, c_vp]),
+    "ofi_amd_flush_test": (ctypes.c_int, [c_vp, c_u32, c_u64]),
     "ofi_amd_flush_read": (ctypes.c_int, [c_vp, c_vp, c_u32, c_vp, c_vp]),
     "ofi_amd_devcopy_register": (ctypes.c_int, [c_vp, ctypes.c_size_t, ctypes.POINTER(c_vp)]),
     "ofi_amd_devcopy_to_device": (ctypes.c_int, [c_vp, c_vp, ctypes.c_size_t, ctypes.c_size_t]),

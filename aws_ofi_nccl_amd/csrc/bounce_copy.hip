@@ -276,6 +276,32 @@ __global__ __launch_bounds__(256) void flush_read_kernel(const uint8_t *__restri
 	}
 }
 
+__global__ __launch_bounds__(64) void flush_fill_kernel(uint64_t *__restrict__ flush_buf, uint64_t sentinel)
+{
+	if (threadIdx.x < 8) {
+		flush_buf[threadIdx.x] = sentinel;
+	}
+}
+
+/* One lane per 8-byte word: 8 words per rail slot.  The flag (word 0 of a slot) is what the
+ * host polls, so it goes last, behind a system-scope release fence. */
+__global__ __launch_bounds__(64) void flush_post_kernel(const uint64_t *__restrict__ flush_buf,
+							uint64_t *__restrict__ slots, uint32_t num_rails)
+{
+	const uint32_t rail = threadIdx.x >> 3, word = threadIdx.x & 7u;
+	if (rail >= num_rails) {
+		return;
+	}
+	const uint64_t v = __hip_atomic_load(&flush_buf[word], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM);
+	if (word != 0) {
+		__hip_atomic_store(&slots[rail * 8u + word], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+	}
+	__builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+	if (word == 0) {
+		__hip_atomic_store(&slots[rail * 8u], v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+	}
+}
+
 } // namespace
 
 struct ofi_amd_devcopy_region {
@@ -357,6 +383,53 @@ int ofi_amd_flush_read(const void *d_arena, const uint64_t *d_dst_off, uint32_t 
 			   d_flush);
 	OFI_AMD_HIP_TRY(hipGetLastError());
 	return 0;
+}
+
+int ofi_amd_flush_buffer_fill(void *d_flush_buf, uint64_t sentinel, void *stream)
+{
+	int rc = require_device();
+	if (rc != 0) {
+		return rc;
+	}
+	if (!d_flush_buf || (reinterpret_cast<uintptr_t>(d_flush_buf) & 7u)) {
+		return -EINVAL;
+	}
+	hipLaunchKernelGGL(flush_fill_kernel, dim3(1), dim3(64), 0, as_stream(stream),
+			   static_cast<uint64_t *>(d_flush_buf), sentinel);
+	OFI_AMD_HIP_TRY(hipGetLastError());
+	return 0;
+}
+
+int ofi_amd_flush_post(const void *d_flush_buf, void *slots_dev, uint32_t num_rails, void *stream)
+{
+	int rc = require_device();
+	if (rc != 0) {
+		return rc;
+	}
+	if (!d_flush_buf || !slots_dev || num_rails < 1 || num_rails > OFI_AMD_MAX_NUM_RAILS ||
+	    (reinterpret_cast<uintptr_t>(d_flush_buf) & 7u) || (reinterpret_cast<uintptr_t>(slots_dev) & 7u)) {
+		return -EINVAL;
+	}
+	hipLaunchKernelGGL(flush_post_kernel, dim3(1), dim3(64), 0, as_stream(stream),
+			   static_cast<const uint64_t *>(d_flush_buf), static_cast<uint64_t *>(slots_dev),
+			   num_rails);
+	OFI_AMD_HIP_TRY(hipGetLastError());
+	return 0;
+}
+
+/* has_flush_completed, src/nccl_ofi_rdma.cpp:2110-2126: only the first 8 bytes of a slot count */
+int ofi_amd_flush_test(const void *slots_host, uint32_t num_rails, uint64_t sentinel)
+{
+	if (!slots_host || num_rails < 1 || num_rails > OFI_AMD_MAX_NUM_RAILS) {
+		return -EINVAL;
+	}
+	const uint64_t *slots = static_cast<const uint64_t *>(slots_host);
+	for (uint32_t r = 0; r < num_rails; r++) {
+		if (__atomic_load_n(&slots[r * 8u], __ATOMIC_ACQUIRE) != sentinel) {
+			return 0;
+		}
+	}
+	return 1;
 }
 
 /* ---- nccl_ofi_device_copy (include/nccl_ofi_device_copy.h:14-69) ---- */

@@ -154,6 +154,25 @@ int ofi_amd_eager_copy_batch(const void *rx_base, const uint64_t *d_rx_off, cons
 int ofi_amd_flush_read(const void *d_arena, const uint64_t *d_dst_off, uint32_t n,
 		       uint32_t *d_flush, void *stream);
 
+/*
+ * The reference's sentinel flush, kept slot for slot.  A 64-byte flush buffer in GPU memory
+ * holds eight copies of a sentinel (0x00000000ffffffff for the RDMA transport,
+ * include/nccl_ofi_rdma.h:45 and src/nccl_ofi_rdma.cpp:7390-7394; 0xdeadbeefdeadbeef for GIN,
+ * include/rdma/gin/nccl_ofi_gin_reqs.h:274); a flush reads it back into one 64-byte host
+ * slot per rail (nccl_net_ofi_flush_data_t, include/nccl_ofi_rdma.h:326-332) and is complete
+ * when the first 8 bytes of every slot equal the sentinel (has_flush_completed,
+ * src/nccl_ofi_rdma.cpp:2110-2126; nccl_ofi_gin_iflush_req::test,
+ * src/rdma/gin/nccl_ofi_gin_reqs.cpp:373-394).  Here the read-back is one small kernel on
+ * `stream` instead of one loop-back fi_read per rail (rdma_flush_req::post, :2664-2713).
+ *   fill: writes the sentinels into d_flush_buf (64 bytes, device memory);
+ *   post: copies d_flush_buf into slots_dev[0..num_rails) -- the device address of pinned
+ *         host memory -- with system-scope ordering; the caller zeroes the slots first;
+ *   test: host side, 1 when every slot shows the sentinel, else 0.
+ */
+int ofi_amd_flush_buffer_fill(void *d_flush_buf, uint64_t sentinel, void *stream);
+int ofi_amd_flush_post(const void *d_flush_buf, void *slots_dev, uint32_t num_rails, void *stream);
+int ofi_amd_flush_test(const void *slots_host, uint32_t num_rails, uint64_t sentinel);
+
 /* nccl_ofi_device_copy, include/nccl_ofi_device_copy.h:14-69: register a device
  * region, then small synchronous host<->device copies at an offset. */
 typedef struct ofi_amd_devcopy_region ofi_amd_devcopy_region_t;

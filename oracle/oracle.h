@@ -373,6 +373,8 @@ void oracle_eager_tx_init(oracle_eager_tx_t *tx);
 void oracle_eager_tx_assign(oracle_eager_tx_t *tx, int32_t tag, oracle_eager_hdr_t *hdr);
 void oracle_eager_tx_advance(oracle_eager_tx_t *tx);
 int oracle_eager_fits(uint64_t size, int64_t eager_send_size);
+void oracle_flush_post(const uint64_t flush_buf[8], uint64_t *slots, uint32_t num_rails);
+int oracle_flush_completed(const uint64_t *slots, uint32_t num_rails, uint64_t sentinel);
 void oracle_eager_copy_batch(const uint8_t *rx_base, const uint64_t *rx_off, const uint32_t *recv_len,
 			     uint8_t *dst_base, const uint64_t *dst_off, const uint32_t *dst_len, uint32_t n,
 			     uint32_t *copied);

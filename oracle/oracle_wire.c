@@ -280,6 +280,28 @@ int oracle_eager_fits(uint64_t size, int64_t eager_send_size)
 	return (int64_t)(size + 8) <= eager_send_size;
 }
 
+/* The sentinel flush.  The GPU flush buffer is one cache line of sentinels
+ * (src/nccl_ofi_rdma.cpp:7390-7394); a flush reads it into the 64-byte host slot of every
+ * rail (rdma_flush_req::post, :2664-2713; slot = rail * 64, :2103-2106). */
+void oracle_flush_post(const uint64_t flush_buf[8], uint64_t *slots, uint32_t num_rails)
+{
+	for (uint32_t r = 0; r < num_rails; r++) {
+		memcpy(&slots[r * 8], flush_buf, 64);
+	}
+}
+
+/* has_flush_completed, :2110-2126, and nccl_ofi_gin_iflush_req::test,
+ * src/rdma/gin/nccl_ofi_gin_reqs.cpp:373-394: the first 8 bytes of every slot */
+int oracle_flush_completed(const uint64_t *slots, uint32_t num_rails, uint64_t sentinel)
+{
+	for (uint32_t r = 0; r < num_rails; r++) {
+		if (slots[r * 8] != sentinel) {
+			return 0;
+		}
+	}
+	return 1;
+}
+
 /* rdma_eager_copy_req::post, :2729-2776, for a batch: payload (after the 8-byte header)
  * of rx buffer i goes to dst[i], truncated to the destination's length; zero-length
  * arrivals copy nothing (:753-762).  copied[i] receives the byte count. */

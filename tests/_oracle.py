@@ -158,6 +158,8 @@ _ORACLE_PROTOS = {
     "oracle_eager_tx_assign": (None, [ctypes.POINTER(EagerTx), c_i32, ctypes.POINTER(EagerHdr)]),
     "oracle_eager_tx_advance": (None, [ctypes.POINTER(EagerTx)]),
     "oracle_eager_fits": (c_int, [c_u64, ctypes.c_int64]),
+    "oracle_flush_post": (None, [c_vp, c_vp, c_u32]),
+    "oracle_flush_completed": (c_int, [c_vp, c_u32, c_u64]),
     "oracle_eager_copy_batch": (None, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_u32, c_vp]),
     "oracle_gin_stream_checksum": (c_u64, [c_u64, c_u32, c_u64, c_u32, c_u32, c_u32, c_u32, c_int,
                                            c_u32, c_u64, c_u64, c_u32, ctypes.POINTER(GinMr)]),

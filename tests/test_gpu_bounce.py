@@ -195,3 +195,30 @@ def test_gpu_glue(lib, gpu):
     host = np.zeros(8, dtype=np.uint8)
     assert lib.ofi_amd_gpu_seg_is_host(host.ctypes.data, ctypes.byref(is_host)) == 0 and is_host.value == 1
     assert lib.ofi_amd_gpu_get_device_for_addr(host.ctypes.data, ctypes.byref(dev)) < 0 and dev.value == -1
+
+
+@pytest.mark.parametrize("sentinel", [0x00000000FFFFFFFF, 0xDEADBEEFDEADBEEF])
+def test_sentinel_flush_reaches_every_rail_slot(lib, oracle, gpu, sentinel):
+    """GPU flush buffer -> one 64-byte pinned host slot per rail; complete when each slot's
+    first word shows the sentinel (RDMA and GIN sentinels of the reference)."""
+    d_buf = torch.zeros(8, dtype=torch.int64, device="cuda")
+    assert lib.ofi_amd_flush_buffer_fill(d_buf.data_ptr(), sentinel, _gpu.stream()) == 0
+    _gpu.sync()
+    assert np.all(_gpu.to_host(d_buf, np.uint64) == np.uint64(sentinel))
+    for rails in (1, 2, 3, 4):
+        slots = torch.zeros(8 * 4 + 8, dtype=torch.int64, pin_memory=True)
+        host = slots.numpy().view(np.uint64)
+        ptr = ctypes.c_void_p(slots.data_ptr())
+        assert lib.ofi_amd_flush_test(ptr, rails, sentinel) == 0
+        assert lib.ofi_amd_flush_post(d_buf.data_ptr(), ptr, rails, _gpu.stream()) == 0
+        _gpu.sync()
+        assert lib.ofi_amd_flush_test(ptr, rails, sentinel) == 1
+        want = np.zeros(40, dtype=np.uint64)
+        buf_host = _gpu.to_host(d_buf, np.uint64).copy()
+        oracle.oracle_flush_post(ctypes.c_void_p(buf_host.ctypes.data), ctypes.c_void_p(want.ctypes.data),
+                                 rails)
+        assert np.array_equal(host, want)               # slots of unused rails and the guard stay zero
+    assert lib.ofi_amd_flush_post(d_buf.data_ptr(), ptr, 0, _gpu.stream()) == -22
+    assert lib.ofi_amd_flush_post(d_buf.data_ptr(), ptr, 5, _gpu.stream()) == -22
+    assert lib.ofi_amd_flush_post(None, ptr, 1, _gpu.stream()) == -22
+    assert lib.ofi_amd_flush_buffer_fill(None, sentinel, _gpu.stream()) == -22

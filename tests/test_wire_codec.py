@@ -268,3 +268,28 @@ def test_product_matches_oracle_on_random_chains(lib, oracle):
         x, y = int(rng.integers(0, 1 << 16)), near(ls, 1 << 16)
         assert oracle.oracle_seq_before(x, y) == lib.ofi_amd_seq_before(x, y)
         assert oracle.oracle_eager_seq_before(x, y) == lib.ofi_amd_eager_seq_before(x, y)
+
+
+# ---- sentinel flush: host-side completion test ----
+
+def test_flush_completion_looks_at_the_first_word_of_every_rail_slot(lib, oracle):
+    import numpy as np
+    rdma, gin = 0x00000000FFFFFFFF, 0xDEADBEEFDEADBEEF          # include/nccl_ofi_rdma.h:45, gin_reqs.h:274
+    for sentinel in (rdma, gin):
+        for rails in (1, 2, 3, 4):
+            slots = np.zeros(8 * 4, dtype=np.uint64)
+            ptr = ctypes.c_void_p(slots.ctypes.data)
+            assert lib.ofi_amd_flush_test(ptr, rails, sentinel) == 0 == oracle.oracle_flush_completed(ptr, rails, sentinel)
+            buf = np.full(8, sentinel, dtype=np.uint64)
+            oracle.oracle_flush_post(ctypes.c_void_p(buf.ctypes.data), ptr, rails)
+            assert np.all(slots[:8 * rails] == sentinel) and not slots[8 * rails:].any()
+            assert lib.ofi_amd_flush_test(ptr, rails, sentinel) == 1 == oracle.oracle_flush_completed(ptr, rails, sentinel)
+            slots[8 * (rails - 1)] = 0                              # last rail's flag not there yet
+            assert lib.ofi_amd_flush_test(ptr, rails, sentinel) == 0 == oracle.oracle_flush_completed(ptr, rails, sentinel)
+            slots[8 * (rails - 1)] = sentinel
+            slots[8 * (rails - 1) + 1] = 0                          # only the first 8 bytes count
+            assert lib.ofi_amd_flush_test(ptr, rails, sentinel) == 1 == oracle.oracle_flush_completed(ptr, rails, sentinel)
+    slots = np.zeros(32, dtype=np.uint64)
+    assert lib.ofi_amd_flush_test(None, 1, rdma) == -22
+    assert lib.ofi_amd_flush_test(ctypes.c_void_p(slots.ctypes.data), 0, rdma) == -22
+    assert lib.ofi_amd_flush_test(ctypes.c_void_p(slots.ctypes.data), 5, rdma) == -22
