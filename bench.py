@@ -250,8 +250,13 @@ def bench_gin(lib, oracle, torch, np, args):
         out["cpu_generate_derive_fold_descs_per_s"] = nctx * sample / s1
         out["cpu_cores"] = 1
         out["cpu_sample"] = "%d ops per context" % sample
-        if sample == ops:
-            out["parity_ok"] = out["drain"]["checksum"] == "%016x" % ck
+        # parity at the full size: the oracle's checksums of the whole stream (a few seconds for the
+        # descriptors, about ten for the derived wire records at 256 x 1,000,000 ops)
+        if sample != ops:
+            ck = oracle.oracle_gin_stream_checksum(SEED, nctx, ops, 1, 64, 1, 1, 0, 4, 131072, 64, 1, omrs)
+        ck_wire = oracle.oracle_gin_stream_checksum(SEED, nctx, ops, 1, 64, 1, 1, 1, 4, 131072, 64, 1, omrs)
+        out["parity_ok"] = (out["drain"]["checksum"] == "%016x" % ck and
+                            out["drain_and_derive_wire"]["checksum"] == "%016x" % ck_wire)
     out["derive_checksums_agree_across_thread_counts"] = (
         out["drain_and_derive_wire"]["checksum"] == out["drain_and_derive_wire_4_proxy_threads"]["checksum"])
     return out
