@@ -28,6 +28,7 @@
  * HBM traffic per message: 8 B read twice + 4 B + 96 B written.
  */
 #include <mutex>
+#include <unordered_map>
 
 #include "common.hpp"
 #include "ofi_amd_hotpath.h"
@@ -357,14 +358,15 @@ __global__ __launch_bounds__(kThreads) void stripe_emit_kernel(
 	}
 }
 
-/* Per-process scratch for tile totals / prefixes, grown on demand. */
+/* Scratch for tile totals / prefixes, one per stream (launches on one stream are ordered, so
+ * they can share; launches on different streams may overlap and must not), grown on demand. */
 struct workspace_t {
-	std::mutex lock;
 	uint32_t *totals = nullptr;
 	uint32_t *prefix = nullptr; /* prefix[capacity] is the seed word */
 	uint32_t tiles = 0;
 };
-workspace_t g_ws;
+std::mutex g_ws_lock;
+std::unordered_map<void *, workspace_t> g_ws_by_stream;
 
 } // namespace
 
@@ -397,9 +399,11 @@ int ofi_amd_sched_batch(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes,
 
 	const uint32_t tiles = (uint32_t)((n + kTile - 1) / kTile);
 	uint32_t *totals, *prefix, *seed0;
-	{
-		std::lock_guard<std::mutex> g(g_ws.lock);
-		if (tiles > g_ws.tiles) {
+	hipStream_t s = as_stream(stream);
+	try {
+		std::lock_guard<std::mutex> g(g_ws_lock);
+		workspace_t &ws = g_ws_by_stream[stream];
+		if (tiles > ws.tiles) {
 			uint32_t want = tiles < 4096 ? 4096 : tiles;
 			uint32_t *a = nullptr, *b = nullptr;
 			OFI_AMD_HIP_TRY(hipMalloc((void **)&a, sizeof(uint32_t) * want));
@@ -407,20 +411,21 @@ int ofi_amd_sched_batch(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes,
 				(void)hipFree(a);
 				return -ENOMEM;
 			}
-			/* older buffers may still be in use by queued launches: sync first */
-			(void)hipDeviceSynchronize();
-			(void)hipFree(g_ws.totals);
-			(void)hipFree(g_ws.prefix);
-			g_ws.totals = a;
-			g_ws.prefix = b;
-			g_ws.tiles = want;
+			/* the older buffers may still be in use by launches queued on this stream */
+			(void)hipStreamSynchronize(s);
+			(void)hipFree(ws.totals);
+			(void)hipFree(ws.prefix);
+			ws.totals = a;
+			ws.prefix = b;
+			ws.tiles = want;
 		}
-		totals = g_ws.totals;
-		prefix = g_ws.prefix;
-		seed0 = g_ws.prefix + g_ws.tiles;
+		totals = ws.totals;
+		prefix = ws.prefix;
+		seed0 = ws.prefix + ws.tiles;
+	} catch (...) {
+		return -ENOMEM;
 	}
 
-	hipStream_t s = as_stream(stream);
 	hipLaunchKernelGGL(stripe_count_kernel, dim3(tiles), dim3(kThreads), 0, s, d_sizes,
 			   (uint32_t)n, d_state, align, totals, seed0, err);
 	if (tiles <= kInlineTiles) {

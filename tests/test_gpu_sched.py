@@ -143,3 +143,28 @@ def test_full_size_configuration(lib, oracle, gpu):
     # invariants that hold at any size
     assert np.array_equal(xf[:, :, 2].sum(axis=1), sizes)
     assert set(np.unique(num)) <= {1, 2, 4}
+
+
+def test_batches_on_two_streams_do_not_share_scratch(lib, oracle, gpu):
+    """Two scheduler instances driven from two streams at once (two endpoints in one process):
+    each stream has its own tile scratch, so overlapping launches cannot mix their seeds."""
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    cases = []
+    for k, (rails, seeds, n) in enumerate([(4, (1, 2), 700_001), (3, (2, 0), 650_003)]):
+        sizes = synthetic.stripe_sizes(900 + k, n)
+        want = _oracle.sched_batch(oracle, sizes, rails, 131072, 64, seeds)
+        cases.append((sizes, want, dev_state(rails, 131072, 64, seeds), _gpu.to_dev(sizes),
+                      torch.full((n,), -1, dtype=torch.int32, device="cuda"),
+                      torch.full((n * 12,), -1, dtype=torch.int64, device="cuda")))
+    torch.cuda.synchronize()
+    for s, (sizes, _w, d_state, d_sizes, d_num, d_xf) in zip(streams, cases):
+        assert lib.ofi_amd_sched_batch(d_state.data_ptr(), d_sizes.data_ptr(), len(sizes), 128,
+                                       d_num.data_ptr(), d_xf.data_ptr(),
+                                       ctypes.c_void_p(s.cuda_stream)) == 0
+    torch.cuda.synchronize()
+    for sizes, (want_num, want_xf, ost), d_state, _d, d_num, d_xf in cases:
+        n = len(sizes)
+        assert np.array_equal(_gpu.to_host(d_num, np.uint32), want_num)
+        assert np.array_equal(_gpu.to_host(d_xf, np.uint64).reshape(n, 4, 3), want_xf)
+        st = read_state(d_state)
+        assert (st.rr_small_counter, st.rr_counter) == (ost.rr_small_counter, ost.rr_counter)
