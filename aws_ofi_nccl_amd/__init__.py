@@ -74,6 +74,12 @@ class GinProxyStats(ctypes.Structure):
                 ("checksum", c_u64), ("seconds", ctypes.c_double), ("empty_polls", c_u64)]
 
 
+class GinDevRing(ctypes.Structure):
+    """ofi_amd_gin_dev_ring_t"""
+    _fields_ = [("records", c_vp), ("sequences", c_vp), ("reserve", c_vp), ("status", c_vp),
+                ("capacity", c_u32), ("context", c_u32)]
+
+
 class GinSignalWork(ctypes.Structure):
     """ofi_amd_gin_signal_work_t (32 bytes)"""
     _fields_ = [("base", c_u64), ("offset", c_u64), ("value", c_u64), ("peer", c_u32),
@@ -227,6 +233,8 @@ PROTOTYPES = {
                                               ctypes.POINTER(c_u32), ctypes.POINTER(c_u32)]),
     "ofi_amd_gin_produce_seeded": (ctypes.c_int, [c_vp, c_u64, c_u64, c_u32, c_u32, c_u32, c_u32,
                                                   c_u64, c_vp]),
+    "ofi_amd_gin_rings_device_view": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(GinDevRing)]),
+    "ofi_amd_gin_produce_table": (ctypes.c_int, [c_vp, c_vp, c_u64, c_u32, c_u64, c_vp]),
     "ofi_amd_gin_producer_status": (ctypes.c_int, [c_vp]),
     "ofi_amd_gin_ring_push": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(GinDesc)]),
     "ofi_amd_gin_ring_pop": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(GinDesc)]),

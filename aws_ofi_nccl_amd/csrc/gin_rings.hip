@@ -19,14 +19,16 @@
  *      1 KiB contiguous per instruction, to the pinned ring;
  *   4. system-scope fence, then each lane publishes sequence = position + 1
  *      with a release store (64 lanes = one contiguous 256-byte write).
- * The ring cursor stays in a register for the whole launch and is written back
- * once at the end.
+ * The ring cursor (device memory, shared with ofi_amd_gin_dev_put) stays in a register for
+ * the whole launch and is written back once at the end: this generator owns its context
+ * for the duration of a launch.
  */
 #include <cstring>
 #include <new>
 
 #include "common.hpp"
 #include "gin_rings.hpp"
+#include "ofi_amd_gin_device.h"
 
 namespace {
 
@@ -35,6 +37,8 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr uint32_t kThreads = 256;
 constexpr uint32_t kWaves = kThreads / 64;
 constexpr uint64_t kDefaultSpinLimit = 1ull << 22;
+static_assert(OFI_AMD_GIN_DEV_TIMEOUT_BIT == ofi_amd::ASYNC_ERR_GIN_TIMEOUT,
+	      "the device header and the status reader agree on the timeout bit");
 
 __device__ __forceinline__ uint64_t mix64(uint64_t z)
 {
@@ -105,8 +109,8 @@ __global__ __launch_bounds__(kThreads) void gin_produce_seeded_kernel(
 	u32x4 *ring = records + (uint64_t)ctx * capacity * 4;
 	uint32_t *seq = sequences + (uint64_t)ctx * capacity;
 
-	uint32_t cursor = __hip_atomic_load(&enqueue_pos[ctx * 16], __ATOMIC_RELAXED,
-					    __HIP_MEMORY_SCOPE_SYSTEM);
+	uint32_t cursor = __hip_atomic_load(&enqueue_pos[ctx * kGinReserveStride], __ATOMIC_RELAXED,
+					    __HIP_MEMORY_SCOPE_AGENT);
 
 	for (uint64_t round = 0; round < ops; round += kThreads) {
 		const uint64_t i = round + threadIdx.x;
@@ -197,8 +201,31 @@ __global__ __launch_bounds__(kThreads) void gin_produce_seeded_kernel(
 	}
 
 	if (threadIdx.x == 0) {
-		__hip_atomic_store(&enqueue_pos[ctx * 16], cursor, __ATOMIC_RELEASE,
-				   __HIP_MEMORY_SCOPE_SYSTEM);
+		__hip_atomic_store(&enqueue_pos[ctx * kGinReserveStride], cursor, __ATOMIC_RELEASE,
+				   __HIP_MEMORY_SCOPE_AGENT);
+	}
+}
+
+/* Multi-producer form: one wavefront per workgroup, `waves` of them per context, each putting
+ * its share of a descriptor table through the device-side put. */
+__global__ __launch_bounds__(64) void gin_produce_table_kernel(
+	ofi_amd_gin_dev_ring_t first, const ofi_amd_gin_desc_t *__restrict__ table, uint64_t ops,
+	uint32_t waves, uint64_t spin_limit)
+{
+	const uint32_t ctx = blockIdx.x / waves, g = blockIdx.x % waves;
+	ofi_amd_gin_dev_ring_t ring = first; /* context 0; the arrays of context c follow at fixed strides */
+	ring.records = static_cast<uint8_t *>(first.records) + (uint64_t)ctx * first.capacity * 64u;
+	ring.sequences = first.sequences + (uint64_t)ctx * first.capacity;
+	ring.reserve = first.reserve + (uint64_t)ctx * kGinReserveStride;
+	ring.context = ctx;
+	const ofi_amd_gin_desc_t *mine = table + (uint64_t)ctx * ops;
+	for (uint64_t group = g; group * 64u < ops; group += waves) {
+		const uint64_t i = group * 64u + threadIdx.x;
+		const bool active = i < ops;
+		const ofi_amd_gin_desc_t d = mine[active ? i : ops - 1];
+		if (ofi_amd_gin_dev_put(ring, &d, active, spin_limit) != 0) {
+			return; /* wave-uniform: the whole wave leaves */
+		}
 	}
 }
 
@@ -217,6 +244,7 @@ int ofi_amd_gin_rings_destroy(ofi_amd_gin_rings_t *r)
 	if (r->sequences) (void)hipHostFree(r->sequences);
 	if (r->enqueue_pos) (void)hipHostFree(r->enqueue_pos);
 	if (r->status) (void)hipHostFree(r->status);
+	if (r->d_reserve) (void)hipFree(r->d_reserve);
 	delete[] r->dequeue_pos;
 	delete r;
 	return 0;
@@ -249,6 +277,9 @@ int ofi_amd_gin_rings_create(uint32_t n_contexts, uint32_t capacity, ofi_amd_gin
 	if (e == hipSuccess) e = hipHostGetDevicePointer((void **)&r->d_sequences, r->sequences, 0);
 	if (e == hipSuccess) e = hipHostGetDevicePointer((void **)&r->d_enqueue_pos, r->enqueue_pos, 0);
 	if (e == hipSuccess) e = hipHostGetDevicePointer((void **)&r->d_status, r->status, 0);
+	const size_t reserve_bytes = (size_t)n_contexts * kGinReserveStride * sizeof(uint32_t);
+	if (e == hipSuccess) e = hipMalloc((void **)&r->d_reserve, reserve_bytes);
+	if (e == hipSuccess) e = hipMemset(r->d_reserve, 0, reserve_bytes);
 	r->dequeue_pos = new (std::nothrow) uint32_t[n_contexts]();
 	if (e != hipSuccess || !r->dequeue_pos) {
 		ofi_amd_gin_rings_destroy(r);
@@ -297,8 +328,49 @@ int ofi_amd_gin_produce_seeded(ofi_amd_gin_rings_t *r, uint64_t seed, uint64_t o
 	}
 	hipLaunchKernelGGL(gin_produce_seeded_kernel, dim3(r->n_contexts), dim3(kThreads), 0,
 			   as_stream(stream), reinterpret_cast<u32x4 *>(r->d_records), r->d_sequences,
-			   r->d_enqueue_pos, r->d_status, r->capacity, seed, ops_per_context, peer_rank,
+			   r->d_reserve, r->d_status, r->capacity, seed, ops_per_context, peer_rank,
 			   signal_every, signal_op, aggregate_mask,
+			   spin_limit ? spin_limit : kDefaultSpinLimit);
+	OFI_AMD_HIP_TRY(hipGetLastError());
+	return 0;
+}
+
+int ofi_amd_gin_rings_device_view(ofi_amd_gin_rings_t *r, uint32_t context, ofi_amd_gin_dev_ring_t *out)
+{
+	if (!r || !out || context >= r->n_contexts) {
+		return -EINVAL;
+	}
+	out->records = r->d_records + (size_t)context * r->capacity;
+	out->sequences = r->d_sequences + (size_t)context * r->capacity;
+	out->reserve = r->d_reserve + (size_t)context * kGinReserveStride;
+	out->status = r->d_status;
+	out->capacity = r->capacity;
+	out->context = context;
+	return 0;
+}
+
+int ofi_amd_gin_produce_table(ofi_amd_gin_rings_t *r, const ofi_amd_gin_desc_t *d_table,
+			      uint64_t ops_per_context, uint32_t waves_per_context, uint64_t spin_limit,
+			      void *stream)
+{
+	int rc = require_device();
+	if (rc != 0) {
+		return rc;
+	}
+	if (!r || !d_table || waves_per_context < 1 || waves_per_context > 1024 ||
+	    ops_per_context > (1ull << 38) || (uint64_t)r->n_contexts * waves_per_context > (1u << 30)) {
+		return -EINVAL;
+	}
+	if (ops_per_context == 0) {
+		return 0;
+	}
+	ofi_amd_gin_dev_ring_t first;
+	rc = ofi_amd_gin_rings_device_view(r, 0, &first);
+	if (rc != 0) {
+		return rc;
+	}
+	hipLaunchKernelGGL(gin_produce_table_kernel, dim3(r->n_contexts * waves_per_context), dim3(64), 0,
+			   as_stream(stream), first, d_table, ops_per_context, waves_per_context,
 			   spin_limit ? spin_limit : kDefaultSpinLimit);
 	OFI_AMD_HIP_TRY(hipGetLastError());
 	return 0;

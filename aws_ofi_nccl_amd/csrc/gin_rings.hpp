@@ -32,6 +32,10 @@ struct ofi_amd_gin_rings {
 	uint32_t *d_sequences;
 	uint32_t *d_enqueue_pos;
 	uint32_t *d_status;
+	/* device memory: reservation cursor of the GPU producers, one per 128-byte line */
+	uint32_t *d_reserve;
 };
+
+constexpr uint32_t kGinReserveStride = 32; /* u32 words between two contexts' cursors */
 
 #endif

@@ -1,0 +1,99 @@
+/*
+ * Device side of the GIN descriptor rings: what a HIP kernel calls to initiate a put or
+ * put-signal.  Compile with hipcc for gfx950; host code only needs ofi_amd_hotpath.h.
+ *
+ * The reference has no such call on AMD or in proxy mode -- NCCL's own GPU-to-CPU queue
+ * feeds its proxy thread, which calls iputSignal (src/rdma/gin/nccl_ofi_gin_api.cpp:370-419);
+ * its GPU-initiated build posts NIC work queue entries from device code instead
+ * (include/rdma/gin/nccl_ofi_gin_gdaki_dev.h:131-336).  Here the device hands the host proxy
+ * the iputSignal argument tuple through a ring with the slot protocol of
+ * include/nccl_ofi_mpsc_ring.h:79-143: a slot's sequence word equals its position when free,
+ * position + 1 when published; the consumer frees it with position + capacity.
+ */
+#ifndef OFI_AMD_GIN_DEVICE_H_
+#define OFI_AMD_GIN_DEVICE_H_
+
+#include <hip/hip_runtime.h>
+
+#include "ofi_amd_hotpath.h"
+
+#define OFI_AMD_GIN_DEV_TIMEOUT_BIT 2u /* the bit ofi_amd_gin_producer_status() reports */
+
+/*
+ * Wave-collective: all 64 lanes of the wavefront call it together (no divergence around
+ * the call); lanes with active == true each put *desc.  Returns 0, or -1 when the ring
+ * stayed full for spin_limit polls -- the timeout bit is then set in the ring's status word
+ * and the reserved slots are never published, so the ring must not be used any further.
+ *
+ * The wave's descriptors take consecutive positions in lane order: one atomic add on the
+ * device-resident cursor per call (not per descriptor, and nothing atomic over the host
+ * link), positions from a ballot and a prefix popcount.  The single consumer frees slots
+ * in position order, so one lane polling the wave's last slot is enough.  Records go out
+ * as four 16-byte stores per lane, then a system-scope release fence, then the sequence
+ * words: the host proxy that sees a published sequence word sees the record.
+ */
+__device__ __forceinline__ int ofi_amd_gin_dev_put(const ofi_amd_gin_dev_ring_t ring,
+						    const ofi_amd_gin_desc_t *desc, bool active,
+						    uint64_t spin_limit)
+{
+	typedef uint32_t ofi_amd_u32x4 __attribute__((ext_vector_type(4)));
+	const uint32_t lane = __lane_id();
+	const uint64_t ballot = __ballot(active);
+	if (ballot == 0) {
+		return 0;
+	}
+	const uint32_t count = (uint32_t)__popcll(ballot);
+	const uint32_t rank = (uint32_t)__popcll(ballot & ((1ull << lane) - 1ull));
+	const uint32_t leader = (uint32_t)__ffsll((unsigned long long)ballot) - 1u;
+	const uint32_t mask = ring.capacity - 1u;
+
+	uint32_t base = 0;
+	if (lane == leader) {
+		base = __hip_atomic_fetch_add(ring.reserve, count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+	}
+	base = __shfl(base, (int)leader, 64);
+	const uint32_t pos = base + rank;
+
+	int timed_out = 0;
+	if (lane == leader) {
+		const uint32_t last_pos = base + count - 1u;
+		uint64_t spins = 0;
+		while (__hip_atomic_load(&ring.sequences[last_pos & mask], __ATOMIC_RELAXED,
+					 __HIP_MEMORY_SCOPE_SYSTEM) != last_pos) {
+			if (++spins > spin_limit) {
+				timed_out = 1;
+				break;
+			}
+			__builtin_amdgcn_s_sleep(16);
+		}
+		if (timed_out) {
+			__hip_atomic_fetch_or(ring.status, OFI_AMD_GIN_DEV_TIMEOUT_BIT, __ATOMIC_RELAXED,
+					      __HIP_MEMORY_SCOPE_SYSTEM);
+		}
+	}
+	if (__shfl(timed_out, (int)leader, 64)) {
+		return -1;
+	}
+	__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+
+	if (active) {
+		ofi_amd_u32x4 *dst = static_cast<ofi_amd_u32x4 *>(ring.records) + (uint64_t)(pos & mask) * 4u;
+		ofi_amd_u32x4 a, b, c, d; /* the descriptor is only 8-byte aligned: copy, do not cast */
+		__builtin_memcpy(&a, reinterpret_cast<const char *>(desc), 16);
+		__builtin_memcpy(&b, reinterpret_cast<const char *>(desc) + 16, 16);
+		__builtin_memcpy(&c, reinterpret_cast<const char *>(desc) + 32, 16);
+		__builtin_memcpy(&d, reinterpret_cast<const char *>(desc) + 48, 16);
+		dst[0] = a;
+		dst[1] = b;
+		dst[2] = c;
+		dst[3] = d;
+	}
+	__builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+	if (active) {
+		__hip_atomic_store(&ring.sequences[pos & mask], pos + 1u, __ATOMIC_RELAXED,
+				   __HIP_MEMORY_SCOPE_SYSTEM);
+	}
+	return 0;
+}
+
+#endif /* OFI_AMD_GIN_DEVICE_H_ */

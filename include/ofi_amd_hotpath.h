@@ -234,6 +234,38 @@ int ofi_amd_gin_produce_seeded(ofi_amd_gin_rings_t *rings, uint64_t seed,
 /* After the stream has been synchronised: 0, or -ETIMEDOUT if any producer gave up. */
 int ofi_amd_gin_producer_status(ofi_amd_gin_rings_t *rings);
 
+/*
+ * What device code needs to put descriptors into the ring of one context from any number
+ * of wavefronts at once (the multi-producer side of nccl_ofi_mpsc_ring,
+ * include/nccl_ofi_mpsc_ring.h:79-118): device addresses of the record and sequence arrays,
+ * the producers' reservation cursor (device memory: only producers touch it, the consumer
+ * goes by the sequence words) and the status word.  Passed to kernels by value; the
+ * wave-collective put itself is ofi_amd_gin_dev_put() in include/ofi_amd_gin_device.h.
+ * A ring takes GPU producers (this cursor) or host producers (ofi_amd_gin_ring_push), not both.
+ */
+typedef struct {
+	void *records;       /* 64-byte records, [capacity] */
+	uint32_t *sequences; /* [capacity] */
+	uint32_t *reserve;   /* next position to hand out */
+	uint32_t *status;
+	uint32_t capacity;
+	uint32_t context;
+} ofi_amd_gin_dev_ring_t;
+int ofi_amd_gin_rings_device_view(ofi_amd_gin_rings_t *rings, uint32_t context,
+				  ofi_amd_gin_dev_ring_t *out);
+
+/*
+ * Multi-producer launch: waves_per_context wavefronts per context (1..1024, each its own
+ * workgroup) put the descriptors of a device-resident table d_table[context][ops_per_context]
+ * through ofi_amd_gin_dev_put().  Wave g of a context takes the 64-descriptor groups g,
+ * g + waves, g + 2*waves, ...; each group lands in 64 consecutive slots, a wave's groups
+ * land in order (per-producer FIFO), the interleaving between waves is up to the hardware.
+ * With one wave per context the ring order is the table order.
+ */
+int ofi_amd_gin_produce_table(ofi_amd_gin_rings_t *rings, const ofi_amd_gin_desc_t *d_table,
+			      uint64_t ops_per_context, uint32_t waves_per_context,
+			      uint64_t spin_limit, void *stream);
+
 /* Host-side push with the same protocol (CPU producer threads; CAS claim as in
  * nccl_ofi_mpsc_ring::push).  1 pushed, 0 full. */
 int ofi_amd_gin_ring_push(ofi_amd_gin_rings_t *rings, uint32_t context,
