@@ -212,7 +212,7 @@ def bench_gin(lib, oracle, torch, np, args):
     nctx, cap, ops = 256, 4096, args.gin_ops
     out = {"contexts": nctx, "ring_capacity": cap, "ops_per_context": ops}
     # NCCL runs up to NCCL_GIN_MAX_CONNECTIONS = 4 GIN proxy threads (nccl/net.h:38)
-    for mode, threads, key in ((0, 1, "drain"), (2, 1, "drain_and_derive_wire"),
+    for mode, threads, key in ((0, 1, "drain"), (0, 4, "drain_4_proxy_threads"), (2, 1, "drain_and_derive_wire"),
                                (2, 4, "drain_and_derive_wire_4_proxy_threads")):
         rings = ctypes.c_void_p()
         m.check(lib.ofi_amd_gin_rings_create(nctx, cap, ctypes.byref(rings)), "rings_create")
@@ -236,6 +236,28 @@ def bench_gin(lib, oracle, torch, np, args):
                     "consumer_ns_per_desc": secs / stats.descriptors * 1e9, "proxy_threads": threads,
                     "checksum": "%016x" % stats.checksum, "rdma_writes": stats.writes}
         lib.ofi_amd_gin_rings_destroy(rings)
+    # the general device-side put: several producing wavefronts per ring, descriptors from a table
+    t_ops = min(ops, 100_000)
+    d_table = torch.randint(0, 1 << 62, (nctx * t_ops * 8,), dtype=torch.int64, device="cuda")
+    for waves in (1, 4):
+        rings = ctypes.c_void_p()
+        m.check(lib.ofi_amd_gin_rings_create(nctx, cap, ctypes.byref(rings)), "rings_create")
+        stats = m.GinProxyStats()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        m.check(lib.ofi_amd_gin_produce_table(rings, d_table.data_ptr(), t_ops, waves, 0, _gpu.stream()),
+                "produce_table")
+        rc = lib.ofi_amd_gin_proxy_drain_mt(rings, t_ops, 0, None, None, None, None, 20000, 4,
+                                            ctypes.byref(stats))
+        torch.cuda.synchronize()
+        secs = time.perf_counter() - t0
+        if rc != 0 or lib.ofi_amd_gin_producer_status(rings) != 0:
+            raise RuntimeError("gin table drain rc=%d" % rc)
+        out["device_put_%d_waves_per_context" % waves] = {
+            "descriptors": stats.descriptors, "seconds": secs, "descs_per_s": stats.descriptors / secs,
+            "host_link_gbs": stats.descriptors * 68 / secs / 1e9, "proxy_threads": 4}
+        lib.ofi_amd_gin_rings_destroy(rings)
+    del d_table
     if not args.skip_cpu:
         # oracle: generate + fold the same stream on one core, on a bounded sample of the ops
         sample = min(ops, 40000)
