@@ -93,6 +93,43 @@ def bench_bounce(lib, oracle, torch, np, args):
         cpu_s = (time.perf_counter() - t0) / reps
         cpu = {"value": algo_bytes / cpu_s / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
                "sample": "%d passes of the full batch (per-buffer memcpy loop, 1 thread)" % reps}
+        # the same loop on every host core the box gives us: contiguous slices of the batch per thread
+        # (the oracle call runs outside the interpreter lock)
+        import threading
+        cores = min(16, os.cpu_count() or 1)
+        bounds = [n * t // cores for t in range(cores + 1)]
+
+        def part(lo, hi):
+            for _ in range(reps):
+                oracle.oracle_bounce_scatter(_oracle.ptr(src), _oracle.ptr(arena),
+                                             _oracle.ptr(w["src_off"][lo:hi]), _oracle.ptr(w["dst_off"][lo:hi]),
+                                             _oracle.ptr(w["len"][lo:hi]), hi - lo, _oracle.ptr(flush[lo:hi]))
+        threads = [threading.Thread(target=part, args=(bounds[t], bounds[t + 1])) for t in range(cores)]
+        t0 = time.perf_counter()
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        out["cpu_all_cores"] = {"value": algo_bytes * reps / (time.perf_counter() - t0) / 1e9, "unit": "GB/s",
+                                "cores": cores}
+        # reference-style: one synchronous copy call per buffer through the device-copy interface
+        # (nccl_ofi_device_copy::copy_to_device), on a bounded sample of the batch
+        import aws_ofi_nccl_amd as m
+        sample = min(n, 8192)
+        region = ctypes.c_void_p()
+        m.check(lib.ofi_amd_devcopy_register(d_arena.data_ptr(), w["arena_bytes"], ctypes.byref(region)),
+                "devcopy_register")
+        t0 = time.perf_counter()
+        for i in range(sample):
+            rc = lib.ofi_amd_devcopy_to_device(src.ctypes.data + int(w["src_off"][i]), region,
+                                               int(w["dst_off"][i]), int(w["len"][i]))
+            if rc != 0:
+                raise RuntimeError("devcopy_to_device: %d" % rc)
+        per_call_s = time.perf_counter() - t0
+        lib.ofi_amd_devcopy_deregister(region)
+        out["per_buffer_copy_calls"] = {
+            "value": float(w["len"][:sample].sum()) / per_call_s / 1e9, "unit": "GB/s payload",
+            "buffers_per_s": sample / per_call_s, "sample": "%d buffers, one host-to-device call each" % sample}
     del d_arena, d_src, d_tmp
     torch.cuda.empty_cache()
     return out, cpu
@@ -321,6 +358,9 @@ def main():
             log(name)
             extra[name] = fn(lib, oracle, torch, np, args)
 
+    baselines = {k: bounce[k] for k in ("cpu_all_cores", "per_buffer_copy_calls") if k in bounce}
+    if baselines:
+        extra["bounce_baselines"] = baselines
     # HBM bytes per launch of bounce_scatter_kernel on this batch, from the rocprofv3 FETCH_SIZE /
     # WRITE_SIZE runs summarised in profiles/bounce_scatter_kernel_65536buf_2GiB_arena.md
     # (273,371.4 KiB read + 266,846.6 KiB written after scaling by the plain-copy factors)
