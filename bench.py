@@ -135,6 +135,56 @@ def bench_bounce(lib, oracle, torch, np, args):
     return out, cpu
 
 
+def bench_eager(lib, oracle, torch, np, args):
+    """Eager arrivals in rx-buffer format (8-byte header + payload per 8320-byte rx buffer) copied to
+    receive buffers at arbitrary alignment: rx pool in HBM, and rx pool in pinned host memory (where
+    the reference's NIC puts them), which is bound by the host link."""
+    import _gpu
+    import _oracle
+    n, stride = 65536, 8320
+    rng = np.random.default_rng(SEED)
+    recv_len = rng.integers(0, 8185, n).astype(np.uint32)
+    rx_off = rng.permutation(n).astype(np.uint64) * np.uint64(stride)
+    dst_off = (rng.permutation((2 << 30) // 16384)[:n].astype(np.uint64) * np.uint64(16384)
+               + rng.integers(0, 64, n).astype(np.uint64))
+    rx_host = torch.empty(n * stride, dtype=torch.uint8, pin_memory=True)
+    rx_host.numpy()[:] = rng.integers(0, 256, n * stride, dtype=np.uint8)
+    rx_dev = rx_host.cuda()
+    d_arena = torch.zeros(2 << 30, dtype=torch.uint8, device="cuda")
+    d_ro, d_rl, d_do = _gpu.to_dev(rx_off), _gpu.to_dev(recv_len), _gpu.to_dev(dst_off)
+    d_copied = torch.zeros(n, dtype=torch.int32, device="cuda")
+    d_flush = torch.zeros(n, dtype=torch.int32, device="cuda")
+    stream = _gpu.stream()
+    payload = int(recv_len.astype(np.int64).sum())
+    out = {"buffers": n, "payload_bytes": payload}
+    for key, pool in (("rx_pool_in_hbm", rx_dev), ("rx_pool_in_pinned_host", rx_host)):
+        def step():
+            rc = lib.ofi_amd_eager_copy_batch(pool.data_ptr(), d_ro.data_ptr(), d_rl.data_ptr(),
+                                              d_arena.data_ptr(), d_do.data_ptr(), d_rl.data_ptr(), n,
+                                              d_copied.data_ptr(), d_flush.data_ptr(), stream)
+            if rc != 0:
+                raise RuntimeError("ofi_amd_eager_copy_batch: %d" % rc)
+        wall_ms, ev_ms = timed_steps(step, max(3, args.steps // 4), 2, torch)
+        out[key] = {"ms_kernel": ev_ms, "payload_gbs": payload / ev_ms / 1e6,
+                    "read_plus_written_gbs": 2 * payload / ev_ms / 1e6}
+    # result check on a strided sample of the buffers against the oracle's copy
+    idx = np.arange(0, n, 97)
+    want = np.zeros(len(idx) * 8192, dtype=np.uint8)
+    w_off = np.arange(len(idx), dtype=np.uint64) * np.uint64(8192)
+    oracle.oracle_eager_copy_batch(_oracle.ptr(rx_host.numpy()), _oracle.ptr(rx_off[idx].copy()),
+                                   _oracle.ptr(recv_len[idx].copy()), _oracle.ptr(want), _oracle.ptr(w_off),
+                                   _oracle.ptr(recv_len[idx].copy()), len(idx), None)
+    ok = True
+    arena_host = None
+    for k, i in enumerate(idx):
+        got = d_arena[int(dst_off[i]):int(dst_off[i]) + int(recv_len[i])].cpu().numpy()
+        ok = ok and bool(np.array_equal(got, want[k * 8192:k * 8192 + int(recv_len[i])]))
+    out["parity_ok"] = ok and bool(np.array_equal(_gpu.to_host(d_copied, np.uint32), recv_len))
+    del d_arena, rx_dev, rx_host, arena_host
+    torch.cuda.empty_cache()
+    return out
+
+
 def bench_sched(lib, oracle, torch, np, args):
     import _gpu
     import _oracle
@@ -328,7 +378,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--gin-ops", type=int, default=1_000_000, help="GIN ops per context")
     ap.add_argument("--skip-extra", action="store_true", help="only the bounce-copy step")
-    ap.add_argument("--extra", default="striping,tuner,gin", help="which other paths to time")
+    ap.add_argument("--extra", default="eager,striping,tuner,gin", help="which other paths to time")
     ap.add_argument("--skip-cpu", action="store_true", help="no CPU baselines")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -352,7 +402,7 @@ def main():
     bounce, cpu = bench_bounce(lib, oracle, torch, np, args)
     extra = {}
     if not args.skip_extra:
-        for name, fn in (("striping", bench_sched), ("tuner", bench_tuner), ("gin", bench_gin)):
+        for name, fn in (("eager", bench_eager), ("striping", bench_sched), ("tuner", bench_tuner), ("gin", bench_gin)):
             if name not in args.extra.split(","):
                 continue
             log(name)
