@@ -67,6 +67,31 @@ def test_every_length_and_source_alignment(lib, oracle, gpu):
     assert np.array_equal(flush, want_flush)
 
 
+def test_lengths_beyond_one_trip_and_every_row_count(lib, oracle, gpu):
+    """Buffers larger than the 8 KiB eager limit loop over whole trips first; every number of
+    1 KiB rows (1..8) in the last trip is hit at word-aligned and byte-misaligned sources."""
+    lens = [r * 1024 + d for r in range(0, 9) for d in (-17, -1, 0, 1, 16)]
+    lens += [8192 * k + d for k in (2, 3, 5) for d in (-1, 0, 1, 1000, 4097)] + [100_000, 1 << 20]
+    lens = [l for l in lens if l >= 0]
+    length = np.array([l for l in lens for _ in range(3)], dtype=np.uint32)
+    n = len(length)
+    align = np.tile(np.array([0, 1, 6], dtype=np.uint64), len(lens))
+    room = ((length.astype(np.uint64) + np.uint64(64 + 63)) // np.uint64(64)) * np.uint64(64)
+    starts = np.concatenate([[np.uint64(0)], np.cumsum(room)[:-1]]).astype(np.uint64)
+    src_off = starts + align
+    slot = np.uint64(((int(length.max()) + 127) // 64) * 64)
+    dst_off = np.random.default_rng(6).permutation(n).astype(np.uint64) * slot
+    total_src = int(starts[-1] + room[-1]) + 64
+    src = synthetic.random_bytes(6, total_src)
+    want = np.full(n * int(slot), 0x33, dtype=np.uint8)
+    want_flush = oracle_scatter(oracle, src, want, src_off, dst_off, length)
+    arena = torch.full((n * int(slot),), 0x33, dtype=torch.uint8, device="cuda")
+    flush = scatter(lib, src, arena, src_off, dst_off, length)
+    assert np.array_equal(arena.cpu().numpy(), want)
+    assert np.array_equal(flush, want_flush)
+    assert _gpu.fetch_async_errors(lib) == 0
+
+
 def test_empty_batch_and_all_zero_lengths(lib, oracle, gpu):
     arena = torch.full((4096,), 9, dtype=torch.uint8, device="cuda")
     assert lib.ofi_amd_bounce_scatter(arena.data_ptr(), arena.data_ptr(), 4096, None, None, None, 0,
