@@ -244,7 +244,7 @@ def test_region_table_matches_reference_source():
 
 
 def test_region_table_shape(oracle):
-    """Which (platform, shape, collective) have regions: SURVEY of nccl_ofi_regions.cpp:295-1882."""
+    """Which (platform, shape, collective) have regions: the per-platform tables of src/tuner/nccl_ofi_regions.cpp:295-1882."""
     algos, protos, nv = (ctypes.c_int * 16)(), (ctypes.c_int * 16)(), (ctypes.c_int * 16)()
     verts = (Point * (16 * 20))()
     count = lambda plat, R, N, coll: oracle.oracle_region_polys(plat, R, N, coll, algos, protos, nv, verts, 16)
