@@ -286,6 +286,22 @@ def bench_tuner(lib, oracle, torch, np, args):
             grids += 1
         out["cpu_region_points_per_s"] = grids * points / (time.perf_counter() - t0)
         out["cpu_cores"] = 1
+        # parity of the timed launches: the first four grids of each kind against the oracle
+        model_step()
+        region_step()
+        torch.cuda.synchronize()
+        g_cost = d_cost.cpu().numpy().reshape(nv, cells)
+        g_choice = d_choice.cpu().numpy().reshape(nv, points * 2)
+        g_reg = d_reg.cpu().numpy().reshape(nv, points, 4)
+        ok = True
+        for v in range(4):
+            oracle.oracle_model_grid(v % 2, 1 + v // 2, 8, 3, *axes, _oracle.ptr(algos), len(algos),
+                                     _oracle.ptr(cost), _oracle.ptr(choice))
+            ok = ok and bool(np.array_equal(g_cost[v], cost)) and bool(np.array_equal(g_choice[v], choice))
+            oracle.oracle_region_grid(v % 4, *axes, _oracle.ptr(rchoice))
+            ok = ok and bool(np.array_equal(g_reg[v][:, :2].astype(np.int32),
+                                            rchoice.reshape(points, 3)[:, :2]))
+        out["parity_ok"] = ok
         out["model_speedup_vs_cpu_core"] = out["model_cells_per_s"] / out["cpu_model_cells_per_s"]
         out["region_speedup_vs_cpu_core"] = out["region_points_per_s"] / out["cpu_region_points_per_s"]
     lib.ofi_amd_tuner_plan_destroy(plan)
