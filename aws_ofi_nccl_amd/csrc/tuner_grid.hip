@@ -5,8 +5,8 @@
  * object and the host-side construction of the log2-space polygon tables
  * (extend_region + set_regions, src/tuner/nccl_ofi_regions.cpp:224-289).
  *
- * Nothing here is matrix-shaped: one thread per cost cell (8-byte coalesced stores)
- * and one thread per decision point.
+ * Nothing here is matrix-shaped: one thread per decision point, which also evaluates the
+ * point's cost cells (staged in LDS, written out as contiguous runs).
  */
 #include <cstring>
 #include <mutex>
@@ -33,82 +33,87 @@ struct grid_dims_t {
 	const double *log2_ranks; /* per (node, ppn): transform_log2 of the rank count */
 };
 
-/* One thread per cost cell. */
-__global__ __launch_bounds__(256) void model_cost_kernel(grid_dims_t g,
+/*
+ * One thread per decision point; blockIdx.y is the variant.  The thread evaluates the
+ * n_algos x 3 cost cells of its point -- contiguous in the output -- and its decision.  Cells
+ * are staged in LDS so that the workgroup writes its 256 x cells-per-point doubles as one
+ * contiguous run (a lane-per-point store would touch 64 cache lines per instruction).
+ */
+template <bool COST, bool CHOICE>
+__global__ __launch_bounds__(256) void model_grid_kernel(grid_dims_t g,
 							 const ofi_amd_tuner_variant_t *__restrict__ variants,
-							 uint32_t n_variants, uint64_t cells_per_variant,
-							 double *__restrict__ cost)
+							 uint32_t points_per_variant, double *__restrict__ cost,
+							 int8_t *__restrict__ choice)
 {
-	const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;
-	if (idx >= cells_per_variant * n_variants) {
-		return;
+	extern __shared__ double stage[]; /* [256][cells per point] when COST */
+	const uint32_t cpp = g.n_algos * NUM_PROTOS;
+	const uint32_t first = blockIdx.x * 256u;
+	const uint32_t p = first + threadIdx.x;
+	const ofi_amd_tuner_variant_t v = variants[blockIdx.y];
+	const bool live = p < points_per_variant;
+	if (live) {
+		uint32_t r = p;
+		const uint32_t pi = r % g.n_ppn; r /= g.n_ppn;
+		const uint32_t ni = r % g.n_nodes; r /= g.n_nodes;
+		const uint32_t si = r % g.n_sizes; r /= g.n_sizes;
+		const uint32_t ci = r;
+		const uint64_t nodes = g.nodes[ni];
+		const uint64_t ranks = nodes * g.ppn[pi];
+		if (COST) {
+			const bool modelled = platform_has_model(v.platform);
+			for (uint32_t ai = 0; ai < g.n_algos; ai++) {
+				for (uint32_t proto = 0; proto < NUM_PROTOS; proto++) {
+					float c = -1.0f;
+					if (modelled) {
+						c = model_cost(v.platform, g.colls[ci], g.algos[ai], (int)proto, v.pipe_ops,
+							       g.sizes[si], ranks, nodes, g.log2_nodes[ni],
+							       v.num_channels, v.net_comp_overhead);
+					}
+					stage[threadIdx.x * cpp + ai * NUM_PROTOS + proto] = (double)c;
+				}
+			}
+		}
+		if (CHOICE) {
+			int algo, proto;
+			model_choose(v.platform, g.colls[ci], g.sizes[si], ranks, nodes, g.log2_nodes[ni], v.pipe_ops,
+				     v.num_channels, v.net_comp_overhead, kAllAllowed, algo, proto);
+			const uint64_t at = ((uint64_t)blockIdx.y * points_per_variant + p) * 2u;
+			choice[at + 0] = (int8_t)algo;
+			choice[at + 1] = (int8_t)proto;
+		}
 	}
-	uint64_t r = idx;
-	const uint32_t proto = (uint32_t)(r % NUM_PROTOS); r /= NUM_PROTOS;
-	const uint32_t ai = (uint32_t)(r % g.n_algos); r /= g.n_algos;
-	const uint32_t pi = (uint32_t)(r % g.n_ppn); r /= g.n_ppn;
-	const uint32_t ni = (uint32_t)(r % g.n_nodes); r /= g.n_nodes;
-	const uint32_t si = (uint32_t)(r % g.n_sizes); r /= g.n_sizes;
-	const uint32_t ci = (uint32_t)(r % g.n_colls); r /= g.n_colls;
-	const ofi_amd_tuner_variant_t v = variants[r];
-
-	const uint64_t nodes = g.nodes[ni];
-	const uint64_t ranks = nodes * g.ppn[pi];
-	float c = -1.0f;
-	if (platform_has_model(v.platform)) {
-		c = model_cost(v.platform, g.colls[ci], g.algos[ai], (int)proto, v.pipe_ops, g.sizes[si],
-			       ranks, nodes, g.log2_nodes[ni], v.num_channels, v.net_comp_overhead);
+	if (COST) {
+		__syncthreads();
+		const uint32_t valid = min(256u, points_per_variant - first);
+		double *out = cost + ((uint64_t)blockIdx.y * points_per_variant + first) * cpp;
+		for (uint32_t k = threadIdx.x; k < valid * cpp; k += 256u) {
+			__builtin_nontemporal_store(stage[k], &out[k]);
+		}
 	}
-	cost[idx] = (double)c;
 }
 
-/* One thread per decision point. */
-__global__ __launch_bounds__(256) void model_choice_kernel(grid_dims_t g,
-							   const ofi_amd_tuner_variant_t *__restrict__ variants,
-							   uint32_t n_variants, uint64_t points_per_variant,
-							   int8_t *__restrict__ choice)
-{
-	const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;
-	if (idx >= points_per_variant * n_variants) {
-		return;
-	}
-	uint64_t r = idx;
-	const uint32_t pi = (uint32_t)(r % g.n_ppn); r /= g.n_ppn;
-	const uint32_t ni = (uint32_t)(r % g.n_nodes); r /= g.n_nodes;
-	const uint32_t si = (uint32_t)(r % g.n_sizes); r /= g.n_sizes;
-	const uint32_t ci = (uint32_t)(r % g.n_colls); r /= g.n_colls;
-	const ofi_amd_tuner_variant_t v = variants[r];
-
-	const uint64_t nodes = g.nodes[ni];
-	int algo, proto;
-	model_choose(v.platform, g.colls[ci], g.sizes[si], nodes * g.ppn[pi], nodes, g.log2_nodes[ni],
-		     v.pipe_ops, v.num_channels, v.net_comp_overhead, kAllAllowed, algo, proto);
-	choice[idx * 2 + 0] = (int8_t)algo;
-	choice[idx * 2 + 1] = (int8_t)proto;
-}
-
-/* One thread per (platform, point). */
+/* One thread per point; blockIdx.y is the platform entry. */
 __global__ __launch_bounds__(256) void region_choice_kernel(grid_dims_t g, region_tables_t t,
 							    const int32_t *__restrict__ platforms,
-							    uint32_t n_platforms,
-							    uint64_t points_per_platform,
+							    uint32_t points_per_platform,
 							    int8_t *__restrict__ choice)
 {
-	const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;
-	if (idx >= points_per_platform * n_platforms) {
+	const uint32_t p = blockIdx.x * 256u + threadIdx.x;
+	if (p >= points_per_platform) {
 		return;
 	}
-	uint64_t r = idx;
-	const uint32_t pi = (uint32_t)(r % g.n_ppn); r /= g.n_ppn;
-	const uint32_t ni = (uint32_t)(r % g.n_nodes); r /= g.n_nodes;
-	const uint32_t si = (uint32_t)(r % g.n_sizes); r /= g.n_sizes;
-	const uint32_t ci = (uint32_t)(r % g.n_colls); r /= g.n_colls;
+	uint32_t r = p;
+	const uint32_t pi = r % g.n_ppn; r /= g.n_ppn;
+	const uint32_t ni = r % g.n_nodes; r /= g.n_nodes;
+	const uint32_t si = r % g.n_sizes; r /= g.n_sizes;
+	const uint32_t ci = r;
 
 	const uint64_t nodes = g.nodes[ni];
 	int algorithm, protocol, nchannels;
-	region_choose(t, platforms[r], g.colls[ci], g.sizes[si], nodes * g.ppn[pi], nodes,
+	region_choose(t, platforms[blockIdx.y], g.colls[ci], g.sizes[si], nodes * g.ppn[pi], nodes,
 		      pt_t{ g.log2_sizes[si], g.log2_ranks[ni * g.n_ppn + pi] }, kAllAllowed, algorithm,
 		      protocol, nchannels);
+	const uint64_t idx = (uint64_t)blockIdx.y * points_per_platform + p;
 	choice[idx * 4 + 0] = (int8_t)algorithm;
 	choice[idx * 4 + 1] = (int8_t)protocol;
 	*reinterpret_cast<int16_t *>(&choice[idx * 4 + 2]) = (int16_t)nchannels;
@@ -267,6 +272,9 @@ struct ofi_amd_tuner_plan {
 	ofi_amd_tuner_variant_t *d_variants;
 	int32_t *d_platforms;
 	uint32_t variants_cap, platforms_cap;
+	/* what d_variants currently holds, so that an unchanged list is not uploaded again */
+	std::vector<ofi_amd_tuner_variant_t> h_variants;
+	std::vector<int32_t> h_platforms;
 };
 
 using namespace ofi_amd;
@@ -330,7 +338,6 @@ int ofi_amd_tuner_plan_create(const int32_t *colls, uint32_t n_colls, const uint
 	if (!plan) {
 		return -ENOMEM;
 	}
-	std::memset(plan, 0, sizeof(*plan));
 	rc = device_region_tables(&plan->t);
 	if (rc != 0) {
 		delete plan;
@@ -413,23 +420,38 @@ int ofi_amd_tuner_model_grid(ofi_amd_tuner_plan_t *plan, const ofi_amd_tuner_var
 		(void)hipFree(plan->d_variants);
 		plan->d_variants = nullptr;
 		plan->variants_cap = 0;
+		plan->h_variants.clear();
 		OFI_AMD_HIP_TRY(hipMalloc((void **)&plan->d_variants, sizeof(*variants) * n_variants));
 		plan->variants_cap = n_variants;
 	}
-	OFI_AMD_HIP_TRY(hipMemcpyAsync(plan->d_variants, variants, sizeof(*variants) * n_variants,
-				       hipMemcpyHostToDevice, s));
-	if (d_cost) {
-		const uint64_t total = plan->cells * n_variants;
-		if (total > (1ull << 38)) {
-			return -EINVAL;
+	/* the variants travel to the device only when they differ from the last call's */
+	try {
+		if (plan->h_variants.size() != n_variants ||
+		    std::memcmp(plan->h_variants.data(), variants, sizeof(*variants) * n_variants) != 0) {
+			plan->h_variants.assign(variants, variants + n_variants);
+			OFI_AMD_HIP_TRY(hipMemcpyAsync(plan->d_variants, plan->h_variants.data(),
+						       sizeof(*variants) * n_variants, hipMemcpyHostToDevice, s));
+			/* the source is pageable host memory owned by the plan: wait until it has been read */
+			OFI_AMD_HIP_TRY(hipStreamSynchronize(s));
 		}
-		hipLaunchKernelGGL(model_cost_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0,
-				   s, plan->g, plan->d_variants, n_variants, plan->cells, d_cost);
+	} catch (...) {
+		return -ENOMEM;
 	}
-	if (d_choice) {
-		const uint64_t total = plan->points * n_variants;
-		hipLaunchKernelGGL(model_choice_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256),
-				   0, s, plan->g, plan->d_variants, n_variants, plan->points, d_choice);
+	if (plan->points > (1ull << 31) || plan->cells * n_variants > (1ull << 38) || n_variants > 65535) {
+		return -EINVAL;
+	}
+	const uint32_t points = (uint32_t)plan->points;
+	const dim3 grid((points + 255u) / 256u, n_variants);
+	const size_t lds = (size_t)256 * plan->g.n_algos * NUM_PROTOS * sizeof(double);
+	if (d_cost && d_choice) {
+		hipLaunchKernelGGL((model_grid_kernel<true, true>), grid, dim3(256), lds, s, plan->g,
+				   plan->d_variants, points, d_cost, d_choice);
+	} else if (d_cost) {
+		hipLaunchKernelGGL((model_grid_kernel<true, false>), grid, dim3(256), lds, s, plan->g,
+				   plan->d_variants, points, d_cost, d_choice);
+	} else if (d_choice) {
+		hipLaunchKernelGGL((model_grid_kernel<false, true>), grid, dim3(256), 0, s, plan->g,
+				   plan->d_variants, points, d_cost, d_choice);
 	}
 	OFI_AMD_HIP_TRY(hipGetLastError());
 	return 0;
@@ -456,14 +478,27 @@ int ofi_amd_tuner_region_grid(ofi_amd_tuner_plan_t *plan, const int32_t *platfor
 		(void)hipFree(plan->d_platforms);
 		plan->d_platforms = nullptr;
 		plan->platforms_cap = 0;
+		plan->h_platforms.clear();
 		OFI_AMD_HIP_TRY(hipMalloc((void **)&plan->d_platforms, sizeof(int32_t) * n_platforms));
 		plan->platforms_cap = n_platforms;
 	}
-	OFI_AMD_HIP_TRY(hipMemcpyAsync(plan->d_platforms, platforms, sizeof(int32_t) * n_platforms,
-				       hipMemcpyHostToDevice, s));
-	const uint64_t total = plan->points * n_platforms;
-	hipLaunchKernelGGL(region_choice_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, s,
-			   plan->g, plan->t, plan->d_platforms, n_platforms, plan->points, d_choice);
+	try {
+		if (plan->h_platforms.size() != n_platforms ||
+		    std::memcmp(plan->h_platforms.data(), platforms, sizeof(int32_t) * n_platforms) != 0) {
+			plan->h_platforms.assign(platforms, platforms + n_platforms);
+			OFI_AMD_HIP_TRY(hipMemcpyAsync(plan->d_platforms, plan->h_platforms.data(),
+						       sizeof(int32_t) * n_platforms, hipMemcpyHostToDevice, s));
+			OFI_AMD_HIP_TRY(hipStreamSynchronize(s));
+		}
+	} catch (...) {
+		return -ENOMEM;
+	}
+	if (plan->points > (1ull << 31) || n_platforms > 65535) {
+		return -EINVAL;
+	}
+	const uint32_t points = (uint32_t)plan->points;
+	hipLaunchKernelGGL(region_choice_kernel, dim3((points + 255u) / 256u, n_platforms), dim3(256), 0, s,
+			   plan->g, plan->t, plan->d_platforms, points, d_choice);
 	OFI_AMD_HIP_TRY(hipGetLastError());
 	return 0;
 }
