@@ -252,12 +252,6 @@ __device__ inline double seg_distance(pt_t x, pt_t y0, pt_t y1, double eps)
 __device__ inline int inside_region(pt_t point, const pt_t *v, int n, pt_t far_point)
 {
 	const double eps = 1e-10;
-	for (int i = 0; i < n; i++) {
-		int k = (i + 1) % n;
-		if (seg_distance(point, v[i], v[k], eps) < eps) {
-			return 0;
-		}
-	}
 	/* y bounds start from vertex 1 as in the reference (:177-178) */
 	double min_x = v[0].x, max_x = v[0].x, min_y = v[1].y, max_y = v[1].y;
 	for (int i = 0; i < n; i++) {
@@ -265,6 +259,23 @@ __device__ inline int inside_region(pt_t point, const pt_t *v, int n, pt_t far_p
 		if (v[i].x < min_x) min_x = v[i].x;
 		if (v[i].y > max_y) max_y = v[i].y;
 		if (v[i].y < min_y) min_y = v[i].y;
+	}
+	/* The reference looks for a point on an edge first (result 0) and rejects by bounding
+	 * box second (result -1).  A point more than 1e-6 outside the box cannot be within
+	 * 1e-10 of an edge -- edges lie inside the box, and the foot of the perpendicular may
+	 * leave the segment by at most eps times its length -- so for such a point the second
+	 * answer is known without the per-edge divisions and square roots.  Most polygons are
+	 * dismissed here. */
+	const double margin = 1e-6;
+	if (point.x < min_x - margin || point.x > max_x + margin || point.y < min_y - margin ||
+	    point.y > max_y + margin) {
+		return -1;
+	}
+	for (int i = 0; i < n; i++) {
+		int k = (i + 1) % n;
+		if (seg_distance(point, v[i], v[k], eps) < eps) {
+			return 0;
+		}
 	}
 	if (point.x < min_x || point.x > max_x || point.y < min_y || point.y > max_y) {
 		return -1;

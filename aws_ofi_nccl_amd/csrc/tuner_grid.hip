@@ -98,15 +98,21 @@ __global__ __launch_bounds__(256) void region_choice_kernel(grid_dims_t g, regio
 							    uint32_t points_per_platform,
 							    int8_t *__restrict__ choice)
 {
-	const uint32_t p = blockIdx.x * 256u + threadIdx.x;
-	if (p >= points_per_platform) {
+	const uint32_t t_idx = blockIdx.x * 256u + threadIdx.x;
+	if (t_idx >= points_per_platform) {
 		return;
 	}
-	uint32_t r = p;
-	const uint32_t pi = r % g.n_ppn; r /= g.n_ppn;
+	/* Threads are laid out with the node count fastest, then the size, then ranks per node,
+	 * then the collective -- not in output order.  Which polygon set a point is tested
+	 * against depends on (collective, ranks per node): this way the lanes of a wavefront
+	 * walk the same polygons instead of serialising over up to four different sets (and
+	 * whole wavefronts of shapes without regions leave at once). */
+	uint32_t r = t_idx;
 	const uint32_t ni = r % g.n_nodes; r /= g.n_nodes;
 	const uint32_t si = r % g.n_sizes; r /= g.n_sizes;
+	const uint32_t pi = r % g.n_ppn; r /= g.n_ppn;
 	const uint32_t ci = r;
+	const uint32_t p = ((ci * g.n_sizes + si) * g.n_nodes + ni) * g.n_ppn + pi; /* output order */
 
 	const uint64_t nodes = g.nodes[ni];
 	int algorithm, protocol, nchannels;
