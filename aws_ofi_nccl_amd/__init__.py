@@ -80,6 +80,13 @@ class GinDevRing(ctypes.Structure):
                 ("capacity", c_u32), ("context", c_u32)]
 
 
+class GinLoopbackStats(ctypes.Structure):
+    """ofi_amd_gin_loopback_stats_t"""
+    _fields_ = [("descriptors", c_u64), ("writes", c_u64), ("copy_entries", c_u64), ("bytes", c_u64),
+                ("signals", c_u64), ("work_items", c_u64), ("acks", c_u64), ("launches", c_u64),
+                ("seconds", ctypes.c_double)]
+
+
 class GinSignalWork(ctypes.Structure):
     """ofi_amd_gin_signal_work_t (32 bytes)"""
     _fields_ = [("base", c_u64), ("offset", c_u64), ("value", c_u64), ("peer", c_u32),
@@ -217,6 +224,9 @@ PROTOTYPES = {
                                               c_vp]),
     "ofi_amd_eager_copy_batch": (ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_u32, c_vp, c_vp,
                                                 c_vp]),
+    "ofi_amd_copy_table": (ctypes.c_int, [c_vp, c_vp, c_vp, c_u32, c_vp]),
+    "ofi_amd_gin_loopback_run": (ctypes.c_int, [c_vp, c_u64, c_vp, c_vp, ctypes.POINTER(GinSignalRegion), c_u32,
+                                                c_u32, c_u32, c_u32, c_vp, ctypes.POINTER(GinLoopbackStats)]),
     "ofi_amd_flush_buffer_fill": (ctypes.c_int, [c_vp, c_u64, c_vp]),
     "ofi_amd_flush_post": (ctypes.c_int, [c_vp, c_vp, c_u32, c_vp]),
     "ofi_amd_flush_test": (ctypes.c_int, [c_vp, c_u32, c_u64]),

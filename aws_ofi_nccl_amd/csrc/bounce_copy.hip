@@ -199,11 +199,42 @@ __global__ __launch_bounds__(kBlock) void bounce_scatter_kernel(
 }
 
 /*
+ * bytes from s to d, neither aligned: the bytes in front of the first 16-byte boundary of the
+ * destination go out singly; from there on it is the aligned-destination copy above, with
+ * whatever source alignment that leaves.  Wave-collective.
+ */
+__device__ __forceinline__ void copy_any(const uint8_t *__restrict__ s, uint8_t *__restrict__ d,
+					 uint32_t bytes, uint32_t lane)
+{
+	if (bytes == 0) {
+		return;
+	}
+	const uint32_t head = min(bytes, (16u - (uint32_t)(reinterpret_cast<uintptr_t>(d) & 15u)) & 15u);
+	/* lanes without a head byte re-copy byte 0: same value, same place */
+	const uint32_t head_at = min(lane, max(head, 1u) - 1u);
+	const uint8_t head_byte = s[head_at];
+	const uint32_t rem = bytes - head;
+	if (rem != 0) {
+		const uint8_t *s2 = s + head;
+		uint8_t *d2 = d + head;
+		const uint32_t nvec = rem >> 4;
+		const uint32_t tail_at = min((nvec << 4) + lane, rem - 1u);
+		const uint8_t tail_byte = s2[tail_at];
+		const uint32_t shift = (uint32_t)(reinterpret_cast<uintptr_t>(s2) & 3u);
+		if (shift == 0) {
+			copy_words<false>(s2, d2, nvec, 0, lane);
+		} else {
+			copy_words<true>(s2 - shift, d2, nvec, shift, lane);
+		}
+		d2[tail_at] = tail_byte;
+	}
+	d[head_at] = head_byte;
+}
+
+/*
  * The same copy for eager arrivals as they sit in rx buffers: an 8-byte header, then the
  * payload, which goes to a receive buffer at any alignment, truncated to that buffer's
- * length (rdma_eager_copy_req::post, src/nccl_ofi_rdma.cpp:2729-2776).  The bytes in front
- * of the first 16-byte boundary of the destination go out singly; from there on it is the
- * aligned-destination copy above, with whatever source alignment that leaves.
+ * length (rdma_eager_copy_req::post, src/nccl_ofi_rdma.cpp:2729-2776).
  */
 __global__ __launch_bounds__(kBlock) void eager_copy_kernel(
 	const uint8_t *__restrict__ rx_base, const uint64_t *__restrict__ rx_off,
@@ -227,28 +258,7 @@ __global__ __launch_bounds__(kBlock) void eager_copy_kernel(
 		copied[buf] = bytes;
 	}
 
-	if (bytes != 0) {
-		const uint32_t head = min(bytes, (16u - (uint32_t)(reinterpret_cast<uintptr_t>(d) & 15u)) & 15u);
-		/* lanes without a head byte re-copy byte 0: same value, same place */
-		const uint32_t head_at = min(lane, max(head, 1u) - 1u);
-		const uint8_t head_byte = s[head_at];
-		const uint32_t rem = bytes - head;
-		if (rem != 0) {
-			const uint8_t *s2 = s + head;
-			uint8_t *d2 = d + head;
-			const uint32_t nvec = rem >> 4;
-			const uint32_t tail_at = min((nvec << 4) + lane, rem - 1u);
-			const uint8_t tail_byte = s2[tail_at];
-			const uint32_t shift = (uint32_t)(reinterpret_cast<uintptr_t>(s2) & 3u);
-			if (shift == 0) {
-				copy_words<false>(s2, d2, nvec, 0, lane);
-			} else {
-				copy_words<true>(s2 - shift, d2, nvec, shift, lane);
-			}
-			d2[tail_at] = tail_byte;
-		}
-		d[head_at] = head_byte;
-	}
+	copy_any(s, d, bytes, lane);
 
 	if (flush != nullptr) {
 		__builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
@@ -263,6 +273,21 @@ __global__ __launch_bounds__(kBlock) void eager_copy_kernel(
 			flush[buf] = word;
 		}
 	}
+}
+
+/* One wavefront per (source address, destination address, length) entry. */
+__global__ __launch_bounds__(kBlock) void copy_table_kernel(const uint64_t *__restrict__ src_addr,
+							     const uint64_t *__restrict__ dst_addr,
+							     const uint32_t *__restrict__ len, uint32_t n)
+{
+	const uint32_t lane = threadIdx.x & 63u;
+	const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const uint32_t i = blockIdx.x * kWavesPerBlock + wave;
+	if (i >= n) {
+		return;
+	}
+	copy_any(reinterpret_cast<const uint8_t *>(src_addr[i]), reinterpret_cast<uint8_t *>(dst_addr[i]), len[i],
+		 lane);
 }
 
 __global__ __launch_bounds__(256) void flush_read_kernel(const uint8_t *__restrict__ arena,
@@ -361,6 +386,25 @@ int ofi_amd_eager_copy_batch(const void *rx_base, const uint64_t *d_rx_off, cons
 	hipLaunchKernelGGL(eager_copy_kernel, dim3(blocks), dim3(kBlock), 0, as_stream(stream),
 			   static_cast<const uint8_t *>(rx_base), d_rx_off, d_recv_len,
 			   static_cast<uint8_t *>(dst_base), d_dst_off, d_dst_len, n, d_copied, d_flush);
+	OFI_AMD_HIP_TRY(hipGetLastError());
+	return 0;
+}
+
+int ofi_amd_copy_table(const uint64_t *d_src_addr, const uint64_t *d_dst_addr, const uint32_t *d_len,
+		       uint32_t n, void *stream)
+{
+	int rc = require_device();
+	if (rc != 0) {
+		return rc;
+	}
+	if (n == 0) {
+		return 0;
+	}
+	if (!d_src_addr || !d_dst_addr || !d_len || n > (1u << 30)) {
+		return -EINVAL;
+	}
+	hipLaunchKernelGGL(copy_table_kernel, dim3((n + kWavesPerBlock - 1) / kWavesPerBlock), dim3(kBlock), 0,
+			   as_stream(stream), d_src_addr, d_dst_addr, d_len, n);
 	OFI_AMD_HIP_TRY(hipGetLastError());
 	return 0;
 }

@@ -1,0 +1,334 @@
+/*
+ * In-process loop-back of the GIN path on one GPU (ofi_amd_gin_loopback_run): descriptors
+ * produced on the device are drained, turned into wire records, "transmitted" -- the RDMA
+ * writes become device-side copies, the completions and metadata messages go to a receiver,
+ * its ACKs come back to the sender -- and the released signals are applied to the counters
+ * in HBM.  It composes the library's own entry points and stands where the reference has
+ * two processes, a libfabric provider and GDRCopy (tests/functional/rma.cpp,
+ * src/rdma/gin/nccl_ofi_gin.cpp:568-864 on the initiator, :1622-1924 on the target).
+ */
+#include <cerrno>
+#include <chrono>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "gin_rings.hpp"
+
+namespace {
+
+constexpr uint32_t kPiece = 64u << 10; /* long writes are cut so that no wavefront copies more */
+constexpr uint64_t kSentinel = 0xdeadbeefdeadbeefull; /* NCCL_OFI_GIN_FLUSH_SENTINEL_VAL */
+
+/* One launch pair's worth of copies and signal work, in pinned host memory the GPU reads in place. */
+struct batch_t {
+	uint64_t *src = nullptr, *dst = nullptr;
+	uint32_t *len = nullptr;
+	ofi_amd_gin_signal_work_t *work = nullptr;
+	void *d_src = nullptr, *d_dst = nullptr, *d_len = nullptr, *d_work = nullptr;
+	/* one 64-byte flush slot: the sentinel arrives here when the batch's launches are done */
+	uint64_t *done_slot = nullptr;
+	void *d_done_slot = nullptr;
+	uint32_t n_copy = 0, n_work = 0;
+	bool launched = false;
+};
+
+int alloc_pinned(void **host, void **dev, size_t bytes)
+{
+	int rc = ofi_amd_gpu_host_alloc(host, bytes);
+	if (rc != 0) {
+		return rc;
+	}
+	return ofi_amd_gpu_host_get_device_pointer(dev, *host);
+}
+
+void free_batch(batch_t &b)
+{
+	if (b.src) (void)ofi_amd_gpu_host_free(b.src);
+	if (b.dst) (void)ofi_amd_gpu_host_free(b.dst);
+	if (b.len) (void)ofi_amd_gpu_host_free(b.len);
+	if (b.work) (void)ofi_amd_gpu_host_free(b.work);
+	if (b.done_slot) (void)ofi_amd_gpu_host_free(b.done_slot);
+	b = batch_t();
+}
+
+int alloc_batch(batch_t &b, uint32_t cap_copy, uint32_t cap_work)
+{
+	int rc = alloc_pinned(reinterpret_cast<void **>(&b.src), &b.d_src, sizeof(uint64_t) * cap_copy);
+	if (rc == 0) rc = alloc_pinned(reinterpret_cast<void **>(&b.dst), &b.d_dst, sizeof(uint64_t) * cap_copy);
+	if (rc == 0) rc = alloc_pinned(reinterpret_cast<void **>(&b.len), &b.d_len, sizeof(uint32_t) * cap_copy);
+	if (rc == 0) rc = alloc_pinned(reinterpret_cast<void **>(&b.work), &b.d_work, sizeof(*b.work) * cap_work);
+	if (rc == 0) rc = alloc_pinned(reinterpret_cast<void **>(&b.done_slot), &b.d_done_slot, 64);
+	if (rc == 0) std::memset(b.done_slot, 0, 64);
+	return rc;
+}
+
+/* A completion on its way from the "NIC" to the receiver. */
+struct event_t {
+	uint32_t peer;
+	uint32_t is_meta;
+	uint32_t imm;
+	uint64_t meta[4];
+};
+
+struct lcg_t {
+	uint64_t s;
+	uint32_t next(uint32_t n)
+	{
+		s = s * 6364136223846793005ull + 1442695040888963407ull;
+		return (uint32_t)((s >> 33) % n);
+	}
+};
+
+} // namespace
+
+extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per_context,
+					ofi_amd_gin_comm_t *comms, const ofi_amd_gin_mr_t *mrs,
+					const ofi_amd_gin_signal_region_t *regions, uint32_t n_regions,
+					uint32_t reorder_window, uint32_t batch_writes, uint32_t timeout_ms,
+					void *stream, ofi_amd_gin_loopback_stats_t *stats)
+{
+	if (!r || !comms || !mrs || !regions || n_regions == 0 || batch_writes == 0 ||
+	    batch_writes > (1u << 24) || reorder_window > 2048) {
+		return -EINVAL;
+	}
+	using clock = std::chrono::steady_clock;
+	const uint32_t nctx = r->n_contexts;
+	/* an op adds at most 4 writes of at most ... pieces; a flush is forced when either table
+	 * cannot take one more op's worth */
+	const uint32_t cap_copy = batch_writes + 4096, cap_work = batch_writes + 64;
+
+	ofi_amd_gin_loopback_stats_t st;
+	std::memset(&st, 0, sizeof(st));
+	batch_t batches[2];
+	ofi_amd_gin_rx_t *rx = nullptr;
+	std::vector<uint32_t> comm_ids;
+	std::vector<event_t> in_flight;
+	std::vector<uint64_t> done;
+	int rc = 0;
+	try {
+		comm_ids.resize(nctx);
+		done.assign(nctx, 0);
+		in_flight.reserve(reorder_window + 8);
+	} catch (...) {
+		return -ENOMEM;
+	}
+	for (uint32_t c = 0; c < nctx; c++) {
+		comm_ids[c] = comms[c].comm_id;
+	}
+	/* completion of a batch is observed the reference's way: a sentinel flush read back into a
+	 * host slot behind the batch's launches (iflush, src/rdma/gin/nccl_ofi_gin.cpp:941-1003) */
+	void *d_flush_buf = nullptr;
+	rc = ofi_amd_gin_rx_create(nctx, comm_ids.data(), &rx);
+	for (int b = 0; b < 2 && rc == 0; b++) {
+		rc = alloc_batch(batches[b], cap_copy, cap_work);
+	}
+	if (rc == 0) rc = ofi_amd_gpu_mem_alloc(&d_flush_buf, 64);
+	if (rc == 0) rc = ofi_amd_flush_buffer_fill(d_flush_buf, kSentinel, stream);
+	auto release = [&]() {
+		free_batch(batches[0]);
+		free_batch(batches[1]);
+		if (d_flush_buf) (void)ofi_amd_gpu_mem_free(d_flush_buf);
+		if (rx) (void)ofi_amd_gin_rx_destroy(rx);
+	};
+	if (rc != 0) {
+		release();
+		return rc;
+	}
+
+	int cur = 0;
+	lcg_t rng{ 0x9E3779B97F4A7C15ull };
+	ofi_amd_gin_ack_t acks[64];
+
+	/* copies first, then the signals that were released while they were queued */
+	auto flush = [&]() -> int {
+		batch_t &b = batches[cur];
+		if (b.n_copy == 0 && b.n_work == 0) {
+			return 0;
+		}
+		int e = 0;
+		if (b.n_copy) {
+			e = ofi_amd_copy_table(static_cast<const uint64_t *>(b.d_src), static_cast<const uint64_t *>(b.d_dst),
+					       static_cast<const uint32_t *>(b.d_len), b.n_copy, stream);
+		}
+		if (e == 0 && b.n_work) {
+			e = ofi_amd_gin_signal_apply(static_cast<const ofi_amd_gin_signal_work_t *>(b.d_work), b.n_work,
+						     regions, n_regions, nullptr, stream);
+		}
+		if (e == 0) {
+			__atomic_store_n(&b.done_slot[0], 0ull, __ATOMIC_RELEASE);
+			e = ofi_amd_flush_post(d_flush_buf, b.d_done_slot, 1, stream);
+		}
+		if (e != 0) {
+			return e;
+		}
+		st.launches++;
+		st.copy_entries += b.n_copy;
+		st.work_items += b.n_work;
+		b.launched = true;
+		cur ^= 1;
+		batch_t &next = batches[cur];
+		if (next.launched) {
+			/* its tables may still be read by the launches before last: wait for its sentinel
+			 * (not for the stream: the batch just launched keeps running meanwhile) */
+			const auto w0 = clock::now();
+			while (ofi_amd_flush_test(next.done_slot, 1, kSentinel) != 1) {
+				if (std::chrono::duration_cast<std::chrono::milliseconds>(clock::now() - w0).count() >
+				    (long long)timeout_ms) {
+					return -ETIMEDOUT;
+				}
+			}
+			next.launched = false;
+		}
+		next.n_copy = next.n_work = 0;
+		return 0;
+	};
+
+	/* hands one completion to the receiver and collects what that releases */
+	auto deliver = [&](const event_t &ev) -> int {
+		int e = ev.is_meta ? ofi_amd_gin_rx_metadata(rx, ev.peer, ev.meta)
+				   : ofi_amd_gin_rx_write_completion(rx, ev.peer, ev.imm);
+		if (e != 0) {
+			return e;
+		}
+		for (;;) {
+			const uint32_t n = ofi_amd_gin_rx_take_acks(rx, acks, 64);
+			for (uint32_t i = 0; i < n; i++) {
+				ofi_amd_gin_apply_ack(&comms[acks[i].peer], acks[i].rx_consumed);
+			}
+			st.acks += n;
+			if (n < 64) {
+				break;
+			}
+		}
+		for (;;) {
+			batch_t &b = batches[cur];
+			const uint32_t n = ofi_amd_gin_rx_take_work(rx, b.work + b.n_work, cap_work - b.n_work);
+			b.n_work += n;
+			if (b.n_work < cap_work) {
+				break;
+			}
+			e = flush();
+			if (e != 0) {
+				return e;
+			}
+		}
+		return 0;
+	};
+
+	auto deliver_some = [&](uint32_t keep) -> int {
+		while (in_flight.size() > keep) {
+			const uint32_t k = rng.next((uint32_t)in_flight.size());
+			const event_t ev = in_flight[k];
+			in_flight[k] = in_flight.back();
+			in_flight.pop_back();
+			int e = deliver(ev);
+			if (e != 0) {
+				return e;
+			}
+		}
+		return 0;
+	};
+
+	const auto t0 = clock::now();
+	auto last_progress = t0;
+	uint64_t remaining = (uint64_t)nctx * ops_per_context;
+	uint32_t idle = 0;
+	while (remaining > 0 && rc == 0) {
+		bool progressed = false;
+		for (uint32_t c = 0; c < nctx && rc == 0; c++) {
+			for (uint32_t burst = 0; burst < 256 && done[c] < ops_per_context; burst++) {
+				ofi_amd_gin_desc_t d;
+				if (ofi_amd_gin_ring_pop(r, c, &d) != 1) {
+					break;
+				}
+				ofi_amd_gin_wire_t wire;
+				rc = ofi_amd_gin_iput_signal(&comms[c], mrs, &d, &wire);
+				if (rc == -EAGAIN) {
+					/* window closed: let everything in flight arrive, which brings the ACKs */
+					rc = deliver_some(0);
+					if (rc == 0) {
+						rc = ofi_amd_gin_iput_signal(&comms[c], mrs, &d, &wire);
+					}
+				}
+				if (rc != 0) {
+					break;
+				}
+				if (batches[cur].n_copy + 4u * (uint32_t)(((uint64_t)d.size >> 16) + 2u) > cap_copy) {
+					rc = flush();
+					if (rc != 0) {
+						break;
+					}
+				}
+				batch_t &b = batches[cur];
+				for (uint32_t k = 0; k < wire.num_writes; k++) {
+					const ofi_amd_gin_write_t &w = wire.writes[k];
+					for (uint64_t off = 0; off < w.len; off += kPiece) {
+						if (b.n_copy == cap_copy) {
+							rc = -EMSGSIZE; /* an op larger than the table: raise batch_writes */
+							break;
+						}
+						const uint64_t n = w.len - off < kPiece ? w.len - off : kPiece;
+						b.src[b.n_copy] = w.src + off;
+						b.dst[b.n_copy] = w.dest + off;
+						b.len[b.n_copy] = (uint32_t)n;
+						b.n_copy++;
+					}
+					st.bytes += w.len;
+					event_t ev;
+					std::memset(&ev, 0, sizeof(ev));
+					ev.peer = c;
+					ev.imm = wire.imm;
+					in_flight.push_back(ev);
+				}
+				if (rc != 0) {
+					break;
+				}
+				st.writes += wire.num_writes;
+				if (wire.has_meta) {
+					event_t ev;
+					std::memset(&ev, 0, sizeof(ev));
+					ev.peer = c;
+					ev.is_meta = 1;
+					std::memcpy(ev.meta, wire.meta, sizeof(ev.meta));
+					in_flight.push_back(ev);
+					st.signals++;
+				}
+				rc = deliver_some(reorder_window);
+				if (rc == 0 && batches[cur].n_copy >= batch_writes) {
+					rc = flush();
+				}
+				done[c]++;
+				remaining--;
+				st.descriptors++;
+				progressed = true;
+			}
+		}
+		if (progressed) {
+			idle = 0;
+			last_progress = clock::now();
+		} else if (++idle >= 64) {
+			idle = 0;
+			if (std::chrono::duration_cast<std::chrono::milliseconds>(clock::now() - last_progress).count() >
+			    (long long)timeout_ms) {
+				rc = -ETIMEDOUT;
+			}
+		}
+	}
+	if (rc == 0) {
+		rc = deliver_some(0);
+	}
+	if (rc == 0) {
+		rc = flush();
+	}
+	int sync_rc = ofi_amd_gpu_stream_synchronize(stream);
+	if (rc == 0) {
+		rc = sync_rc;
+	}
+	st.seconds = std::chrono::duration<double>(clock::now() - t0).count();
+	if (stats) {
+		*stats = st;
+	}
+	release();
+	return rc;
+}

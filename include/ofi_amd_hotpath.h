@@ -149,6 +149,16 @@ int ofi_amd_eager_copy_batch(const void *rx_base, const uint64_t *d_rx_off, cons
 			     void *dst_base, const uint64_t *d_dst_off, const uint32_t *d_dst_len,
 			     uint32_t n, uint32_t *d_copied, uint32_t *d_flush, void *stream);
 
+/*
+ * The general form: entry i copies d_len[i] bytes from address d_src_addr[i] to address
+ * d_dst_addr[i] (any device-accessible addresses, any alignment, ranges of one batch
+ * disjoint), one wavefront per entry.  This is the data movement of a batch of RDMA writes
+ * whose source and target live on the same device -- what a loop-back provider does for
+ * fi_writemsg (src/rdma/gin/nccl_ofi_gin_reqs.cpp:244-310).  Tables are device-accessible.
+ */
+int ofi_amd_copy_table(const uint64_t *d_src_addr, const uint64_t *d_dst_addr, const uint32_t *d_len,
+		       uint32_t n, void *stream);
+
 /* Flush only: d_flush[i] = 4 bytes at d_arena + d_dst_off[i], read with
  * device-scope acquire semantics (the C5 read-back without a copy). */
 int ofi_amd_flush_read(const void *d_arena, const uint64_t *d_dst_off, uint32_t n,
@@ -435,6 +445,43 @@ typedef struct {
 int ofi_amd_gin_signal_apply(const ofi_amd_gin_signal_work_t *d_work, uint32_t n,
 			     const ofi_amd_gin_signal_region_t *regions, uint32_t n_regions,
 			     uint32_t *d_rejected, void *stream);
+
+/*
+ * In-process loop-back of the whole GIN path on one GPU: initiator and target are the same
+ * device, the "network" is this call.  For every descriptor drained from the rings it
+ *   1. derives the wire record (ofi_amd_gin_iput_signal on comms[context], ack_model 0),
+ *   2. queues each RDMA write as a (source, destination, length) copy -- source
+ *      mrs[src_mr].local_base + src_off, destination the write's `dest` (give the
+ *      destination MR's remote_address_offset the device address of the target buffer) --
+ *      long writes cut into 64 KiB pieces,
+ *   3. delivers the write completions and the metadata message to a receiver
+ *      (ofi_amd_gin_rx_*, one peer per context), up to reorder_window events out of order,
+ *   4. returns the receiver's ACKs to the sender (ofi_amd_gin_apply_ack),
+ * and every batch_writes queued copies (and at the end) launches, in this order on `stream`,
+ * ofi_amd_copy_table for the copies and ofi_amd_gin_signal_apply for the signals the
+ * receiver has released: a signal is applied after the payloads it covers.  `stream` must
+ * not be the stream the producing kernel runs on (that kernel waits for this call to drain
+ * its rings; work queued behind it would never start).  What the
+ * reference does with two processes, libfabric and GDRCopy (tests/functional/rma.cpp), runs
+ * here as GPU producer -> host proxy -> GPU copy and atomics.
+ */
+typedef struct {
+	uint64_t descriptors;
+	uint64_t writes;          /* RDMA writes derived */
+	uint64_t copy_entries;    /* after cutting long writes */
+	uint64_t bytes;           /* payload bytes moved */
+	uint64_t signals;         /* put-signal operations */
+	uint64_t work_items;      /* folded signal deliveries applied */
+	uint64_t acks;            /* ACKs returned to the senders */
+	uint64_t launches;        /* copy + apply launch pairs */
+	double seconds;
+} ofi_amd_gin_loopback_stats_t;
+
+int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *rings, uint64_t ops_per_context,
+			     ofi_amd_gin_comm_t *comms, const ofi_amd_gin_mr_t *mrs,
+			     const ofi_amd_gin_signal_region_t *regions, uint32_t n_regions,
+			     uint32_t reorder_window, uint32_t batch_writes, uint32_t timeout_ms,
+			     void *stream, ofi_amd_gin_loopback_stats_t *stats);
 
 /* ======================================================================
  * 5. Tuner: batched cost model and region lookup.

@@ -1,0 +1,161 @@
+"""The GIN path end to end on one GPU, in process: device-side puts -> rings -> host proxy ->
+wire records -> (loop-back "network": RDMA writes become device copies, completions and
+metadata go to the receiver out of order, ACKs return) -> signal counters in HBM.
+
+What the reference checks with two processes and a NIC (tests/functional/rma.cpp: payload
+bytes and signal counters at the target) is checked here bit for bit against a plain numpy
+replay of the same operations; the wire-level bookkeeping must also close: every op
+retired, every signal delivered once, the sender's window never stuck."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import _gpu
+import aws_ofi_nccl_amd as m
+
+pytestmark = pytest.mark.gpu
+
+SIG_BASE = 0x7F5500000000
+N_SLOTS = 64
+
+
+def build_ops(rng, nctx, ops, src_bytes, max_size):
+    """table[ctx][i] of 8 u64 words (ofi_amd_gin_desc_t) with disjoint destinations"""
+    table = np.zeros((nctx, ops, 8), dtype=np.uint64)
+    dst_pos = 0
+    replay = []
+    for c in range(nctx):
+        for i in range(ops):
+            kind = rng.random()
+            if kind < 0.08:
+                size = 0                                           # signal only
+            elif kind < 0.6:
+                size = int(rng.integers(1, 4096))
+            else:
+                size = int(2 ** rng.uniform(3, np.log2(max_size)))
+            src_off = int(rng.integers(0, src_bytes - size))
+            dst_off = dst_pos + int(rng.integers(0, 24))           # arbitrary alignment
+            dst_pos = dst_off + size + int(rng.integers(0, 8))
+            signal = size == 0 or (i % 5) == 4
+            sop = (1 if rng.random() < 0.5 else 2) if signal else 0
+            sval = int(rng.integers(1, 1 << 40)) if sop == 2 else 0
+            slot = int(rng.integers(0, N_SLOTS))
+            flags = int(rng.integers(0, 2))                        # doorbell aggregation hint
+            table[c, i] = [src_off, dst_off, size, 8 * slot if sop else 0, sval,
+                           1 | (sop << 32), flags | (c << 32),
+                           0 | (1 << 16) | ((2 if sop else 0xFFFF) << 32) | ((2 if sop else 1) << 48)]
+            replay.append((src_off, dst_off, size, sop, sval, slot))
+    return table, replay, dst_pos + 64
+
+
+@pytest.mark.parametrize("nctx,ops,waves,reorder,batch,max_size", [
+    (1, 300, 1, 0, 64, 70_000),
+    (4, 1500, 3, 37, 512, 300_000),
+    (3, 6000, 2, 500, 4096, 40_000),      # more than 4096 ops per context in flight at times: ACKs matter
+])
+def test_puts_and_signals_arrive_bit_exact(lib, gpu, nctx, ops, waves, reorder, batch, max_size):
+    rng = np.random.default_rng(nctx * 1000 + ops)
+    src_bytes = 32 << 20
+    src = rng.integers(0, 256, src_bytes, dtype=np.uint8)
+    table, replay, dst_bytes = build_ops(rng, nctx, ops, src_bytes, max_size)
+    d_src = _gpu.to_dev(src)
+    d_dst = torch.full((dst_bytes,), 0xEE, dtype=torch.uint8, device="cuda")
+    start = rng.integers(0, 1 << 63, N_SLOTS, dtype=np.uint64)
+    d_cnt = _gpu.to_dev(start)
+    d_table = _gpu.to_dev(table)
+
+    mrs = (m.GinMr * 3)()
+    mrs[0].local_base = d_src.data_ptr()                       # source MR: local address
+    mrs[1].remote_address_offset = d_dst.data_ptr()            # target MR: where writes land
+    mrs[2].remote_address = SIG_BASE                           # signal MR: the address the peer knows
+    for i in range(3):
+        for r in range(4):
+            mrs[i].key[r] = 0x100 * (i + 1) + r
+    comms = (m.GinComm * nctx)()
+    for c in range(nctx):
+        assert lib.ofi_amd_gin_comm_init(ctypes.byref(comms[c]), 100 + c, 4, 131072, 64, 0) == 0
+    regions = (m.GinSignalRegion * 1)(m.GinSignalRegion(SIG_BASE, 8 * N_SLOTS, d_cnt.data_ptr()))
+    rings = ctypes.c_void_p()
+    assert lib.ofi_amd_gin_rings_create(nctx, 1024, ctypes.byref(rings)) == 0
+
+    assert lib.ofi_amd_gin_produce_table(rings, d_table.data_ptr(), ops, waves, 0, _gpu.stream()) == 0
+    stats = m.GinLoopbackStats()
+    # the copies and signal updates go on their own stream: the producer kernel occupies the first
+    side = torch.cuda.Stream()
+    rc = lib.ofi_amd_gin_loopback_run(rings, ops, ctypes.cast(comms, ctypes.c_void_p),
+                                      ctypes.cast(mrs, ctypes.c_void_p), regions, 1, reorder, batch, 20000,
+                                      ctypes.c_void_p(side.cuda_stream), ctypes.byref(stats))
+    torch.cuda.synchronize()
+    assert rc == 0 and lib.ofi_amd_gin_producer_status(rings) == 0
+
+    # payload: a plain replay of the puts on the host
+    want = np.full(dst_bytes, 0xEE, dtype=np.uint8)
+    counters = [int(x) for x in start]
+    n_signals = 0
+    for src_off, dst_off, size, sop, sval, slot in replay:
+        want[dst_off:dst_off + size] = src[src_off:src_off + size]
+        if sop:
+            counters[slot] = (counters[slot] + (1 if sop == 1 else sval)) % (1 << 64)
+            n_signals += 1
+    assert np.array_equal(d_dst.cpu().numpy(), want)
+    assert [int(x) for x in _gpu.to_host(d_cnt, np.uint64)] == counters
+
+    # bookkeeping closes
+    total = nctx * ops
+    assert stats.descriptors == total and stats.signals == n_signals
+    assert stats.bytes == sum(r[2] for r in replay)
+    assert stats.writes >= sum(1 for r in replay if r[2]) and stats.copy_entries >= stats.writes
+    assert 0 < stats.work_items <= n_signals          # same-slot neighbours may have been folded
+    for c in range(nctx):
+        assert comms[c].tx_head == ops % 16384
+        outstanding = (comms[c].tx_head - comms[c].tx_tail) & 0x3FFF
+        assert outstanding < 8192
+        if ops > 4096 + 64:
+            assert outstanding < ops                  # ACKs did come back
+    if ops > 4096 + 64:
+        assert stats.acks > 0
+    assert _gpu.fetch_async_errors(lib) == 0
+    lib.ofi_amd_gin_rings_destroy(rings)
+
+
+def test_copy_table_matches_a_host_replay(lib, gpu):
+    """The loop-back's data mover by itself: address triples at any alignment and length."""
+    rng = np.random.default_rng(5)
+    n = 3000
+    src = rng.integers(0, 256, 8 << 20, dtype=np.uint8)
+    lens = np.concatenate([rng.integers(0, 300, n // 2), (2 ** rng.uniform(3, 16.5, n - n // 2)).astype(np.int64)])
+    lens = lens.astype(np.uint32)
+    src_off = rng.integers(0, len(src) - int(lens.max()), n).astype(np.uint64)
+    gaps = rng.integers(0, 20, n).astype(np.uint64)
+    dst_off = (np.cumsum(lens.astype(np.uint64) + gaps) - lens.astype(np.uint64)).astype(np.uint64)
+    total = int(dst_off[-1] + lens[-1]) + 32
+    d_src = _gpu.to_dev(src)
+    d_dst = torch.full((total,), 0x77, dtype=torch.uint8, device="cuda")
+    a_src = _gpu.to_dev(src_off + np.uint64(d_src.data_ptr()))
+    a_dst = _gpu.to_dev(dst_off + np.uint64(d_dst.data_ptr()))
+    d_len = _gpu.to_dev(lens)
+    assert lib.ofi_amd_copy_table(a_src.data_ptr(), a_dst.data_ptr(), d_len.data_ptr(), n, _gpu.stream()) == 0
+    _gpu.sync()
+    want = np.full(total, 0x77, dtype=np.uint8)
+    for s, d, l in zip(src_off, dst_off, lens):
+        want[int(d):int(d) + int(l)] = src[int(s):int(s) + int(l)]
+    assert np.array_equal(d_dst.cpu().numpy(), want)
+    assert lib.ofi_amd_copy_table(None, a_dst.data_ptr(), d_len.data_ptr(), 1, _gpu.stream()) == -22
+    assert lib.ofi_amd_copy_table(a_src.data_ptr(), a_dst.data_ptr(), d_len.data_ptr(), 0, _gpu.stream()) == 0
+
+
+def test_bad_arguments(lib, gpu):
+    rings = ctypes.c_void_p()
+    assert lib.ofi_amd_gin_rings_create(1, 256, ctypes.byref(rings)) == 0
+    comms = (m.GinComm * 1)()
+    mrs = (m.GinMr * 3)()
+    regions = (m.GinSignalRegion * 1)()
+    stats = m.GinLoopbackStats()
+    args = (ctypes.cast(comms, ctypes.c_void_p), ctypes.cast(mrs, ctypes.c_void_p), regions)
+    assert lib.ofi_amd_gin_loopback_run(None, 1, *args, 1, 0, 64, 10, None, ctypes.byref(stats)) == -22
+    assert lib.ofi_amd_gin_loopback_run(rings, 1, *args, 0, 0, 64, 10, None, ctypes.byref(stats)) == -22
+    assert lib.ofi_amd_gin_loopback_run(rings, 1, *args, 1, 0, 0, 10, None, ctypes.byref(stats)) == -22
+    assert lib.ofi_amd_gin_loopback_run(rings, 1, *args, 1, 5000, 64, 10, None, ctypes.byref(stats)) == -22
+    lib.ofi_amd_gin_rings_destroy(rings)
