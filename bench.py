@@ -361,6 +361,43 @@ def bench_gin(lib, oracle, torch, np, args):
             "host_link_gbs": stats.descriptors * 68 / secs / 1e9, "proxy_threads": 4}
         lib.ofi_amd_gin_rings_destroy(rings)
     del d_table
+    # the whole path in process: seeded puts (8 B..1 MiB) -> proxy -> wire records -> device copies for
+    # the RDMA writes, completions to the receiver, ACKs back, signals applied in HBM.  One proxy thread.
+    l_ctx, l_ops = 32, min(ops, 20_000)
+    window = (1 << 30) + (1 << 20)
+    d_srcbuf = torch.randint(0, 255, (window,), dtype=torch.uint8, device="cuda")
+    d_dstbuf = torch.zeros(window, dtype=torch.uint8, device="cuda")
+    d_cnt = torch.zeros(512, dtype=torch.int64, device="cuda")
+    mrs = (m.GinMr * 3)()
+    mrs[0].local_base, mrs[1].remote_address_offset, mrs[2].remote_address = (
+        d_srcbuf.data_ptr(), d_dstbuf.data_ptr(), 0x7F5500000000)
+    comms = (m.GinComm * l_ctx)()
+    for c in range(l_ctx):
+        lib.ofi_amd_gin_comm_init(ctypes.byref(comms[c]), c, 4, 131072, 64, 0)
+    regions = (m.GinSignalRegion * 1)(m.GinSignalRegion(0x7F5500000000, 4096, d_cnt.data_ptr()))
+    rings = ctypes.c_void_p()
+    m.check(lib.ofi_amd_gin_rings_create(l_ctx, cap, ctypes.byref(rings)), "rings_create")
+    side = torch.cuda.Stream()
+    lstats = m.GinLoopbackStats()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    m.check(lib.ofi_amd_gin_produce_seeded(rings, SEED, l_ops, 1, 64, 1, 1, 0, _gpu.stream()), "produce")
+    rc = lib.ofi_amd_gin_loopback_run(rings, l_ops, ctypes.cast(comms, ctypes.c_void_p),
+                                      ctypes.cast(mrs, ctypes.c_void_p), regions, 1, 32, 4096, 20000,
+                                      ctypes.c_void_p(side.cuda_stream), ctypes.byref(lstats))
+    torch.cuda.synchronize()
+    secs = time.perf_counter() - t0
+    if rc != 0 or lib.ofi_amd_gin_producer_status(rings) != 0:
+        raise RuntimeError("gin loopback rc=%d" % rc)
+    signals_seen = int(d_cnt.sum().item())
+    out["loopback"] = {"contexts": l_ctx, "ops_per_context": l_ops, "puts_per_s": lstats.descriptors / secs,
+                       "payload_gbs": lstats.bytes / secs / 1e9, "payload_bytes": lstats.bytes,
+                       "rdma_writes": lstats.writes, "copy_launches": lstats.launches, "acks": lstats.acks,
+                       "signals": lstats.signals,
+                       "signals_counted_in_hbm_ok": signals_seen == l_ctx * (l_ops // 64), "proxy_threads": 1}
+    lib.ofi_amd_gin_rings_destroy(rings)
+    del d_srcbuf, d_dstbuf
+    torch.cuda.empty_cache()
     if not args.skip_cpu:
         # oracle: generate + fold the same stream on one core, on a bounded sample of the ops
         sample = min(ops, 40000)
