@@ -68,7 +68,7 @@ uint32_t ofi_amd_ctrl_mailbox_slot(uint16_t msg_seq_num)
 	return msg_seq_num % OFI_AMD_CTRL_MAILBOX_SIZE;
 }
 
-/* nccl_net_ofi_rdma_recv_comm::recv, mailbox update, src/nccl_ofi_rdma.cpp:3446-3474 */
+/* nccl_net_ofi_rdma_recv_comm::allocate_recv_req, mailbox update, src/nccl_ofi_rdma.cpp:3446-3474 */
 int ofi_amd_ctrl_msg_fill(ofi_amd_ctrl_msg_t *mailbox, uint16_t msg_seq_num, uint16_t num_recvs,
 			  const uint64_t *buff_offsets, const uint32_t *sizes, const int *tags,
 			  const uint64_t *mr_keys, uint32_t num_rails, int recv_completion_optional)

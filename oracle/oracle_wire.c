@@ -40,7 +40,7 @@ uint32_t oracle_ctrl_mailbox_slot(uint16_t msg_seq_num)
 	return msg_seq_num % MAILBOX_SIZE; /* :3447 */
 }
 
-/* recv(): mailbox update, :3446-3474 */
+/* allocate_recv_req (called by recv): mailbox update, :3446-3474 */
 int oracle_ctrl_msg_fill(oracle_ctrl_msg_t *mailbox, uint16_t msg_seq_num, uint16_t num_recvs,
 			 const uint64_t *buff_offsets, const uint32_t *sizes, const int *tags,
 			 const uint64_t *mr_keys, uint32_t num_rails, int recv_completion_optional)
