@@ -44,6 +44,30 @@ def timed_steps(fn, steps, warmup, torch):
     return wall, e0.elapsed_time(e1) / steps
 
 
+def per_launch_ms(fn, reps, torch):
+    """Each launch bracketed by its own pair of events: (median, min) in ms."""
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    for a, b in pairs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    t = sorted(a.elapsed_time(b) for a, b in pairs)
+    return t[len(t) // 2], t[0]
+
+
+def run_threads(fn, parts):
+    """fn(part) on one thread per part (oracle calls run outside the interpreter lock); seconds."""
+    import threading
+    threads = [threading.Thread(target=fn, args=(p,)) for p in parts]
+    t0 = time.perf_counter()
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    return time.perf_counter() - t0
+
+
 def bench_bounce(lib, oracle, torch, np, args):
     import _gpu
     import _oracle
@@ -65,6 +89,7 @@ def bench_bounce(lib, oracle, torch, np, args):
             raise RuntimeError("ofi_amd_bounce_scatter: %d" % rc)
 
     wall_ms, ev_ms = timed_steps(step, args.steps, args.warmup, torch)
+    med_ms, min_ms = per_launch_ms(step, max(10, args.steps), torch)
     algo_bytes = 2 * w["src_bytes"] + 8 * n          # payload read + write, 4 B flush read + 4 B write
     # result check of the timed configuration: flush words and an arena checksum against the oracle
     arena = np.zeros(w["arena_bytes"], dtype=np.uint8)
@@ -81,7 +106,7 @@ def bench_bounce(lib, oracle, torch, np, args):
     out = {"ms_wall": wall_ms, "ms_kernel": ev_ms, "algo_bytes": algo_bytes,
            "gbs": algo_bytes / ev_ms / 1e6, "gbs_wall": algo_bytes / wall_ms / 1e6,
            "device_copy_gbs": 2 * w["src_bytes"] / copy_ms / 1e6, "parity_ok": ok, "buffers": n,
-           "payload_bytes": w["src_bytes"]}
+           "payload_bytes": w["src_bytes"], "ms_kernel_median": med_ms, "ms_kernel_min": min_ms}
     cpu = None
     if not args.skip_cpu:
         reps = max(2, min(40, int(8.0 / max(first_cpu_s, 1e-3))))
@@ -227,6 +252,20 @@ def bench_sched(lib, oracle, torch, np, args):
                 reps += 1
             out[name] = n * reps / (time.perf_counter() - t0)
         out["cpu_cores"] = 1
+        # every core: one scheduler instance per thread (the reference has one per endpoint), each
+        # striping its slice of the batch
+        cores = min(16, os.cpu_count() or 1)
+        bounds = [n * t // cores for t in range(cores + 1)]
+        reps = 20
+
+        def part(t):
+            lo, hi = bounds[t], bounds[t + 1]
+            ost = _oracle.Sched(1, 3, 64, 131072, 4, 0)
+            for _ in range(reps):
+                oracle.oracle_sched_batch(ctypes.byref(ost), _oracle.ptr(sizes[lo:hi]), hi - lo, 128,
+                                          _oracle.ptr(num[lo:hi]), _oracle.ptr(xf[lo:hi]))
+        out["cpu_all_cores_msgs_per_s"] = n * reps / run_threads(part, range(cores))
+        out["cpu_all_cores"] = cores
     return out
 
 
@@ -286,6 +325,23 @@ def bench_tuner(lib, oracle, torch, np, args):
             grids += 1
         out["cpu_region_points_per_s"] = grids * points / (time.perf_counter() - t0)
         out["cpu_cores"] = 1
+        # every core: whole grids per thread (cells are independent)
+        cores = min(16, os.cpu_count() or 1)
+        per_thread = 12
+
+        def model_part(t):
+            c, ch = np.zeros(cells, dtype=np.float64), np.zeros(points * 2, dtype=np.int8)
+            for g in range(per_thread):
+                oracle.oracle_model_grid(g % 2, 1 + g // 2, 8, 3, *axes, _oracle.ptr(algos), len(algos),
+                                         _oracle.ptr(c), _oracle.ptr(ch))
+
+        def region_part(t):
+            rc_ = np.zeros(points * 3, dtype=np.int32)
+            for g in range(per_thread):
+                oracle.oracle_region_grid(g % 4, *axes, _oracle.ptr(rc_))
+        out["cpu_all_cores_model_cells_per_s"] = cores * per_thread * cells / run_threads(model_part, range(cores))
+        out["cpu_all_cores_region_points_per_s"] = cores * per_thread * points / run_threads(region_part, range(cores))
+        out["cpu_all_cores"] = cores
         # parity of the timed launches: the first four grids of each kind against the oracle
         model_step()
         region_step()
@@ -412,6 +468,15 @@ def bench_gin(lib, oracle, torch, np, args):
         out["cpu_generate_derive_fold_descs_per_s"] = nctx * sample / s1
         out["cpu_cores"] = 1
         out["cpu_sample"] = "%d ops per context" % sample
+        # CPU producer threads pushing the same records through the reference's ring protocol (push
+        # with CAS, one ring per context) to one consumer thread
+        for producers in (1, 4):
+            rck, rsec = ctypes.c_uint64(), ctypes.c_double()
+            rc = oracle.oracle_gin_cpu_rings_run(SEED, nctx, sample, cap, producers, 1, 64, 1, 1,
+                                                 ctypes.byref(rck), ctypes.byref(rsec))
+            out["cpu_%d_producers_through_rings" % producers] = {
+                "descs_per_s": nctx * sample / rsec.value if rc == 0 else None,
+                "consumer_threads": 1, "checksum_ok": rc == 0 and rck.value == ck}
         # parity at the full size: the oracle's checksums of the whole stream (a few seconds for the
         # descriptors, about ten for the derived wire records at 256 x 1,000,000 ops)
         if sample != ops:
@@ -480,6 +545,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": bounce["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": bounce["gbs"] / HBM_PEAK_GBS, "traffic": traffic,
                      "kernel": "bounce_scatter_kernel", "kernel_ms": bounce["ms_kernel"],
+                     "kernel_ms_median": bounce["ms_kernel_median"], "kernel_ms_min": bounce["ms_kernel_min"],
                      "algorithmic_bytes_per_launch": bounce["algo_bytes"],
                      "device_copy_GBps_same_payload": bounce["device_copy_gbs"]},
         "cpu_baseline": cpu,

@@ -245,6 +245,12 @@ uint64_t oracle_gin_stream_checksum(uint64_t seed, uint32_t n_contexts, uint64_t
 				    uint32_t aggregate_mask, int with_wire, uint32_t num_rails,
 				    uint64_t min_stripe, uint64_t max_small, uint32_t ack_model,
 				    const oracle_gin_mr_t *mrs);
+/* CPU producer threads -> one MPSC ring per context (push with CAS) -> the calling thread as
+ * the only consumer; *checksum equals oracle_gin_stream_checksum(with_wire = 0) */
+int oracle_gin_cpu_rings_run(uint64_t seed, uint32_t n_contexts, uint64_t ops, uint32_t capacity,
+			     uint32_t producers, uint32_t peer_rank, uint32_t signal_every,
+			     uint32_t signal_op, uint32_t aggregate_mask, uint64_t *checksum,
+			     double *seconds);
 
 /* ------------------------------------------------------------------- tuner */
 

@@ -323,3 +323,122 @@ uint64_t oracle_gin_stream_checksum(uint64_t seed, uint32_t n_contexts, uint64_t
 	}
 	return total;
 }
+
+/* ---- CPU producers through the reference's ring protocol ----
+ * `producers` threads generate the seeded descriptors of their contexts and push them
+ * through one MPSC ring per context (push with CAS, include/nccl_ofi_mpsc_ring.h:79-118);
+ * the calling thread is the single consumer of every ring, as the GIN progress loop is
+ * (src/rdma/gin/nccl_ofi_gin.cpp:1560-1574), and folds what it pops.  The result equals
+ * oracle_gin_stream_checksum(with_wire = 0) of the same stream.  Returns 0 or -errno;
+ * *seconds covers thread start to the last pop. */
+#include <pthread.h>
+#include <stdlib.h>
+#include <time.h>
+
+struct cpu_ring_producer {
+	oracle_mpsc_t **rings;
+	uint64_t seed, ops;
+	uint32_t first, last; /* contexts [first, last) */
+	uint32_t peer_rank, signal_every, signal_op, aggregate_mask;
+};
+
+static void *cpu_ring_producer_main(void *p)
+{
+	struct cpu_ring_producer *a = (struct cpu_ring_producer *)p;
+	uint32_t n = a->last - a->first;
+	uint64_t *next = (uint64_t *)calloc(n ? n : 1, sizeof(uint64_t));
+	uint32_t open = n;
+	if (!next) {
+		return (void *)1;
+	}
+	while (open > 0) {
+		open = 0;
+		for (uint32_t k = 0; k < n; k++) {
+			/* a burst per visit: stay on a ring while it takes entries */
+			for (int burst = 0; burst < 64 && next[k] < a->ops; burst++) {
+				oracle_gin_desc_t d;
+				oracle_gin_gen_desc(a->seed, a->first + k, next[k], a->peer_rank,
+						    a->signal_every, a->signal_op, a->aggregate_mask, &d);
+				if (!oracle_mpsc_push(a->rings[a->first + k], &d)) {
+					break;
+				}
+				next[k]++;
+			}
+			open += next[k] < a->ops;
+		}
+	}
+	free(next);
+	return NULL;
+}
+
+int oracle_gin_cpu_rings_run(uint64_t seed, uint32_t n_contexts, uint64_t ops, uint32_t capacity,
+			     uint32_t producers, uint32_t peer_rank, uint32_t signal_every,
+			     uint32_t signal_op, uint32_t aggregate_mask, uint64_t *checksum,
+			     double *seconds)
+{
+	if (n_contexts == 0 || producers == 0 || producers > 64 || producers > n_contexts || !checksum ||
+	    !seconds) {
+		return -22;
+	}
+	oracle_mpsc_t **rings = (oracle_mpsc_t **)calloc(n_contexts, sizeof(*rings));
+	uint64_t *hash = (uint64_t *)calloc(n_contexts, sizeof(uint64_t));
+	uint64_t *popped = (uint64_t *)calloc(n_contexts, sizeof(uint64_t));
+	struct cpu_ring_producer args[64];
+	pthread_t th[64];
+	int rc = 0;
+	if (!rings || !hash || !popped) {
+		rc = -12;
+	}
+	for (uint32_t c = 0; rc == 0 && c < n_contexts; c++) {
+		rings[c] = oracle_mpsc_create(capacity, sizeof(oracle_gin_desc_t));
+		hash[c] = 0x9E3779B97F4A7C15ull ^ c;
+		if (!rings[c]) {
+			rc = -12;
+		}
+	}
+	if (rc == 0) {
+		struct timespec t0, t1;
+		clock_gettime(CLOCK_MONOTONIC, &t0);
+		for (uint32_t p = 0; p < producers; p++) {
+			args[p] = (struct cpu_ring_producer){ rings, seed, ops,
+				(uint32_t)((uint64_t)n_contexts * p / producers),
+				(uint32_t)((uint64_t)n_contexts * (p + 1) / producers),
+				peer_rank, signal_every, signal_op, aggregate_mask };
+			pthread_create(&th[p], NULL, cpu_ring_producer_main, &args[p]);
+		}
+		uint64_t left = (uint64_t)n_contexts * ops;
+		while (left > 0) {
+			for (uint32_t c = 0; c < n_contexts; c++) {
+				oracle_gin_desc_t d;
+				while (popped[c] < ops && oracle_mpsc_pop(rings[c], &d)) {
+					hash[c] = oracle_gin_fold(hash[c], (const uint64_t *)&d, 8);
+					popped[c]++;
+					left--;
+				}
+			}
+		}
+		clock_gettime(CLOCK_MONOTONIC, &t1);
+		for (uint32_t p = 0; p < producers; p++) {
+			void *ret = NULL;
+			pthread_join(th[p], &ret);
+			if (ret) {
+				rc = -12;
+			}
+		}
+		*seconds = (double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec);
+		uint64_t total = 0;
+		for (uint32_t c = 0; c < n_contexts; c++) {
+			total += hash[c];
+		}
+		*checksum = total;
+	}
+	for (uint32_t c = 0; rings && c < n_contexts; c++) {
+		if (rings[c]) {
+			oracle_mpsc_destroy(rings[c]);
+		}
+	}
+	free(rings);
+	free(hash);
+	free(popped);
+	return rc;
+}

@@ -163,6 +163,8 @@ _ORACLE_PROTOS = {
     "oracle_eager_copy_batch": (None, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_u32, c_vp]),
     "oracle_gin_stream_checksum": (c_u64, [c_u64, c_u32, c_u64, c_u32, c_u32, c_u32, c_u32, c_int,
                                            c_u32, c_u64, c_u64, c_u32, ctypes.POINTER(GinMr)]),
+    "oracle_gin_cpu_rings_run": (c_int, [c_u64, c_u32, c_u64, c_u32, c_u32, c_u32, c_u32, c_u32, c_u32,
+                                         ctypes.POINTER(c_u64), ctypes.POINTER(ctypes.c_double)]),
     "oracle_model_cost": (ctypes.c_float, [c_int, c_int, c_int, c_int, c_int, c_u64, c_u64, c_u64,
                                            c_int, c_int]),
     "oracle_model_decide": (None, [c_int, c_int, c_int, c_u64, c_u64, c_u64, c_int, c_int,
