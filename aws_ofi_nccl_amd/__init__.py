@@ -136,6 +136,39 @@ class EagerTx(ctypes.Structure):
                 ("pad", ctypes.c_uint16)]
 
 
+class SendAction(ctypes.Structure):
+    """ofi_amd_send_action_t"""
+    _fields_ = [("kind", c_i32), ("req", c_i32), ("msg_seq_num", ctypes.c_uint16),
+                ("recv_idx", ctypes.c_uint8), ("no_target_completion", ctypes.c_uint8), ("imm", c_u32),
+                ("hdr", EagerHdr), ("size", c_u64), ("remote_buff_offset", c_u64), ("mr_key", c_u64 * 4),
+                ("num_xfers", c_u32), ("pad", c_u32), ("xfers", XferInfo * 4)]
+
+
+class SendState(ctypes.Structure):
+    """ofi_amd_send_state_t"""
+    _fields_ = [("next_msg_seq_num", ctypes.c_uint16), ("group_sends_remaining", ctypes.c_uint16),
+                ("group_num_recvs", ctypes.c_uint16), ("cur_eager_seq", ctypes.c_uint16),
+                ("eager_seq_next", ctypes.c_uint16), ("eager_queue_count", ctypes.c_uint8),
+                ("eager_offset_next", ctypes.c_uint8), ("prev_eager_batch_count", ctypes.c_uint8),
+                ("pad", ctypes.c_uint8 * 3), ("num_inflight_reqs", c_u32), ("num_inflight_writes", c_u32),
+                ("n_ctrl_received", c_u64)]
+
+
+class EagerCopyItem(ctypes.Structure):
+    """ofi_amd_eager_copy_item_t"""
+    _fields_ = [("rx_cookie", c_u64), ("dst", c_u64), ("dst_len", c_u64), ("recv_len", c_u32),
+                ("req", c_i32), ("sub_idx", c_i32), ("needs_copy", c_i32)]
+
+
+class RecvState(ctypes.Structure):
+    """ofi_amd_recv_state_t"""
+    _fields_ = [("next_msg_seq_num", ctypes.c_uint16), ("eager_drain_recv_seq", ctypes.c_uint16),
+                ("last_eager_seq", ctypes.c_uint16), ("last_completed_seq", ctypes.c_uint16),
+                ("last_eager_offset", ctypes.c_uint8), ("has_processed_eager", ctypes.c_uint8),
+                ("pad", ctypes.c_uint8 * 2), ("num_inflight_reqs", c_u32), ("eager_pending", c_u32),
+                ("pad2", c_u32), ("n_ctrl_sent", c_u64)]
+
+
 class TunerQuery(ctypes.Structure):
     """ofi_amd_tuner_query_t (64 bytes)"""
     _fields_ = [("platform", c_i32), ("kind", c_i32), ("coll", c_i32), ("pipe_ops", c_i32),
@@ -295,6 +328,40 @@ PROTOTYPES = {
     "ofi_amd_eager_tx_assign": (None, [ctypes.POINTER(EagerTx), c_i32, ctypes.POINTER(EagerHdr)]),
     "ofi_amd_eager_tx_advance": (None, [ctypes.POINTER(EagerTx)]),
     "ofi_amd_eager_fits": (ctypes.c_int, [c_u64, ctypes.c_int64]),
+    "ofi_amd_msgbuff_create": (ctypes.c_int, [ctypes.c_uint16, ctypes.c_uint16, ctypes.c_uint16,
+                                              ctypes.POINTER(c_vp)]),
+    "ofi_amd_msgbuff_destroy": (ctypes.c_int, [c_vp]),
+    "ofi_amd_msgbuff_insert": (ctypes.c_int, [c_vp, ctypes.c_uint16, c_vp, ctypes.c_int,
+                                              ctypes.POINTER(ctypes.c_int)]),
+    "ofi_amd_msgbuff_replace": (ctypes.c_int, [c_vp, ctypes.c_uint16, c_vp, ctypes.c_int,
+                                               ctypes.POINTER(ctypes.c_int)]),
+    "ofi_amd_msgbuff_retrieve": (ctypes.c_int, [c_vp, ctypes.c_uint16, ctypes.POINTER(c_vp),
+                                                ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]),
+    "ofi_amd_msgbuff_complete": (ctypes.c_int, [c_vp, ctypes.c_uint16, ctypes.POINTER(ctypes.c_int)]),
+    "ofi_amd_send_comm_create": (ctypes.c_int, [c_u32, c_u32, ctypes.c_int64, c_u64, c_u64,
+                                                ctypes.POINTER(c_vp)]),
+    "ofi_amd_send_comm_destroy": (ctypes.c_int, [c_vp]),
+    "ofi_amd_send_comm_mailbox": (ctypes.POINTER(CtrlMsg), [c_vp]),
+    "ofi_amd_send_comm_send": (ctypes.c_int, [c_vp, c_u64, c_i32, ctypes.POINTER(SendAction)]),
+    "ofi_amd_send_comm_completion": (ctypes.c_int, [c_vp, c_i32]),
+    "ofi_amd_send_comm_test": (ctypes.c_int, [c_vp, c_i32, ctypes.POINTER(ctypes.c_int),
+                                              ctypes.POINTER(c_u64)]),
+    "ofi_amd_send_comm_state": (None, [c_vp, ctypes.POINTER(SendState)]),
+    "ofi_amd_recv_comm_create": (ctypes.c_int, [c_u32, ctypes.POINTER(c_vp)]),
+    "ofi_amd_recv_comm_destroy": (ctypes.c_int, [c_vp]),
+    "ofi_amd_recv_comm_recv": (ctypes.c_int, [c_vp, ctypes.c_int, ctypes.POINTER(c_u64),
+                                              ctypes.POINTER(c_u64), ctypes.POINTER(ctypes.c_int),
+                                              ctypes.POINTER(c_u64), ctypes.c_int, ctypes.POINTER(CtrlMsg),
+                                              ctypes.POINTER(c_i32), ctypes.POINTER(ctypes.c_uint16)]),
+    "ofi_amd_recv_comm_eager_arrival": (ctypes.c_int, [c_vp, ctypes.c_uint16, ctypes.POINTER(EagerHdr),
+                                                       c_u32, c_u64]),
+    "ofi_amd_recv_comm_write_arrival": (ctypes.c_int, [c_vp, c_u32, c_u64]),
+    "ofi_amd_recv_comm_ctrl_sent": (ctypes.c_int, [c_vp, c_i32]),
+    "ofi_amd_recv_comm_take_copies": (c_u32, [c_vp, ctypes.POINTER(EagerCopyItem), c_u32]),
+    "ofi_amd_recv_comm_copy_done": (ctypes.c_int, [c_vp, c_i32, c_i32]),
+    "ofi_amd_recv_comm_test": (ctypes.c_int, [c_vp, c_i32, ctypes.POINTER(ctypes.c_int),
+                                              ctypes.POINTER(ctypes.c_int)]),
+    "ofi_amd_recv_comm_state": (None, [c_vp, ctypes.POINTER(RecvState)]),
     "ofi_amd_tuner_plan_create": (ctypes.c_int, [c_vp, c_u32, c_vp, c_u32, c_vp, c_u32, c_vp,
                                                  c_u32, c_vp, c_u32, ctypes.POINTER(c_vp)]),
     "ofi_amd_tuner_plan_destroy": (ctypes.c_int, [c_vp]),

@@ -40,6 +40,14 @@
  *                    regression) and the static_asserts of include/nccl_ofi_rdma.h
  *                    (8 / 64 / 512 / 560 bytes); sender numbering -> reordered
  *                    delivery -> chain drain returns send order
+ *   message buffer   the scenario of tests/unit/msgbuff.cpp:42-122 (4 in flight, 4-bit
+ *                    numbers, four rounds) plus wrap, skip and out-of-order cases
+ *   send/recv state  who-receives-what and reported sizes of the scenarios of
+ *   machines         tests/functional/eager_multirecv.cpp (T5-T19, T21-T25) replayed with
+ *                    the test as the wire; per-tag order under random interleavings
+ *                    with unique tags.  The decision stream itself (which call returns
+ *                    "again", eager header values beyond ctrl_msg.cpp's): PARITY UNPINNED
+ *                    (no reference test observes it; the source does not build here)
  */
 #ifndef ORACLE_H_
 #define ORACLE_H_
@@ -384,6 +392,107 @@ int oracle_flush_completed(const uint64_t *slots, uint32_t num_rails, uint64_t s
 void oracle_eager_copy_batch(const uint8_t *rx_base, const uint64_t *rx_off, const uint32_t *recv_len,
 			     uint8_t *dst_base, const uint64_t *dst_off, const uint32_t *dst_len, uint32_t n,
 			     uint32_t *copied);
+
+/* ------------------------------------------- send/receive protocol state machines */
+
+/* nccl_ofi_msgbuff_status_t / _result_t / _elemtype_t, include/nccl_ofi_msgbuff.h:42-69 */
+enum { ORACLE_MSGBUFF_COMPLETED = 0, ORACLE_MSGBUFF_INPROGRESS, ORACLE_MSGBUFF_NOTSTARTED,
+       ORACLE_MSGBUFF_UNAVAILABLE };
+enum { ORACLE_MSGBUFF_SUCCESS = 0, ORACLE_MSGBUFF_INVALID_IDX, ORACLE_MSGBUFF_ERROR };
+enum { ORACLE_MSGBUFF_REQ = 0, ORACLE_MSGBUFF_BUFF };
+
+typedef struct oracle_msgbuff oracle_msgbuff_t;
+oracle_msgbuff_t *oracle_msgbuff_create(uint16_t max_inprogress, uint16_t bit_width, uint16_t start_seq);
+void oracle_msgbuff_destroy(oracle_msgbuff_t *m);
+int oracle_msgbuff_insert(oracle_msgbuff_t *m, uint16_t msg_index, void *elem, int type, int *status);
+int oracle_msgbuff_replace(oracle_msgbuff_t *m, uint16_t msg_index, void *elem, int type, int *status);
+int oracle_msgbuff_retrieve(oracle_msgbuff_t *m, uint16_t msg_index, void **elem, int *type, int *status);
+int oracle_msgbuff_complete(oracle_msgbuff_t *m, uint16_t msg_index, int *status);
+
+enum { ORACLE_SEND_AGAIN = 0, ORACLE_SEND_EAGER = 1, ORACLE_SEND_WRITE = 2 };
+
+/* what send() would hand to the fabric */
+typedef struct {
+	int32_t kind;
+	int32_t req;
+	uint16_t msg_seq_num;
+	uint8_t recv_idx;
+	uint8_t no_target_completion;
+	uint32_t imm;
+	oracle_eager_hdr_t hdr;
+	uint64_t size;
+	uint64_t remote_buff_offset;
+	uint64_t mr_key[4];
+	uint32_t num_xfers;
+	uint32_t pad;
+	oracle_xfer_t xfers[4];
+} oracle_send_action_t;
+
+typedef struct {
+	uint16_t next_msg_seq_num;
+	uint16_t group_sends_remaining;
+	uint16_t group_num_recvs;
+	uint16_t cur_eager_seq;
+	uint16_t eager_seq_next;
+	uint8_t eager_queue_count;
+	uint8_t eager_offset_next;
+	uint8_t prev_eager_batch_count;
+	uint8_t pad[3];
+	uint32_t num_inflight_reqs;
+	uint32_t num_inflight_writes;
+	uint64_t n_ctrl_received;
+} oracle_send_state_t;
+
+typedef struct oracle_send_comm oracle_send_comm_t;
+oracle_send_comm_t *oracle_send_comm_create(uint32_t remote_comm_id, uint32_t num_rails,
+					    int64_t eager_send_size, uint64_t min_stripe,
+					    uint64_t max_small);
+void oracle_send_comm_destroy(oracle_send_comm_t *s);
+oracle_ctrl_msg_t *oracle_send_comm_mailbox(oracle_send_comm_t *s);
+void oracle_send_comm_state(const oracle_send_comm_t *s, oracle_send_state_t *out);
+int oracle_send_comm_send(oracle_send_comm_t *s, uint64_t size, int32_t tag, oracle_send_action_t *act);
+int oracle_send_comm_completion(oracle_send_comm_t *s, int32_t req);
+int oracle_send_comm_test(oracle_send_comm_t *s, int32_t req, int *done, uint64_t *size);
+
+/* one eager arrival matched to a posted receive: the copy the reference posts as a loop-back read */
+typedef struct {
+	uint64_t rx_cookie;
+	uint64_t dst;
+	uint64_t dst_len;
+	uint32_t recv_len;
+	int32_t req;
+	int32_t sub_idx;
+	int32_t needs_copy; /* 0: zero-length message, completed at the match */
+} oracle_eager_copy_item_t;
+
+typedef struct {
+	uint16_t next_msg_seq_num;
+	uint16_t eager_drain_recv_seq;
+	uint16_t last_eager_seq;
+	uint16_t last_completed_seq;
+	uint8_t last_eager_offset;
+	uint8_t has_processed_eager;
+	uint8_t pad[2];
+	uint32_t num_inflight_reqs;
+	uint32_t eager_pending;
+	uint32_t pad2;
+	uint64_t n_ctrl_sent;
+} oracle_recv_state_t;
+
+typedef struct oracle_recv_comm oracle_recv_comm_t;
+oracle_recv_comm_t *oracle_recv_comm_create(uint32_t num_rails);
+void oracle_recv_comm_destroy(oracle_recv_comm_t *r);
+int oracle_recv_comm_recv(oracle_recv_comm_t *r, int n, const uint64_t *dsts, const uint64_t *sizes,
+			  const int *tags, const uint64_t *mr_keys, int completion_optional,
+			  oracle_ctrl_msg_t *mailbox, int32_t *req_out, uint16_t *seq_out);
+int oracle_recv_comm_eager_arrival(oracle_recv_comm_t *r, uint16_t msg_seq_num,
+				   const oracle_eager_hdr_t *hdr, uint32_t recv_len, uint64_t rx_cookie);
+int oracle_recv_comm_write_arrival(oracle_recv_comm_t *r, uint32_t imm, uint64_t len);
+int oracle_recv_comm_ctrl_sent(oracle_recv_comm_t *r, int32_t req);
+uint32_t oracle_recv_comm_take_copies(oracle_recv_comm_t *r, oracle_eager_copy_item_t *out, uint32_t cap);
+int oracle_recv_comm_copy_done(oracle_recv_comm_t *r, int32_t req, int32_t sub_idx);
+int oracle_recv_comm_test(oracle_recv_comm_t *r, int32_t req, int *done, int *sizes);
+void oracle_recv_comm_state(const oracle_recv_comm_t *r, oracle_recv_state_t *out);
 
 #ifdef __cplusplus
 }

@@ -95,6 +95,35 @@ class EagerTx(ctypes.Structure):
                 ("pad", ctypes.c_uint16)]
 
 
+class SendAction(ctypes.Structure):
+    _fields_ = [("kind", c_i32), ("req", c_i32), ("msg_seq_num", ctypes.c_uint16),
+                ("recv_idx", ctypes.c_uint8), ("no_target_completion", ctypes.c_uint8), ("imm", c_u32),
+                ("hdr", EagerHdr), ("size", c_u64), ("remote_buff_offset", c_u64), ("mr_key", c_u64 * 4),
+                ("num_xfers", c_u32), ("pad", c_u32), ("xfers", Xfer * 4)]
+
+
+class SendState(ctypes.Structure):
+    _fields_ = [("next_msg_seq_num", ctypes.c_uint16), ("group_sends_remaining", ctypes.c_uint16),
+                ("group_num_recvs", ctypes.c_uint16), ("cur_eager_seq", ctypes.c_uint16),
+                ("eager_seq_next", ctypes.c_uint16), ("eager_queue_count", ctypes.c_uint8),
+                ("eager_offset_next", ctypes.c_uint8), ("prev_eager_batch_count", ctypes.c_uint8),
+                ("pad", ctypes.c_uint8 * 3), ("num_inflight_reqs", c_u32), ("num_inflight_writes", c_u32),
+                ("n_ctrl_received", c_u64)]
+
+
+class EagerCopyItem(ctypes.Structure):
+    _fields_ = [("rx_cookie", c_u64), ("dst", c_u64), ("dst_len", c_u64), ("recv_len", c_u32),
+                ("req", c_i32), ("sub_idx", c_i32), ("needs_copy", c_i32)]
+
+
+class RecvState(ctypes.Structure):
+    _fields_ = [("next_msg_seq_num", ctypes.c_uint16), ("eager_drain_recv_seq", ctypes.c_uint16),
+                ("last_eager_seq", ctypes.c_uint16), ("last_completed_seq", ctypes.c_uint16),
+                ("last_eager_offset", ctypes.c_uint8), ("has_processed_eager", ctypes.c_uint8),
+                ("pad", ctypes.c_uint8 * 2), ("num_inflight_reqs", c_u32), ("eager_pending", c_u32),
+                ("pad2", c_u32), ("n_ctrl_sent", c_u64)]
+
+
 class Point(ctypes.Structure):
     _fields_ = [("x", ctypes.c_double), ("y", ctypes.c_double)]
 
@@ -163,6 +192,33 @@ _ORACLE_PROTOS = {
     "oracle_eager_copy_batch": (None, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_u32, c_vp]),
     "oracle_gin_stream_checksum": (c_u64, [c_u64, c_u32, c_u64, c_u32, c_u32, c_u32, c_u32, c_int,
                                            c_u32, c_u64, c_u64, c_u32, ctypes.POINTER(GinMr)]),
+    "oracle_msgbuff_create": (c_vp, [ctypes.c_uint16, ctypes.c_uint16, ctypes.c_uint16]),
+    "oracle_msgbuff_destroy": (None, [c_vp]),
+    "oracle_msgbuff_insert": (c_int, [c_vp, ctypes.c_uint16, c_vp, c_int, ctypes.POINTER(c_int)]),
+    "oracle_msgbuff_replace": (c_int, [c_vp, ctypes.c_uint16, c_vp, c_int, ctypes.POINTER(c_int)]),
+    "oracle_msgbuff_retrieve": (c_int, [c_vp, ctypes.c_uint16, ctypes.POINTER(c_vp), ctypes.POINTER(c_int),
+                                        ctypes.POINTER(c_int)]),
+    "oracle_msgbuff_complete": (c_int, [c_vp, ctypes.c_uint16, ctypes.POINTER(c_int)]),
+    "oracle_send_comm_create": (c_vp, [c_u32, c_u32, ctypes.c_int64, c_u64, c_u64]),
+    "oracle_send_comm_destroy": (None, [c_vp]),
+    "oracle_send_comm_mailbox": (ctypes.POINTER(CtrlMsg), [c_vp]),
+    "oracle_send_comm_state": (None, [c_vp, ctypes.POINTER(SendState)]),
+    "oracle_send_comm_send": (c_int, [c_vp, c_u64, c_i32, ctypes.POINTER(SendAction)]),
+    "oracle_send_comm_completion": (c_int, [c_vp, c_i32]),
+    "oracle_send_comm_test": (c_int, [c_vp, c_i32, ctypes.POINTER(c_int), ctypes.POINTER(c_u64)]),
+    "oracle_recv_comm_create": (c_vp, [c_u32]),
+    "oracle_recv_comm_destroy": (None, [c_vp]),
+    "oracle_recv_comm_recv": (c_int, [c_vp, c_int, ctypes.POINTER(c_u64), ctypes.POINTER(c_u64),
+                                      ctypes.POINTER(c_int), ctypes.POINTER(c_u64), c_int,
+                                      ctypes.POINTER(CtrlMsg), ctypes.POINTER(c_i32),
+                                      ctypes.POINTER(ctypes.c_uint16)]),
+    "oracle_recv_comm_eager_arrival": (c_int, [c_vp, ctypes.c_uint16, ctypes.POINTER(EagerHdr), c_u32, c_u64]),
+    "oracle_recv_comm_write_arrival": (c_int, [c_vp, c_u32, c_u64]),
+    "oracle_recv_comm_ctrl_sent": (c_int, [c_vp, c_i32]),
+    "oracle_recv_comm_take_copies": (c_u32, [c_vp, ctypes.POINTER(EagerCopyItem), c_u32]),
+    "oracle_recv_comm_copy_done": (c_int, [c_vp, c_i32, c_i32]),
+    "oracle_recv_comm_test": (c_int, [c_vp, c_i32, ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
+    "oracle_recv_comm_state": (None, [c_vp, ctypes.POINTER(RecvState)]),
     "oracle_gin_cpu_rings_run": (c_int, [c_u64, c_u32, c_u64, c_u32, c_u32, c_u32, c_u32, c_u32, c_u32,
                                          ctypes.POINTER(c_u64), ctypes.POINTER(ctypes.c_double)]),
     "oracle_model_cost": (ctypes.c_float, [c_int, c_int, c_int, c_int, c_int, c_u64, c_u64, c_u64,

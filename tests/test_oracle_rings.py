@@ -165,3 +165,17 @@ def test_spsc_side_by_side(oracle, ref):
             assert ra == rb and (not ra or a.value == b.value)
     ref.ref_spsc_destroy(rr)
     oracle.oracle_spsc_destroy(orr)
+
+
+@pytest.mark.parametrize("producers", [1, 3])
+def test_cpu_producers_through_rings_deliver_the_seeded_stream(oracle, producers):
+    """Producer threads -> one ring per context -> one consumer: what the consumer folds is the
+    seeded stream itself, whatever the interleaving (small rings, so full and wrap both occur)."""
+    ck, secs = ctypes.c_uint64(), ctypes.c_double()
+    assert oracle.oracle_gin_cpu_rings_run(7, 12, 3000, 64, producers, 1, 64, 1, 1,
+                                           ctypes.byref(ck), ctypes.byref(secs)) == 0
+    want = oracle.oracle_gin_stream_checksum(7, 12, 3000, 1, 64, 1, 1, 0, 4, 131072, 64, 1,
+                                             _oracle.default_mrs())
+    assert ck.value == want and secs.value > 0
+    assert oracle.oracle_gin_cpu_rings_run(7, 2, 10, 64, 3, 1, 64, 1, 1, ctypes.byref(ck),
+                                           ctypes.byref(secs)) == -22    # more producers than contexts
