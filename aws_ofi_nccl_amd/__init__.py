@@ -169,6 +169,14 @@ class RecvState(ctypes.Structure):
                 ("pad2", c_u32), ("n_ctrl_sent", c_u64)]
 
 
+class SendrecvLoopbackStats(ctypes.Structure):
+    """ofi_amd_sendrecv_loopback_stats_t"""
+    _fields_ = [("messages", c_u64), ("payload_bytes", c_u64), ("eager_messages", c_u64),
+                ("write_messages", c_u64), ("rdma_writes", c_u64), ("copy_entries", c_u64),
+                ("rounds", c_u64), ("launches", c_u64), ("send_again", c_u64),
+                ("seconds", ctypes.c_double)]
+
+
 class TunerQuery(ctypes.Structure):
     """ofi_amd_tuner_query_t (64 bytes)"""
     _fields_ = [("platform", c_i32), ("kind", c_i32), ("coll", c_i32), ("pipe_ops", c_i32),
@@ -362,6 +370,9 @@ PROTOTYPES = {
     "ofi_amd_recv_comm_test": (ctypes.c_int, [c_vp, c_i32, ctypes.POINTER(ctypes.c_int),
                                               ctypes.POINTER(ctypes.c_int)]),
     "ofi_amd_recv_comm_state": (None, [c_vp, ctypes.POINTER(RecvState)]),
+    "ofi_amd_sendrecv_loopback_run": (ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_u64, c_u32, c_u32, c_vp,
+                                                     c_u64, c_u32, c_vp,
+                                                     ctypes.POINTER(SendrecvLoopbackStats)]),
     "ofi_amd_tuner_plan_create": (ctypes.c_int, [c_vp, c_u32, c_vp, c_u32, c_vp, c_u32, c_vp,
                                                  c_u32, c_vp, c_u32, ctypes.POINTER(c_vp)]),
     "ofi_amd_tuner_plan_destroy": (ctypes.c_int, [c_vp]),

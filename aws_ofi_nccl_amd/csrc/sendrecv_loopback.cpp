@@ -1,0 +1,279 @@
+/*
+ * In-process loop-back of the send/receive path on one GPU (ofi_amd_sendrecv_loopback_run):
+ * one send comm and one receive comm of this library, with this file standing where the
+ * reference has two ranks and a libfabric provider (the isend/irecv/test loop of
+ * tests/functional/nccl_message_transfer.cpp:19-56).  An eager send becomes a device copy of header
+ * and payload into an rx buffer; the RDMA writes of a rendezvous become device copies stripe by
+ * stripe; what the receiver decides to copy out of rx buffers goes through the batched eager
+ * copy.  `inflight` messages are open at a time; each round is two launches and one wait.
+ */
+#include <cerrno>
+#include <chrono>
+#include <cstring>
+#include <vector>
+
+#include "ofi_amd_sendrecv.h"
+
+namespace {
+
+constexpr uint32_t kPiece = 256u << 10;  /* a long write is cut so that no wavefront copies more */
+constexpr uint32_t kRxStride = 8320;     /* 8192 + header room, rounded to the 128-byte rx alignment */
+constexpr int64_t kEagerSendSize = 8192; /* OFI_NCCL_EAGER_MAX_SIZE default, src/nccl_ofi_rdma.cpp:6808 */
+
+struct pinned_t {
+	void *host = nullptr;
+	void *dev = nullptr;
+	int alloc(size_t bytes)
+	{
+		int rc = ofi_amd_gpu_host_alloc(&host, bytes ? bytes : 8);
+		return rc ? rc : ofi_amd_gpu_host_get_device_pointer(&dev, host);
+	}
+	void release()
+	{
+		if (host) {
+			(void)ofi_amd_gpu_host_free(host);
+		}
+		host = dev = nullptr;
+	}
+	template <typename T> T *as() { return static_cast<T *>(host); }
+	template <typename T> const T *dev_as() const { return static_cast<const T *>(dev); }
+};
+
+struct open_msg_t {
+	uint64_t index;
+	int32_t send_req = -1;
+	int32_t recv_req = -1;
+	ofi_amd_send_action_t action;
+	bool sent = false;
+};
+
+uint64_t pieces_of(uint64_t bytes)
+{
+	return bytes == 0 ? 1 : (bytes + kPiece - 1) / kPiece;
+}
+
+} // namespace
+
+extern "C" int ofi_amd_sendrecv_loopback_run(const uint64_t *src_addrs, const uint64_t *dst_addrs,
+					     const uint64_t *sizes, const uint64_t *dst_sizes,
+					     const int32_t *tags, uint64_t n_msgs, uint32_t inflight,
+					     uint32_t num_rails, void *rx_pool, uint64_t rx_pool_bytes,
+					     uint32_t flags, void *stream,
+					     ofi_amd_sendrecv_loopback_stats_t *stats)
+{
+	if (!src_addrs || !dst_addrs || !sizes || !dst_sizes || !rx_pool || !stats || inflight == 0 ||
+	    inflight > OFI_AMD_MAX_REQUESTS || num_rails < 1 || num_rails > OFI_AMD_WIRE_MAX_RAILS ||
+	    rx_pool_bytes < (uint64_t)inflight * kRxStride) {
+		return -EINVAL;
+	}
+	for (uint64_t i = 0; i < n_msgs; i++) {
+		if (sizes[i] > 0xFFFFFFFFull || dst_sizes[i] > 0xFFFFFFFFull) {
+			return -EMSGSIZE; /* the control message carries a 32-bit length */
+		}
+	}
+	using clock = std::chrono::steady_clock;
+	ofi_amd_sendrecv_loopback_stats_t st;
+	std::memset(&st, 0, sizeof(st));
+
+	/* table room for the fullest round */
+	uint64_t cap_copy = 0;
+	for (uint64_t lo = 0; lo < n_msgs; lo += inflight) {
+		uint64_t need = 0;
+		for (uint64_t i = lo; i < n_msgs && i < lo + inflight; i++) {
+			need += pieces_of(sizes[i]) + OFI_AMD_WIRE_MAX_RAILS + 2;
+		}
+		cap_copy = need > cap_copy ? need : cap_copy;
+	}
+	if (cap_copy > (1ull << 30)) {
+		return -EINVAL;
+	}
+
+	ofi_amd_send_comm_t *sc = nullptr;
+	ofi_amd_recv_comm_t *rcv = nullptr;
+	pinned_t t_src, t_dst, t_len, hdrs, e_rx, e_len, e_dst, e_cap, e_copied;
+	std::vector<open_msg_t> open;
+	std::vector<ofi_amd_eager_copy_item_t> items;
+	int rc = ofi_amd_send_comm_create(1, num_rails, kEagerSendSize, 131072, 64, &sc);
+	if (rc == 0) rc = ofi_amd_recv_comm_create(num_rails, &rcv);
+	if (rc == 0) rc = t_src.alloc(sizeof(uint64_t) * cap_copy);
+	if (rc == 0) rc = t_dst.alloc(sizeof(uint64_t) * cap_copy);
+	if (rc == 0) rc = t_len.alloc(sizeof(uint32_t) * cap_copy);
+	if (rc == 0) rc = hdrs.alloc(sizeof(ofi_amd_eager_hdr_t) * inflight);
+	if (rc == 0) rc = e_rx.alloc(sizeof(uint64_t) * inflight);
+	if (rc == 0) rc = e_len.alloc(sizeof(uint32_t) * inflight);
+	if (rc == 0) rc = e_dst.alloc(sizeof(uint64_t) * inflight);
+	if (rc == 0) rc = e_cap.alloc(sizeof(uint32_t) * inflight);
+	if (rc == 0) rc = e_copied.alloc(sizeof(uint32_t) * inflight);
+	try {
+		open.reserve(inflight);
+		items.resize(inflight);
+	} catch (...) {
+		rc = rc ? rc : -ENOMEM;
+	}
+	auto release = [&]() {
+		for (pinned_t *p : { &t_src, &t_dst, &t_len, &hdrs, &e_rx, &e_len, &e_dst, &e_cap, &e_copied }) {
+			p->release();
+		}
+		if (sc) (void)ofi_amd_send_comm_destroy(sc);
+		if (rcv) (void)ofi_amd_recv_comm_destroy(rcv);
+	};
+	if (rc != 0) {
+		release();
+		return rc;
+	}
+	ofi_amd_ctrl_msg_t *mailbox = ofi_amd_send_comm_mailbox(sc);
+	const bool receiver_first = (flags & 1u) != 0;
+	const auto t0 = clock::now();
+
+	for (uint64_t lo = 0; lo < n_msgs && rc == 0; lo += inflight) {
+		const uint64_t hi = lo + inflight < n_msgs ? lo + inflight : n_msgs;
+		open.clear();
+
+		/* ---- both ranks post: the sender first unless told otherwise, so that whatever fits
+		 * goes eager ahead of its control message; the rest waits for the receive ---- */
+		for (uint64_t i = lo; i < hi && rc == 0; i++) {
+			open_msg_t m;
+			m.index = i;
+			const int32_t tag = tags ? tags[i] : 1;
+			if (!receiver_first) {
+				rc = ofi_amd_send_comm_send(sc, sizes[i], tag, &m.action);
+				m.sent = rc == 0 && m.action.kind != OFI_AMD_SEND_AGAIN;
+				st.send_again += rc == 0 && !m.sent;
+			}
+			if (rc == 0) {
+				const uint64_t keys[OFI_AMD_WIRE_MAX_RAILS] = { i, i, i, i };
+				const int tg = tag;
+				uint16_t seq = 0;
+				rc = ofi_amd_recv_comm_recv(rcv, 1, &dst_addrs[i], &dst_sizes[i], &tg, keys, 0, mailbox,
+							    &m.recv_req, &seq);
+				/* the control message is in the sender's mailbox: its post is complete */
+				if (rc == 0) rc = ofi_amd_recv_comm_ctrl_sent(rcv, m.recv_req);
+			}
+			if (rc == 0 && !m.sent) {
+				rc = ofi_amd_send_comm_send(sc, sizes[i], tag, &m.action);
+				if (rc == 0 && m.action.kind == OFI_AMD_SEND_AGAIN) {
+					rc = -EPROTO; /* its control message is there: the send must go */
+				}
+				m.sent = rc == 0;
+			}
+			if (rc == 0) {
+				m.send_req = m.action.req;
+				open.push_back(m);
+			}
+		}
+		if (rc != 0) {
+			break;
+		}
+
+		/* ---- the wire: one table of device copies for everything the sender handed out ---- */
+		uint64_t *src = t_src.as<uint64_t>(), *dst = t_dst.as<uint64_t>();
+		uint32_t *len = t_len.as<uint32_t>();
+		uint32_t n_copy = 0, n_eager = 0;
+		for (open_msg_t &m : open) {
+			const ofi_amd_send_action_t &a = m.action;
+			if (a.kind == OFI_AMD_SEND_EAGER) {
+				const uint64_t slot = reinterpret_cast<uint64_t>(rx_pool) + (uint64_t)n_eager * kRxStride;
+				hdrs.as<ofi_amd_eager_hdr_t>()[n_eager] = a.hdr;
+				src[n_copy] = reinterpret_cast<uint64_t>(hdrs.dev) + n_eager * sizeof(ofi_amd_eager_hdr_t);
+				dst[n_copy] = slot;
+				len[n_copy++] = OFI_AMD_EAGER_HEADER_SIZE;
+				if (a.size) {
+					src[n_copy] = src_addrs[m.index];
+					dst[n_copy] = slot + OFI_AMD_EAGER_HEADER_SIZE;
+					len[n_copy++] = static_cast<uint32_t>(a.size);
+				}
+				rc = ofi_amd_recv_comm_eager_arrival(rcv, a.msg_seq_num, &a.hdr, static_cast<uint32_t>(a.size),
+								     n_eager);
+				n_eager++;
+				st.eager_messages++;
+			} else {
+				for (uint32_t k = 0; k < a.num_xfers && rc == 0; k++) {
+					const ofi_amd_xfer_info_t &x = a.xfers[k];
+					for (uint64_t off = 0; off < x.msg_size; off += kPiece) {
+						const uint64_t n = x.msg_size - off < kPiece ? x.msg_size - off : kPiece;
+						src[n_copy] = src_addrs[m.index] + x.offset + off;
+						dst[n_copy] = a.remote_buff_offset + x.offset + off;
+						len[n_copy++] = static_cast<uint32_t>(n);
+					}
+					rc = ofi_amd_recv_comm_write_arrival(rcv, a.imm, x.msg_size);
+					st.rdma_writes++;
+				}
+				st.write_messages++;
+			}
+			/* the sender's completions: the eager send, or every write of the schedule */
+			for (uint32_t k = 0; k < (a.kind == OFI_AMD_SEND_EAGER ? 1u : a.num_xfers) && rc == 0; k++) {
+				rc = ofi_amd_send_comm_completion(sc, m.send_req);
+			}
+			if (rc != 0) {
+				break;
+			}
+		}
+		if (rc == 0 && n_copy) {
+			rc = ofi_amd_copy_table(t_src.dev_as<uint64_t>(), t_dst.dev_as<uint64_t>(), t_len.dev_as<uint32_t>(),
+						n_copy, stream);
+			st.launches++;
+			st.copy_entries += n_copy;
+		}
+
+		/* ---- receiver: everything matched so far leaves the rx buffers in one launch ---- */
+		uint32_t n_items = 0;
+		if (rc == 0) {
+			n_items = ofi_amd_recv_comm_take_copies(rcv, items.data(), inflight);
+			if (n_items != n_eager) {
+				rc = -EPROTO; /* every receive of the round is posted: every arrival must match */
+			}
+		}
+		uint32_t n_ecopy = 0;
+		for (uint32_t k = 0; k < n_items && rc == 0; k++) {
+			if (!items[k].needs_copy) {
+				continue;
+			}
+			e_rx.as<uint64_t>()[n_ecopy] = items[k].rx_cookie * kRxStride;
+			e_len.as<uint32_t>()[n_ecopy] = items[k].recv_len;
+			e_dst.as<uint64_t>()[n_ecopy] = items[k].dst;
+			e_cap.as<uint32_t>()[n_ecopy] = static_cast<uint32_t>(items[k].dst_len);
+			n_ecopy++;
+		}
+		if (rc == 0 && n_ecopy) {
+			rc = ofi_amd_eager_copy_batch(rx_pool, e_rx.dev_as<uint64_t>(), e_len.dev_as<uint32_t>(), nullptr,
+						      e_dst.dev_as<uint64_t>(), e_cap.dev_as<uint32_t>(), n_ecopy,
+						      static_cast<uint32_t *>(e_copied.dev), nullptr, stream);
+			st.launches++;
+		}
+		if (rc == 0) rc = ofi_amd_gpu_stream_synchronize(stream);
+		for (uint32_t k = 0, j = 0; k < n_items && rc == 0; k++) {
+			if (!items[k].needs_copy) {
+				continue;
+			}
+			const uint32_t want = items[k].recv_len < items[k].dst_len ? items[k].recv_len
+										    : static_cast<uint32_t>(items[k].dst_len);
+			if (e_copied.as<uint32_t>()[j++] != want) {
+				rc = -EIO;
+				break;
+			}
+			rc = ofi_amd_recv_comm_copy_done(rcv, items[k].req, items[k].sub_idx);
+		}
+
+		/* ---- both ranks test their requests: all of the round must be complete ---- */
+		for (open_msg_t &m : open) {
+			if (rc != 0) {
+				break;
+			}
+			int done = 0, rsize = 0;
+			uint64_t ssize = 0;
+			rc = ofi_amd_send_comm_test(sc, m.send_req, &done, &ssize);
+			if (rc == 0 && !done) rc = -EPROTO;
+			if (rc == 0) rc = ofi_amd_recv_comm_test(rcv, m.recv_req, &done, &rsize);
+			if (rc == 0 && !done) rc = -EPROTO;
+			const uint64_t moved = sizes[m.index] < dst_sizes[m.index] ? sizes[m.index] : dst_sizes[m.index];
+			if (rc == 0 && ssize != moved) rc = -EIO;
+			st.payload_bytes += moved;
+			st.messages++;
+		}
+		st.rounds++;
+	}
+	st.seconds = std::chrono::duration<double>(clock::now() - t0).count();
+	release();
+	*stats = st;
+	return rc;
+}

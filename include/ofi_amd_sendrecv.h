@@ -183,6 +183,40 @@ int ofi_amd_recv_comm_copy_done(ofi_amd_recv_comm_t *r, int32_t req, int32_t sub
 int ofi_amd_recv_comm_test(ofi_amd_recv_comm_t *r, int32_t req, int *done, int *sizes);
 void ofi_amd_recv_comm_state(const ofi_amd_recv_comm_t *r, ofi_amd_recv_state_t *out);
 
+/* ======================================================================
+ * The whole send/receive path in one process on one GPU.
+ *   Stands where the reference needs two ranks and a libfabric provider: the isend / irecv /
+ *   test loop of tests/functional/nccl_message_transfer.cpp:19-56 (ten send/receive size
+ *   pairs, NCCL_NET_MAX_REQUESTS requests in flight, tests/functional/functional_test.h:28).
+ *   Message i moves min(sizes[i], dst_sizes[i]) bytes from
+ *   src_addrs[i] to dst_addrs[i] (device addresses); `inflight` (1..128) messages are open at
+ *   a time.  Small messages leave as eager sends ahead of their control message (header +
+ *   payload copied into an rx buffer of rx_pool, then out of it by ofi_amd_eager_copy_batch);
+ *   the others wait for the receive and go as striped RDMA writes (ofi_amd_copy_table).
+ *   rx_pool: device-accessible memory, inflight x 8320 bytes.  flags bit 0: the receiver
+ *   posts first, so nothing goes eager.  tags may be NULL (all 1).  Blocks until done;
+ *   `stream` carries the launches.  -EPROTO if the state machines disagree with the wire,
+ *   -EIO if a size reported back is not the size moved.
+ * ====================================================================== */
+typedef struct {
+	uint64_t messages;
+	uint64_t payload_bytes;
+	uint64_t eager_messages;
+	uint64_t write_messages;
+	uint64_t rdma_writes;   /* stripes */
+	uint64_t copy_entries;  /* table entries of the wire launches (stripes cut to 256 KiB) */
+	uint64_t rounds;
+	uint64_t launches;
+	uint64_t send_again;    /* isend calls answered "call again" */
+	double seconds;
+} ofi_amd_sendrecv_loopback_stats_t;
+
+int ofi_amd_sendrecv_loopback_run(const uint64_t *src_addrs, const uint64_t *dst_addrs,
+				  const uint64_t *sizes, const uint64_t *dst_sizes, const int32_t *tags,
+				  uint64_t n_msgs, uint32_t inflight, uint32_t num_rails, void *rx_pool,
+				  uint64_t rx_pool_bytes, uint32_t flags, void *stream,
+				  ofi_amd_sendrecv_loopback_stats_t *stats);
+
 #ifdef __cplusplus
 }
 #endif

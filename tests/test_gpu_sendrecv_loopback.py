@@ -1,0 +1,102 @@
+"""The send/receive path end to end in one process on one GPU (ofi_amd_sendrecv_loopback_run):
+send comm and receive comm state machines, eager sends through rx buffers and the batched eager
+copy, rendezvous as striped device copies.  Checked byte for byte against the source buffers.
+
+Sizes: the ten (send, receive) pairs of the reference's tests/functional/
+nccl_message_transfer.cpp:44-56 with NCCL_NET_MAX_REQUESTS = 32 requests each, and the
+powers of two of the configured sweep (8 B up; 64 MiB here) with 64 in flight."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import _gpu
+import aws_ofi_nccl_amd as m
+
+pytestmark = pytest.mark.gpu
+
+RX_STRIDE = 8320
+PAIRS = [(512, 512), (4096, 4096), (16384, 16384), (1 << 20, 1 << 20), (5120, 4096), (17408, 16384),
+         (2 << 20, 1 << 20), (4096, 5120), (16384, 17408), (1 << 20, 2 << 20)]
+
+
+def run(lib, send_sizes, recv_sizes, inflight, flags=0, dst_skew=0, seed=0):
+    """Distinct source and receive buffers per message; returns (stats, per-message check)."""
+    n = len(send_sizes)
+    rng = np.random.default_rng(seed)
+    srcs = [torch.from_numpy(rng.integers(0, 256, max(s, 1), dtype=np.uint8)).cuda() for s in send_sizes]
+    dsts = [torch.full((max(r, 1) + 64,), 0xCD, dtype=torch.uint8, device="cuda") for r in recv_sizes]
+    pool = torch.zeros(inflight * RX_STRIDE, dtype=torch.uint8, device="cuda")
+    a_src = np.array([t.data_ptr() for t in srcs], dtype=np.uint64)
+    a_dst = np.array([t.data_ptr() + dst_skew for t in dsts], dtype=np.uint64)
+    a_size = np.array(send_sizes, dtype=np.uint64)
+    a_cap = np.array(recv_sizes, dtype=np.uint64)
+    stats = m.SendrecvLoopbackStats()
+    torch.cuda.synchronize()
+    rc = lib.ofi_amd_sendrecv_loopback_run(a_src.ctypes.data, a_dst.ctypes.data, a_size.ctypes.data,
+                                           a_cap.ctypes.data, None, n, inflight, 4, pool.data_ptr(),
+                                           pool.numel(), flags, _gpu.stream(), ctypes.byref(stats))
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    for i in range(n):
+        k = min(send_sizes[i], recv_sizes[i])
+        got = dsts[i].cpu().numpy()
+        want = srcs[i].cpu().numpy()
+        assert np.array_equal(got[dst_skew:dst_skew + k], want[:k]), (i, send_sizes[i], recv_sizes[i])
+        assert np.all(got[:dst_skew] == 0xCD) and np.all(got[dst_skew + k:] == 0xCD), (i, "wrote outside")
+    assert stats.messages == n and stats.payload_bytes == sum(min(s, r) for s, r in zip(send_sizes, recv_sizes))
+    assert stats.eager_messages + stats.write_messages == n
+    return stats
+
+
+@pytest.mark.parametrize("pair", PAIRS)
+def test_reference_size_pairs_thirty_two_requests_each(lib, gpu, pair):
+    send, recv = pair
+    st = run(lib, [send] * 32, [recv] * 32, 32, seed=send + recv)
+    if send + 8 <= 8192:
+        assert st.eager_messages >= 1                # the sender was ahead of the receiver
+    else:
+        assert st.eager_messages == 0 and st.write_messages == 32
+
+
+def test_power_of_two_sweep_sixty_four_in_flight(lib, gpu):
+    sizes = [8 << k for k in range(24)]                       # 8 B .. 64 MiB
+    for size in sizes:
+        count = 64 if size <= (1 << 20) else max(2, (128 << 20) // size)
+        st = run(lib, [size] * count, [size] * count, 64, seed=size)
+        stripes = 1 if size <= 131072 else (2 if size <= 262144 else 4)
+        if size + 8 > 8192:
+            assert st.rdma_writes == count * stripes
+
+
+def test_receiver_first_sends_everything_as_writes(lib, gpu):
+    sizes = [8, 100, 1024, 8184, 8185, 70000, 300000, 1 << 20] * 8
+    st = run(lib, sizes, sizes, 64, flags=1, seed=3)
+    assert st.eager_messages == 0 and st.write_messages == len(sizes) and st.send_again == 0
+
+
+def test_mixed_sizes_unaligned_receive_buffers_and_zero_length(lib, gpu):
+    rng = np.random.default_rng(11)
+    sizes = [int(s) for s in rng.choice([0, 1, 7, 8, 63, 64, 1000, 8184, 8185, 9000, 131072, 131073, 524289], 192)]
+    caps = [s if rng.random() < 0.7 else max(s // 3, 1) for s in sizes]
+    st = run(lib, sizes, caps, 64, dst_skew=5, seed=12)
+    assert st.eager_messages > 0 and st.write_messages > 0 and st.rounds == 3
+
+
+def test_rejects_bad_arguments(lib, gpu):
+    pool = torch.zeros(64 * RX_STRIDE, dtype=torch.uint8, device="cuda")
+    one = np.array([pool.data_ptr()], dtype=np.uint64)
+    size = np.array([8], dtype=np.uint64)
+    big = np.array([1 << 32], dtype=np.uint64)
+    stats = m.SendrecvLoopbackStats()
+    call = lib.ofi_amd_sendrecv_loopback_run
+    p = lambda a: a.ctypes.data
+    assert call(p(one), p(one), p(size), p(size), None, 1, 0, 4, pool.data_ptr(), pool.numel(), 0,
+                _gpu.stream(), ctypes.byref(stats)) == -22          # nothing in flight
+    assert call(p(one), p(one), p(size), p(size), None, 1, 129, 4, pool.data_ptr(), pool.numel(), 0,
+                _gpu.stream(), ctypes.byref(stats)) == -22          # more than the receiver allows
+    assert call(p(one), p(one), p(size), p(size), None, 1, 64, 4, pool.data_ptr(), 1000, 0,
+                _gpu.stream(), ctypes.byref(stats)) == -22          # rx pool too small
+    assert call(p(one), p(one), p(big), p(big), None, 1, 64, 4, pool.data_ptr(), pool.numel(), 0,
+                _gpu.stream(), ctypes.byref(stats)) == -90          # -EMSGSIZE: 32-bit control length
