@@ -489,14 +489,79 @@ def bench_gin(lib, oracle, torch, np, args):
     return out
 
 
+def bench_sendrecv(lib, oracle, torch, np, args):
+    """The send/receive path in one process: sizes 8 B .. 1 GiB in powers of two, 64 messages in
+    flight, bf16 payloads (random 16-bit words), 4 rails.  Both state machines run on the host;
+    eager sends and RDMA writes are executed as device copies by the library."""
+    import _gpu
+    import aws_ofi_nccl_amd as m
+    inflight, stride = 64, 8320
+    top = args.sendrecv_max_bytes
+    # one source and one receive buffer per message in flight (a shared source would be served from
+    # the last-level cache and overstate the rate): 2 x 64 GiB at the full sweep
+    src = torch.empty(inflight * top // 2, dtype=torch.int16, device="cuda")
+    for k in range(inflight):
+        src[k * (top // 2):(k + 1) * (top // 2)].random_(-32768, 32767)
+    dst = torch.empty(inflight * top, dtype=torch.uint8, device="cuda")
+    pool = torch.zeros(inflight * stride, dtype=torch.uint8, device="cuda")
+    out = {"inflight": inflight, "rails": 4, "sizes": []}
+    size = 8
+    while size <= top:
+        rounds = 32 if size <= (1 << 20) else (4 if size <= (64 << 20) else 1)
+        n = inflight * rounds
+        a_src = np.array([src.data_ptr() + (i % inflight) * top for i in range(n)], dtype=np.uint64)
+        a_dst = np.array([dst.data_ptr() + (i % inflight) * top for i in range(n)], dtype=np.uint64)
+        a_size = np.full(n, size, dtype=np.uint64)
+        stats = m.SendrecvLoopbackStats()
+        best = None
+        for _ in range(2):                                       # first pass warms up
+            torch.cuda.synchronize()
+            rc = lib.ofi_amd_sendrecv_loopback_run(a_src.ctypes.data, a_dst.ctypes.data, a_size.ctypes.data,
+                                                   a_size.ctypes.data, None, n, inflight, 4, pool.data_ptr(),
+                                                   pool.numel(), 0, _gpu.stream(), ctypes.byref(stats))
+            if rc != 0:
+                raise RuntimeError("sendrecv loopback rc=%d at %d bytes" % (rc, size))
+            best = stats.seconds if best is None else min(best, stats.seconds)
+        ok = all(bool(torch.equal(dst[k * top:k * top + size], src.view(torch.uint8)[k * top:k * top + size]))
+                 for k in (0, inflight // 2, inflight - 1))
+        out["sizes"].append({"bytes": size, "messages": n, "msgs_per_s": n / best,
+                             "payload_gbs": n * size / best / 1e9,
+                             "read_plus_written_gbs": 2 * n * size / best / 1e9, "eager": stats.eager_messages,
+                             "writes": stats.rdma_writes, "parity_ok": ok})
+        size *= 2
+    out["parity_ok"] = all(s["parity_ok"] for s in out["sizes"])
+    out["peak_payload_gbs"] = max(s["payload_gbs"] for s in out["sizes"])
+    out["peak_msgs_per_s"] = max(s["msgs_per_s"] for s in out["sizes"])
+    # the same harness with host buffers (pinned, read and written in place over the host link)
+    if not args.skip_cpu:
+        hsize, hn = 1 << 20, inflight * 4
+        h_src = torch.randint(0, 255, (hsize,), dtype=torch.uint8).pin_memory()
+        h_dst = torch.empty(inflight * hsize, dtype=torch.uint8, pin_memory=True)
+        a_src = np.full(hn, h_src.data_ptr(), dtype=np.uint64)
+        a_dst = np.array([h_dst.data_ptr() + (i % inflight) * hsize for i in range(hn)], dtype=np.uint64)
+        a_size = np.full(hn, hsize, dtype=np.uint64)
+        stats = m.SendrecvLoopbackStats()
+        rc = lib.ofi_amd_sendrecv_loopback_run(a_src.ctypes.data, a_dst.ctypes.data, a_size.ctypes.data,
+                                               a_size.ctypes.data, None, hn, inflight, 4, pool.data_ptr(),
+                                               pool.numel(), 0, _gpu.stream(), ctypes.byref(stats))
+        if rc != 0:
+            raise RuntimeError("sendrecv loopback (host buffers) rc=%d" % rc)
+        out["host_buffers_1MiB"] = {"payload_gbs": hn * hsize / stats.seconds / 1e9,
+                                    "parity_ok": bool(torch.equal(h_dst[:hsize], h_src))}
+    del src, dst, pool
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--gin-ops", type=int, default=1_000_000, help="GIN ops per context")
+    ap.add_argument("--sendrecv-max-bytes", type=int, default=1 << 30, help="largest message of the send/receive sweep")
     ap.add_argument("--skip-extra", action="store_true", help="only the bounce-copy step")
-    ap.add_argument("--extra", default="eager,striping,tuner,gin", help="which other paths to time")
+    ap.add_argument("--extra", default="eager,striping,tuner,gin,sendrecv", help="which other paths to time")
     ap.add_argument("--skip-cpu", action="store_true", help="no CPU baselines")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -520,7 +585,8 @@ def main():
     bounce, cpu = bench_bounce(lib, oracle, torch, np, args)
     extra = {}
     if not args.skip_extra:
-        for name, fn in (("eager", bench_eager), ("striping", bench_sched), ("tuner", bench_tuner), ("gin", bench_gin)):
+        for name, fn in (("eager", bench_eager), ("striping", bench_sched), ("tuner", bench_tuner), ("gin", bench_gin),
+                         ("sendrecv", bench_sendrecv)):
             if name not in args.extra.split(","):
                 continue
             log(name)
