@@ -24,6 +24,7 @@
  *                           totals of the tiles before it by itself (at most 16 KiB
  *                           from L2) instead of waiting for a scan launch, and the
  *                           last workgroup writes the new counters back.
+ * A tile is 512 messages for batches up to 2^21 messages and 2048 beyond.
  *
  * HBM traffic per message: 8 B read twice + 4 B + 96 B written.
  */
@@ -38,8 +39,12 @@ namespace {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr uint32_t kThreads = 256;
-constexpr uint32_t kPasses = 4;
-constexpr uint32_t kTile = kThreads * kPasses; /* messages per workgroup */
+/* Messages per workgroup = kThreads * PASSES.  Small batches want many small tiles (the
+ * launch is short, so ramp-up and tail dominate: 1,000,000 messages take 26.7 us with two
+ * passes per workgroup against 29.4 with four); large ones want fewer, longer workgroups
+ * (16,000,000: 348 us with eight passes against 360 with four). */
+constexpr uint32_t kPassesSmall = 2, kPassesLarge = 8;
+constexpr uint64_t kSmallBatch = 1ull << 21;
 constexpr uint32_t kScanThreads = 1024;
 constexpr uint64_t kMaxBatch = 1ull << 28;
 /* residues are < 4, so packed 16-bit sums over this many tiles cannot overflow */
@@ -132,6 +137,7 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, uint32_t lan
 	return v;
 }
 
+template <uint32_t PASSES>
 __global__ __launch_bounds__(kThreads) void stripe_count_kernel(
 	const uint64_t *__restrict__ sizes, uint32_t n, const ofi_amd_sched_state_t *__restrict__ state,
 	uint64_t align, uint32_t *__restrict__ tile_totals, uint32_t *__restrict__ seed0,
@@ -148,10 +154,10 @@ __global__ __launch_bounds__(kThreads) void stripe_count_kernel(
 	if (blockIdx.x == 0 && threadIdx.x == 0) {
 		*seed0 = ((state->rr_small_counter % p.num_rails) << 16) | (state->rr_counter % p.num_rails);
 	}
-	const uint32_t base = blockIdx.x * kTile;
+	const uint32_t base = blockIdx.x * (kThreads * PASSES);
 	uint32_t acc = 0;
 #pragma unroll
-	for (uint32_t pass = 0; pass < kPasses; pass++) {
+	for (uint32_t pass = 0; pass < PASSES; pass++) {
 		uint32_t i = base + pass * kThreads + threadIdx.x;
 		if (i < n) {
 			uint32_t k;
@@ -232,7 +238,7 @@ __global__ __launch_bounds__(kScanThreads) void stripe_scan_kernel(
 
 /* INLINE: tile_prefix holds the per-tile totals (residues) and *seed0 the batch's seed;
  * otherwise tile_prefix holds each tile's finished seed. */
-template <bool INLINE>
+template <bool INLINE, uint32_t PASSES>
 __global__ __launch_bounds__(kThreads) void stripe_emit_kernel(
 	const uint64_t *__restrict__ sizes, uint32_t n, ofi_amd_sched_state_t *__restrict__ state,
 	uint64_t align, const uint32_t *__restrict__ tile_prefix, const uint32_t *__restrict__ seed0,
@@ -246,7 +252,7 @@ __global__ __launch_bounds__(kThreads) void stripe_emit_kernel(
 	__shared__ u32x4 rows[kThreads * 6];
 	__shared__ uint32_t wave_sum[kThreads / 64];
 	const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-	const uint32_t base = blockIdx.x * kTile;
+	const uint32_t base = blockIdx.x * (kThreads * PASSES);
 	const uint32_t R = p.num_rails;
 
 	uint32_t seed;
@@ -272,7 +278,7 @@ __global__ __launch_bounds__(kThreads) void stripe_emit_kernel(
 	}
 	uint32_t carry_small = seed >> 16, carry_big = seed & 0xffffu; /* both < R */
 
-	for (uint32_t pass = 0; pass < kPasses; pass++) {
+	for (uint32_t pass = 0; pass < PASSES; pass++) {
 		const uint32_t first = base + pass * kThreads;
 		if (first >= n) {
 			break;
@@ -368,6 +374,29 @@ struct workspace_t {
 std::mutex g_ws_lock;
 std::unordered_map<void *, workspace_t> g_ws_by_stream;
 
+uint32_t pick_passes(uint64_t n)
+{
+	return n <= kSmallBatch ? kPassesSmall : kPassesLarge;
+}
+
+template <uint32_t PASSES>
+void launch_batch(hipStream_t s, uint32_t tiles, const uint64_t *d_sizes, uint32_t n,
+		  ofi_amd_sched_state_t *d_state, uint64_t align, uint32_t *totals, uint32_t *prefix,
+		  uint32_t *seed0, uint32_t *d_num_xfers, u32x4 *d_xfers, uint32_t *err)
+{
+	hipLaunchKernelGGL(stripe_count_kernel<PASSES>, dim3(tiles), dim3(kThreads), 0, s, d_sizes, n, d_state,
+			   align, totals, seed0, err);
+	if (tiles <= kInlineTiles) {
+		hipLaunchKernelGGL((stripe_emit_kernel<true, PASSES>), dim3(tiles), dim3(kThreads), 0, s, d_sizes, n,
+				   d_state, align, totals, seed0, d_num_xfers, d_xfers);
+	} else {
+		hipLaunchKernelGGL(stripe_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, totals, tiles, d_state,
+				   prefix, err);
+		hipLaunchKernelGGL((stripe_emit_kernel<false, PASSES>), dim3(tiles), dim3(kThreads), 0, s, d_sizes, n,
+				   d_state, align, prefix, seed0, d_num_xfers, d_xfers);
+	}
+}
+
 } // namespace
 
 using namespace ofi_amd;
@@ -397,7 +426,8 @@ int ofi_amd_sched_batch(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes,
 		return -ENOMEM;
 	}
 
-	const uint32_t tiles = (uint32_t)((n + kTile - 1) / kTile);
+	const uint32_t passes = pick_passes(n);
+	const uint32_t tiles = (uint32_t)((n + kThreads * passes - 1) / (kThreads * passes));
 	uint32_t *totals, *prefix, *seed0;
 	hipStream_t s = as_stream(stream);
 	try {
@@ -426,18 +456,12 @@ int ofi_amd_sched_batch(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes,
 		return -ENOMEM;
 	}
 
-	hipLaunchKernelGGL(stripe_count_kernel, dim3(tiles), dim3(kThreads), 0, s, d_sizes,
-			   (uint32_t)n, d_state, align, totals, seed0, err);
-	if (tiles <= kInlineTiles) {
-		hipLaunchKernelGGL(stripe_emit_kernel<true>, dim3(tiles), dim3(kThreads), 0, s, d_sizes,
-				   (uint32_t)n, d_state, align, totals, seed0, d_num_xfers,
-				   reinterpret_cast<u32x4 *>(d_xfers));
+	if (passes == kPassesSmall) {
+		launch_batch<kPassesSmall>(s, tiles, d_sizes, (uint32_t)n, d_state, align, totals, prefix, seed0,
+					   d_num_xfers, reinterpret_cast<u32x4 *>(d_xfers), err);
 	} else {
-		hipLaunchKernelGGL(stripe_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, totals, tiles,
-				   d_state, prefix, err);
-		hipLaunchKernelGGL(stripe_emit_kernel<false>, dim3(tiles), dim3(kThreads), 0, s, d_sizes,
-				   (uint32_t)n, d_state, align, prefix, seed0, d_num_xfers,
-				   reinterpret_cast<u32x4 *>(d_xfers));
+		launch_batch<kPassesLarge>(s, tiles, d_sizes, (uint32_t)n, d_state, align, totals, prefix, seed0,
+					   d_num_xfers, reinterpret_cast<u32x4 *>(d_xfers), err);
 	}
 	OFI_AMD_HIP_TRY(hipGetLastError());
 	return 0;
