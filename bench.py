@@ -497,6 +497,9 @@ def bench_sendrecv(lib, oracle, torch, np, args):
     import aws_ofi_nccl_amd as m
     inflight, stride = 64, 8320
     top = args.sendrecv_max_bytes
+    free_bytes, _ = torch.cuda.mem_get_info()
+    while top > (1 << 20) and 2 * inflight * top + (8 << 30) > free_bytes:
+        top //= 2                                  # the sweep stops where the buffers no longer fit
     # one source and one receive buffer per message in flight (a shared source would be served from
     # the last-level cache and overstate the rate): 2 x 64 GiB at the full sweep
     src = torch.empty(inflight * top // 2, dtype=torch.int16, device="cuda")
@@ -504,7 +507,7 @@ def bench_sendrecv(lib, oracle, torch, np, args):
         src[k * (top // 2):(k + 1) * (top // 2)].random_(-32768, 32767)
     dst = torch.empty(inflight * top, dtype=torch.uint8, device="cuda")
     pool = torch.zeros(inflight * stride, dtype=torch.uint8, device="cuda")
-    out = {"inflight": inflight, "rails": 4, "sizes": []}
+    out = {"inflight": inflight, "rails": 4, "largest_message": top, "sizes": []}
     size = 8
     while size <= top:
         rounds = 32 if size <= (1 << 20) else (4 if size <= (64 << 20) else 1)
