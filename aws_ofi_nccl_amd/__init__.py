@@ -370,8 +370,8 @@ PROTOTYPES = {
     "ofi_amd_recv_comm_test": (ctypes.c_int, [c_vp, c_i32, ctypes.POINTER(ctypes.c_int),
                                               ctypes.POINTER(ctypes.c_int)]),
     "ofi_amd_recv_comm_state": (None, [c_vp, ctypes.POINTER(RecvState)]),
-    "ofi_amd_sendrecv_loopback_run": (ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_u64, c_u32, c_u32, c_vp,
-                                                     c_u64, c_u32, c_vp,
+    "ofi_amd_sendrecv_loopback_run": (ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_u64, c_u32, c_u32, c_u32,
+                                                     c_vp, c_u64, c_u32, c_vp,
                                                      ctypes.POINTER(SendrecvLoopbackStats)]),
     "ofi_amd_tuner_plan_create": (ctypes.c_int, [c_vp, c_u32, c_vp, c_u32, c_vp, c_u32, c_vp,
                                                  c_u32, c_vp, c_u32, ctypes.POINTER(c_vp)]),

@@ -43,6 +43,8 @@ struct open_msg_t {
 	uint64_t index;
 	int32_t send_req = -1;
 	int32_t recv_req = -1;
+	int32_t sub_idx = 0;
+	uint32_t group_size = 1;
 	ofi_amd_send_action_t action;
 	bool sent = false;
 };
@@ -57,13 +59,13 @@ uint64_t pieces_of(uint64_t bytes)
 extern "C" int ofi_amd_sendrecv_loopback_run(const uint64_t *src_addrs, const uint64_t *dst_addrs,
 					     const uint64_t *sizes, const uint64_t *dst_sizes,
 					     const int32_t *tags, uint64_t n_msgs, uint32_t inflight,
-					     uint32_t num_rails, void *rx_pool, uint64_t rx_pool_bytes,
-					     uint32_t flags, void *stream,
+					     uint32_t num_rails, uint32_t group, void *rx_pool,
+					     uint64_t rx_pool_bytes, uint32_t flags, void *stream,
 					     ofi_amd_sendrecv_loopback_stats_t *stats)
 {
 	if (!src_addrs || !dst_addrs || !sizes || !dst_sizes || !rx_pool || !stats || inflight == 0 ||
 	    inflight > OFI_AMD_MAX_REQUESTS || num_rails < 1 || num_rails > OFI_AMD_WIRE_MAX_RAILS ||
-	    rx_pool_bytes < (uint64_t)inflight * kRxStride) {
+	    group < 1 || group > OFI_AMD_WIRE_MAX_RECVS || rx_pool_bytes < (uint64_t)inflight * kRxStride) {
 		return -EINVAL;
 	}
 	for (uint64_t i = 0; i < n_msgs; i++) {
@@ -129,36 +131,49 @@ extern "C" int ofi_amd_sendrecv_loopback_run(const uint64_t *src_addrs, const ui
 		const uint64_t hi = lo + inflight < n_msgs ? lo + inflight : n_msgs;
 		open.clear();
 
-		/* ---- both ranks post: the sender first unless told otherwise, so that whatever fits
-		 * goes eager ahead of its control message; the rest waits for the receive ---- */
-		for (uint64_t i = lo; i < hi && rc == 0; i++) {
-			open_msg_t m;
-			m.index = i;
-			const int32_t tag = tags ? tags[i] : 1;
-			if (!receiver_first) {
-				rc = ofi_amd_send_comm_send(sc, sizes[i], tag, &m.action);
-				m.sent = rc == 0 && m.action.kind != OFI_AMD_SEND_AGAIN;
-				st.send_again += rc == 0 && !m.sent;
-			}
-			if (rc == 0) {
-				const uint64_t keys[OFI_AMD_WIRE_MAX_RAILS] = { i, i, i, i };
-				const int tg = tag;
-				uint16_t seq = 0;
-				rc = ofi_amd_recv_comm_recv(rcv, 1, &dst_addrs[i], &dst_sizes[i], &tg, keys, 0, mailbox,
-							    &m.recv_req, &seq);
-				/* the control message is in the sender's mailbox: its post is complete */
-				if (rc == 0) rc = ofi_amd_recv_comm_ctrl_sent(rcv, m.recv_req);
-			}
-			if (rc == 0 && !m.sent) {
-				rc = ofi_amd_send_comm_send(sc, sizes[i], tag, &m.action);
-				if (rc == 0 && m.action.kind == OFI_AMD_SEND_AGAIN) {
-					rc = -EPROTO; /* its control message is there: the send must go */
+		/* ---- both ranks post, one (grouped) receive at a time: the sender first unless told
+		 * otherwise, so that whatever fits goes eager ahead of its control message; the rest
+		 * waits for the receive.  Messages g .. g+group-1 share one receive request. ---- */
+		for (uint64_t g = lo; g < hi && rc == 0; g += group) {
+			const uint32_t gn = static_cast<uint32_t>(hi - g < group ? hi - g : group);
+			const size_t first = open.size();
+			int gtags[OFI_AMD_WIRE_MAX_RECVS];
+			uint64_t keys[OFI_AMD_WIRE_MAX_RECVS * OFI_AMD_WIRE_MAX_RAILS];
+			for (uint32_t k = 0; k < gn && rc == 0; k++) {
+				open_msg_t m;
+				m.index = g + k;
+				gtags[k] = tags ? tags[g + k] : static_cast<int>(1 + k);
+				for (uint32_t r = 0; r < num_rails; r++) {
+					keys[k * num_rails + r] = g + k;
 				}
-				m.sent = rc == 0;
-			}
-			if (rc == 0) {
-				m.send_req = m.action.req;
+				if (!receiver_first) {
+					rc = ofi_amd_send_comm_send(sc, sizes[g + k], gtags[k], &m.action);
+					m.sent = rc == 0 && m.action.kind != OFI_AMD_SEND_AGAIN;
+					st.send_again += rc == 0 && !m.sent;
+				}
 				open.push_back(m);
+			}
+			int32_t recv_req = -1;
+			if (rc == 0) {
+				uint16_t seq = 0;
+				rc = ofi_amd_recv_comm_recv(rcv, static_cast<int>(gn), &dst_addrs[g], &dst_sizes[g], gtags, keys, 0,
+							    mailbox, &recv_req, &seq);
+				/* the control message is in the sender's mailbox: its post is complete */
+				if (rc == 0) rc = ofi_amd_recv_comm_ctrl_sent(rcv, recv_req);
+			}
+			for (uint32_t k = 0; k < gn && rc == 0; k++) {
+				open_msg_t &m = open[first + k];
+				m.recv_req = recv_req;
+				m.sub_idx = static_cast<int32_t>(k);
+				m.group_size = gn;
+				if (!m.sent) {
+					rc = ofi_amd_send_comm_send(sc, sizes[m.index], gtags[k], &m.action);
+					if (rc == 0 && m.action.kind == OFI_AMD_SEND_AGAIN) {
+						rc = -EPROTO; /* its control message is there: the send must go */
+					}
+					m.sent = rc == 0;
+				}
+				m.send_req = m.action.req;
 			}
 		}
 		if (rc != 0) {
@@ -259,12 +274,16 @@ extern "C" int ofi_amd_sendrecv_loopback_run(const uint64_t *src_addrs, const ui
 			if (rc != 0) {
 				break;
 			}
-			int done = 0, rsize = 0;
+			int done = 0;
+			int rsizes[OFI_AMD_WIRE_MAX_RECVS] = {};
 			uint64_t ssize = 0;
 			rc = ofi_amd_send_comm_test(sc, m.send_req, &done, &ssize);
 			if (rc == 0 && !done) rc = -EPROTO;
-			if (rc == 0) rc = ofi_amd_recv_comm_test(rcv, m.recv_req, &done, &rsize);
-			if (rc == 0 && !done) rc = -EPROTO;
+			if (rc == 0 && m.sub_idx == static_cast<int32_t>(m.group_size) - 1) {
+				/* the group's last message: the receive request is complete with it */
+				rc = ofi_amd_recv_comm_test(rcv, m.recv_req, &done, rsizes);
+				if (rc == 0 && !done) rc = -EPROTO;
+			}
 			const uint64_t moved = sizes[m.index] < dst_sizes[m.index] ? sizes[m.index] : dst_sizes[m.index];
 			if (rc == 0 && ssize != moved) rc = -EIO;
 			st.payload_bytes += moved;

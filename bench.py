@@ -520,7 +520,7 @@ def bench_sendrecv(lib, oracle, torch, np, args):
         for _ in range(2):                                       # first pass warms up
             torch.cuda.synchronize()
             rc = lib.ofi_amd_sendrecv_loopback_run(a_src.ctypes.data, a_dst.ctypes.data, a_size.ctypes.data,
-                                                   a_size.ctypes.data, None, n, inflight, 4, pool.data_ptr(),
+                                                   a_size.ctypes.data, None, n, inflight, 4, 1, pool.data_ptr(),
                                                    pool.numel(), 0, _gpu.stream(), ctypes.byref(stats))
             if rc != 0:
                 raise RuntimeError("sendrecv loopback rc=%d at %d bytes" % (rc, size))
@@ -545,7 +545,7 @@ def bench_sendrecv(lib, oracle, torch, np, args):
         a_size = np.full(hn, hsize, dtype=np.uint64)
         stats = m.SendrecvLoopbackStats()
         rc = lib.ofi_amd_sendrecv_loopback_run(a_src.ctypes.data, a_dst.ctypes.data, a_size.ctypes.data,
-                                               a_size.ctypes.data, None, hn, inflight, 4, pool.data_ptr(),
+                                               a_size.ctypes.data, None, hn, inflight, 4, 1, pool.data_ptr(),
                                                pool.numel(), 0, _gpu.stream(), ctypes.byref(stats))
         if rc != 0:
             raise RuntimeError("sendrecv loopback (host buffers) rc=%d" % rc)

@@ -193,8 +193,10 @@ void ofi_amd_recv_comm_state(const ofi_amd_recv_comm_t *r, ofi_amd_recv_state_t 
  *   a time.  Small messages leave as eager sends ahead of their control message (header +
  *   payload copied into an rx buffer of rx_pool, then out of it by ofi_amd_eager_copy_batch);
  *   the others wait for the receive and go as striped RDMA writes (ofi_amd_copy_table).
+ *   `group` (1..8) consecutive messages share one grouped receive request, matched by tag
+ *   (tags NULL: 1..group within each request; tags given: distinct within a request).
  *   rx_pool: device-accessible memory, inflight x 8320 bytes.  flags bit 0: the receiver
- *   posts first, so nothing goes eager.  tags may be NULL (all 1).  Blocks until done;
+ *   posts first, so nothing goes eager.  Blocks until done;
  *   `stream` carries the launches.  -EPROTO if the state machines disagree with the wire,
  *   -EIO if a size reported back is not the size moved.
  * ====================================================================== */
@@ -213,8 +215,8 @@ typedef struct {
 
 int ofi_amd_sendrecv_loopback_run(const uint64_t *src_addrs, const uint64_t *dst_addrs,
 				  const uint64_t *sizes, const uint64_t *dst_sizes, const int32_t *tags,
-				  uint64_t n_msgs, uint32_t inflight, uint32_t num_rails, void *rx_pool,
-				  uint64_t rx_pool_bytes, uint32_t flags, void *stream,
+				  uint64_t n_msgs, uint32_t inflight, uint32_t num_rails, uint32_t group,
+				  void *rx_pool, uint64_t rx_pool_bytes, uint32_t flags, void *stream,
 				  ofi_amd_sendrecv_loopback_stats_t *stats);
 
 #ifdef __cplusplus

@@ -21,7 +21,7 @@ PAIRS = [(512, 512), (4096, 4096), (16384, 16384), (1 << 20, 1 << 20), (5120, 40
          (2 << 20, 1 << 20), (4096, 5120), (16384, 17408), (1 << 20, 2 << 20)]
 
 
-def run(lib, send_sizes, recv_sizes, inflight, flags=0, dst_skew=0, seed=0):
+def run(lib, send_sizes, recv_sizes, inflight, flags=0, dst_skew=0, seed=0, group=1, tags=None):
     """Distinct source and receive buffers per message; returns (stats, per-message check)."""
     n = len(send_sizes)
     rng = np.random.default_rng(seed)
@@ -34,8 +34,10 @@ def run(lib, send_sizes, recv_sizes, inflight, flags=0, dst_skew=0, seed=0):
     a_cap = np.array(recv_sizes, dtype=np.uint64)
     stats = m.SendrecvLoopbackStats()
     torch.cuda.synchronize()
+    a_tags = None if tags is None else np.array(tags, dtype=np.int32)
     rc = lib.ofi_amd_sendrecv_loopback_run(a_src.ctypes.data, a_dst.ctypes.data, a_size.ctypes.data,
-                                           a_cap.ctypes.data, None, n, inflight, 4, pool.data_ptr(),
+                                           a_cap.ctypes.data, None if tags is None else a_tags.ctypes.data, n,
+                                           inflight, 4, group, pool.data_ptr(),
                                            pool.numel(), flags, _gpu.stream(), ctypes.byref(stats))
     assert rc == 0, rc
     torch.cuda.synchronize()
@@ -84,6 +86,23 @@ def test_mixed_sizes_unaligned_receive_buffers_and_zero_length(lib, gpu):
     assert st.eager_messages > 0 and st.write_messages > 0 and st.rounds == 3
 
 
+@pytest.mark.parametrize("group", [2, 3, 8])
+def test_grouped_receives_mixed_eager_and_write_subreceives(lib, gpu, group):
+    """`group` messages per grouped receive (the phase shape of the reference's
+    tests/functional/grouped_recv.cpp): sub-receive k of a request gets the message with tag 1 + k,
+    eager where it fits and as striped writes where it does not, sizes 1 KiB * (k + 1) and larger."""
+    rng = np.random.default_rng(group)
+    n = 64 * 3 + group - 1                                      # the last request is a short one
+    sizes = [int(rng.choice([1024 * (1 + i % group), 262144, 8184, 8185, 0, 524288 + 3])) for i in range(n)]
+    caps = [s if i % 5 else max(s // 2, 1) for i, s in enumerate(sizes)]
+    st = run(lib, sizes, caps, 64, seed=100 + group, group=group, dst_skew=1)
+    assert st.eager_messages > 0 and st.write_messages > 0
+    # explicit tags, distinct within each request but not in order
+    tags = [1000 + (7 * i) % group for i in range(n)]
+    if len(set(tags[:group])) == group:
+        run(lib, sizes, caps, 64, seed=200 + group, group=group, tags=tags)
+
+
 def test_rejects_bad_arguments(lib, gpu):
     pool = torch.zeros(64 * RX_STRIDE, dtype=torch.uint8, device="cuda")
     one = np.array([pool.data_ptr()], dtype=np.uint64)
@@ -92,11 +111,13 @@ def test_rejects_bad_arguments(lib, gpu):
     stats = m.SendrecvLoopbackStats()
     call = lib.ofi_amd_sendrecv_loopback_run
     p = lambda a: a.ctypes.data
-    assert call(p(one), p(one), p(size), p(size), None, 1, 0, 4, pool.data_ptr(), pool.numel(), 0,
+    assert call(p(one), p(one), p(size), p(size), None, 1, 0, 4, 1, pool.data_ptr(), pool.numel(), 0,
                 _gpu.stream(), ctypes.byref(stats)) == -22          # nothing in flight
-    assert call(p(one), p(one), p(size), p(size), None, 1, 129, 4, pool.data_ptr(), pool.numel(), 0,
+    assert call(p(one), p(one), p(size), p(size), None, 1, 129, 4, 1, pool.data_ptr(), pool.numel(), 0,
                 _gpu.stream(), ctypes.byref(stats)) == -22          # more than the receiver allows
-    assert call(p(one), p(one), p(size), p(size), None, 1, 64, 4, pool.data_ptr(), 1000, 0,
+    assert call(p(one), p(one), p(size), p(size), None, 1, 64, 4, 1, pool.data_ptr(), 1000, 0,
                 _gpu.stream(), ctypes.byref(stats)) == -22          # rx pool too small
-    assert call(p(one), p(one), p(big), p(big), None, 1, 64, 4, pool.data_ptr(), pool.numel(), 0,
+    assert call(p(one), p(one), p(big), p(big), None, 1, 64, 4, 1, pool.data_ptr(), pool.numel(), 0,
                 _gpu.stream(), ctypes.byref(stats)) == -90          # -EMSGSIZE: 32-bit control length
+    assert call(p(one), p(one), p(size), p(size), None, 1, 64, 4, 9, pool.data_ptr(), pool.numel(), 0,
+                _gpu.stream(), ctypes.byref(stats)) == -22          # more sub-receives than a request holds
