@@ -229,6 +229,9 @@ int oracle_gin_rx_metadata(oracle_gin_rx_t *rx, uint32_t peer, const uint64_t me
 uint32_t oracle_gin_rx_take_work(oracle_gin_rx_t *rx, oracle_gin_signal_work_t *out, uint32_t cap)
 {
 	uint32_t n = rx->n_work < cap ? rx->n_work : cap;
+	if (n == 0) {
+		return 0; /* the queue may not be allocated yet */
+	}
 	memcpy(out, rx->work, n * sizeof(*out));
 	memmove(rx->work, rx->work + n, (rx->n_work - n) * sizeof(*out));
 	rx->n_work -= n;
@@ -238,6 +241,9 @@ uint32_t oracle_gin_rx_take_work(oracle_gin_rx_t *rx, oracle_gin_signal_work_t *
 uint32_t oracle_gin_rx_take_acks(oracle_gin_rx_t *rx, oracle_gin_ack_t *out, uint32_t cap)
 {
 	uint32_t n = rx->n_acks < cap ? rx->n_acks : cap;
+	if (n == 0) {
+		return 0;
+	}
 	memcpy(out, rx->acks, n * sizeof(*out));
 	memmove(rx->acks, rx->acks + n, (rx->n_acks - n) * sizeof(*out));
 	rx->n_acks -= n;

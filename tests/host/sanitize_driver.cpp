@@ -1,0 +1,490 @@
+/*
+ * Host-side differential driver, meant to be built with -fsanitize=address,undefined:
+ * the product's plain-C++ state machines (message buffer, send/receive comms, eager receive
+ * queue, GIN receiver) run side by side with the CPU oracle on random programs.  Any
+ * disagreement, and anything the sanitizers see, ends the run with a non-zero status.
+ * Test infrastructure: built and run by tests/test_host_sanitizers.py, CPU only.
+ */
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <deque>
+#include <vector>
+
+#include "ofi_amd_sendrecv.h"
+#include "oracle.h"
+
+namespace {
+
+struct rng_t {
+	uint64_t s;
+	uint64_t next()
+	{
+		s += 0x9E3779B97F4A7C15ull;
+		uint64_t z = s;
+		z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+		z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+		return z ^ (z >> 31);
+	}
+	uint32_t below(uint32_t n) { return (uint32_t)(next() % n); }
+	bool chance(uint32_t pct) { return below(100) < pct; }
+};
+
+[[noreturn]] void fail(const char *what, uint64_t a = 0, uint64_t b = 0)
+{
+	std::fprintf(stderr, "MISMATCH: %s (%llu vs %llu)\n", what, (unsigned long long)a, (unsigned long long)b);
+	std::exit(1);
+}
+
+#define SAME(what, a, b)                                        \
+	do {                                                    \
+		if ((uint64_t)(a) != (uint64_t)(b)) {           \
+			fail(what, (uint64_t)(a), (uint64_t)(b)); \
+		}                                               \
+	} while (0)
+
+/* ------------------------------------------------------------ message buffer */
+void run_msgbuff(uint64_t seed, uint16_t window, uint16_t bits, int steps)
+{
+	rng_t rng{ seed };
+	const uint16_t field = (uint16_t)(1u << bits);
+	const uint16_t start = (uint16_t)rng.below(field);
+	oracle_msgbuff_t *a = oracle_msgbuff_create(window, bits, start);
+	ofi_amd_msgbuff_t *b = nullptr;
+	const int rc = ofi_amd_msgbuff_create(window, bits, start, &b);
+	SAME("msgbuff create", a != nullptr, rc == 0);
+	if (!a) {
+		return;
+	}
+	static char cells[4096];
+	uint16_t head = start;
+	for (int i = 0; i < steps; i++) {
+		const uint16_t idx = (uint16_t)((head + field + rng.below(2u * window + 5u) - window - 2u) % field);
+		void *elem = &cells[rng.below(sizeof(cells))];
+		int sa = -1, sb = -1, ta = -1, tb = -1;
+		void *ea = nullptr, *eb = nullptr;
+		switch (rng.below(4)) {
+		case 0: {
+			const int type = (int)rng.below(2);
+			const int ra = oracle_msgbuff_insert(a, idx, elem, type, &sa);
+			SAME("insert result", ra, ofi_amd_msgbuff_insert(b, idx, elem, type, &sb));
+			if (ra == ORACLE_MSGBUFF_SUCCESS) {
+				head = (uint16_t)((idx + 1) % field);
+			}
+			break;
+		}
+		case 1:
+			SAME("replace result", oracle_msgbuff_replace(a, idx, elem, 1, &sa),
+			     ofi_amd_msgbuff_replace(b, idx, elem, 1, &sb));
+			break;
+		case 2: {
+			const int ra = oracle_msgbuff_retrieve(a, idx, &ea, &ta, &sa);
+			SAME("retrieve result", ra, ofi_amd_msgbuff_retrieve(b, idx, &eb, &tb, &sb));
+			if (ra == ORACLE_MSGBUFF_SUCCESS) {
+				SAME("retrieve elem", (uintptr_t)ea, (uintptr_t)eb);
+				SAME("retrieve type", ta, tb);
+			}
+			break;
+		}
+		default:
+			SAME("complete result", oracle_msgbuff_complete(a, idx, &sa), ofi_amd_msgbuff_complete(b, idx, &sb));
+			break;
+		}
+		SAME("status", sa, sb);
+	}
+	oracle_msgbuff_destroy(a);
+	ofi_amd_msgbuff_destroy(b);
+}
+
+/* -------------------------------------------------------- send / receive comms */
+struct msg_t {
+	uint64_t size;
+	int32_t tag;
+};
+struct recv_plan_t {
+	int n;
+	uint64_t sizes[8];
+	int tags[8];
+};
+struct flight_t {
+	int kind; /* 1 eager, 2 write stripe */
+	int32_t req_a, req_b;
+	oracle_send_action_t act;
+	uint32_t stripe;
+};
+
+void same_action(const oracle_send_action_t &x, const ofi_amd_send_action_t &y)
+{
+	SAME("action kind", x.kind, y.kind);
+	SAME("action seq", x.msg_seq_num, y.msg_seq_num);
+	SAME("action recv_idx", x.recv_idx, y.recv_idx);
+	SAME("action imm", x.imm, y.imm);
+	SAME("action size", x.size, y.size);
+	SAME("action remote", x.remote_buff_offset, y.remote_buff_offset);
+	SAME("action xfers", x.num_xfers, y.num_xfers);
+	SAME("action no_target_completion", x.no_target_completion, y.no_target_completion);
+	SAME("action hdr", std::memcmp(&x.hdr, &y.hdr, sizeof(x.hdr)), 0);
+	for (uint32_t k = 0; k < x.num_xfers; k++) {
+		SAME("xfer rail", x.xfers[k].rail_id, y.xfers[k].rail_id);
+		SAME("xfer offset", x.xfers[k].offset, y.xfers[k].offset);
+		SAME("xfer size", x.xfers[k].msg_size, y.xfers[k].msg_size);
+	}
+	for (int r = 0; r < 4; r++) {
+		SAME("action key", x.mr_key[r], y.mr_key[r]);
+	}
+}
+
+void run_sendrecv(uint64_t seed, uint32_t n_msgs, bool unique_tags)
+{
+	rng_t rng{ seed };
+	static const uint64_t kSizes[] = { 0, 8, 100, 1024, 8184, 8185, 16384, 200000, 600000 };
+	std::vector<msg_t> msgs(n_msgs);
+	for (uint32_t i = 0; i < n_msgs; i++) {
+		msgs[i] = msg_t{ kSizes[rng.below(9)], unique_tags ? (int32_t)(100 + i) : (int32_t)(1 + rng.below(5)) };
+	}
+	std::vector<recv_plan_t> plans;
+	for (uint32_t i = 0; i < n_msgs;) {
+		recv_plan_t p{};
+		p.n = (int)(1 + rng.below(4));
+		if ((uint32_t)p.n > n_msgs - i) {
+			p.n = (int)(n_msgs - i);
+		}
+		for (int k = 0; k < p.n; k++) { /* a rotation of the group's sends */
+			const msg_t &m = msgs[i + (uint32_t)((k + 1) % p.n)];
+			p.tags[k] = m.tag;
+			p.sizes[k] = rng.chance(80) ? m.size : (m.size / 2 ? m.size / 2 : 1);
+		}
+		plans.push_back(p);
+		i += (uint32_t)p.n;
+	}
+
+	oracle_send_comm_t *sa = oracle_send_comm_create(77, 4, 8192, 131072, 64);
+	oracle_recv_comm_t *ra = oracle_recv_comm_create(4);
+	ofi_amd_send_comm_t *sb = nullptr;
+	ofi_amd_recv_comm_t *rb = nullptr;
+	if (!sa || !ra || ofi_amd_send_comm_create(77, 4, 8192, 131072, 64, &sb) != 0 ||
+	    ofi_amd_recv_comm_create(4, &rb) != 0) {
+		fail("create comms");
+	}
+	oracle_ctrl_msg_t *mba = oracle_send_comm_mailbox(sa);
+	ofi_amd_ctrl_msg_t *mbb = ofi_amd_send_comm_mailbox(sb);
+
+	std::deque<uint32_t> queue;
+	for (uint32_t i = 0; i < n_msgs; i++) {
+		queue.push_back(i);
+	}
+	std::vector<flight_t> wire;
+	std::vector<std::pair<int32_t, int32_t>> send_reqs, recv_reqs;
+	std::vector<int> recv_n;
+	size_t next_plan = 0;
+	uint64_t next_dst = 0x10000000, cookie = 1;
+
+	for (int round = 0; round < 300; round++) {
+		/* sends: a tag that was told to call again blocks later sends of that tag */
+		std::vector<int32_t> blocked;
+		std::deque<uint32_t> again;
+		for (uint32_t i : queue) {
+			bool skip = rng.chance(20);
+			for (int32_t t : blocked) {
+				skip = skip || t == msgs[i].tag;
+			}
+			if (skip) {
+				blocked.push_back(msgs[i].tag);
+				again.push_back(i);
+				continue;
+			}
+			oracle_send_action_t xa;
+			ofi_amd_send_action_t xb;
+			SAME("send rc", oracle_send_comm_send(sa, msgs[i].size, msgs[i].tag, &xa),
+			     ofi_amd_send_comm_send(sb, msgs[i].size, msgs[i].tag, &xb));
+			same_action(xa, xb);
+			if (xa.kind == ORACLE_SEND_AGAIN) {
+				blocked.push_back(msgs[i].tag);
+				again.push_back(i);
+				continue;
+			}
+			send_reqs.emplace_back(xa.req, xb.req);
+			if (xa.kind == ORACLE_SEND_EAGER) {
+				wire.push_back(flight_t{ 1, xa.req, xb.req, xa, 0 });
+			} else {
+				for (uint32_t k = 0; k < xa.num_xfers; k++) {
+					wire.push_back(flight_t{ 2, xa.req, xb.req, xa, k });
+				}
+			}
+		}
+		queue.swap(again);
+		/* receives */
+		for (uint32_t r = rng.below(3); r > 0 && next_plan < plans.size(); r--) {
+			const recv_plan_t &p = plans[next_plan];
+			uint64_t dsts[8], keys[32];
+			for (int k = 0; k < p.n; k++) {
+				dsts[k] = next_dst + 0x100000ull * (uint64_t)k;
+				for (int q = 0; q < 4; q++) {
+					keys[k * 4 + q] = 0xA000 + next_plan * 32 + (uint64_t)(k * 4 + q);
+				}
+			}
+			int32_t qa = -1, qb = -1;
+			uint16_t seq_a = 0, seq_b = 0;
+			const int rca = oracle_recv_comm_recv(ra, p.n, dsts, p.sizes, p.tags, keys, 0, mba, &qa, &seq_a);
+			SAME("recv rc", rca, ofi_amd_recv_comm_recv(rb, p.n, dsts, p.sizes, p.tags, keys, 0, mbb, &qb, &seq_b));
+			if (rca != 0) {
+				break; /* the receiver is full: try again in a later round */
+			}
+			SAME("recv seq", seq_a, seq_b);
+			SAME("ctrl_sent", oracle_recv_comm_ctrl_sent(ra, qa), ofi_amd_recv_comm_ctrl_sent(rb, qb));
+			recv_reqs.emplace_back(qa, qb);
+			recv_n.push_back(p.n);
+			next_dst += 0x800000;
+			next_plan++;
+		}
+		/* the wire, in random order */
+		if (rng.chance(80)) {
+			while (!wire.empty()) {
+				const size_t k = rng.below((uint32_t)wire.size());
+				const flight_t f = wire[k];
+				wire[k] = wire.back();
+				wire.pop_back();
+				if (f.kind == 1) {
+					ofi_amd_eager_hdr_t hb;
+					std::memcpy(&hb, &f.act.hdr, sizeof(hb));
+					SAME("eager arrival",
+					     oracle_recv_comm_eager_arrival(ra, f.act.msg_seq_num, &f.act.hdr, (uint32_t)f.act.size, cookie),
+					     ofi_amd_recv_comm_eager_arrival(rb, f.act.msg_seq_num, &hb, (uint32_t)f.act.size, cookie));
+					cookie++;
+				} else {
+					const uint64_t len = f.act.xfers[f.stripe].msg_size;
+					SAME("write arrival", oracle_recv_comm_write_arrival(ra, f.act.imm, len),
+					     ofi_amd_recv_comm_write_arrival(rb, f.act.imm, len));
+				}
+				SAME("send completion", oracle_send_comm_completion(sa, f.req_a),
+				     ofi_amd_send_comm_completion(sb, f.req_b));
+			}
+		}
+		/* eager copies */
+		for (;;) {
+			oracle_eager_copy_item_t ia[16];
+			ofi_amd_eager_copy_item_t ib[16];
+			const uint32_t na = oracle_recv_comm_take_copies(ra, ia, 16);
+			SAME("copies", na, ofi_amd_recv_comm_take_copies(rb, ib, 16));
+			for (uint32_t k = 0; k < na; k++) {
+				SAME("copy cookie", ia[k].rx_cookie, ib[k].rx_cookie);
+				SAME("copy dst", ia[k].dst, ib[k].dst);
+				SAME("copy dst_len", ia[k].dst_len, ib[k].dst_len);
+				SAME("copy recv_len", ia[k].recv_len, ib[k].recv_len);
+				SAME("copy sub", ia[k].sub_idx, ib[k].sub_idx);
+				SAME("copy needs", ia[k].needs_copy, ib[k].needs_copy);
+				if (ia[k].needs_copy) {
+					SAME("copy done", oracle_recv_comm_copy_done(ra, ia[k].req, ia[k].sub_idx),
+					     ofi_amd_recv_comm_copy_done(rb, ib[k].req, ib[k].sub_idx));
+				}
+			}
+			if (na < 16) {
+				break;
+			}
+		}
+		/* test() on a random subset of the open requests */
+		for (size_t k = 0; k < send_reqs.size(); k++) {
+			if (send_reqs[k].first < 0 || !rng.chance(70)) {
+				continue;
+			}
+			int da = 0, db = 0;
+			uint64_t za = 0, zb = 0;
+			SAME("send test", oracle_send_comm_test(sa, send_reqs[k].first, &da, &za),
+			     ofi_amd_send_comm_test(sb, send_reqs[k].second, &db, &zb));
+			SAME("send done", da, db);
+			if (da) {
+				SAME("send size", za, zb);
+				send_reqs[k].first = -1;
+			}
+		}
+		for (size_t k = 0; k < recv_reqs.size(); k++) {
+			if (recv_reqs[k].first < 0 || !rng.chance(70)) {
+				continue;
+			}
+			int da = 0, db = 0, za[8] = {}, zb[8] = {};
+			SAME("recv test", oracle_recv_comm_test(ra, recv_reqs[k].first, &da, za),
+			     ofi_amd_recv_comm_test(rb, recv_reqs[k].second, &db, zb));
+			SAME("recv done", da, db);
+			if (da) {
+				for (int q = 0; q < recv_n[k]; q++) {
+					SAME("recv size", za[q], zb[q]);
+				}
+				recv_reqs[k].first = -1;
+			}
+		}
+		oracle_send_state_t ssa;
+		ofi_amd_send_state_t ssb;
+		oracle_send_comm_state(sa, &ssa);
+		ofi_amd_send_comm_state(sb, &ssb);
+		static_assert(sizeof(ssa) == sizeof(ssb), "state layouts");
+		SAME("send state", std::memcmp(&ssa, &ssb, sizeof(ssa)), 0);
+		oracle_recv_state_t rsa;
+		ofi_amd_recv_state_t rsb;
+		oracle_recv_comm_state(ra, &rsa);
+		ofi_amd_recv_comm_state(rb, &rsb);
+		static_assert(sizeof(rsa) == sizeof(rsb), "state layouts");
+		SAME("recv state", std::memcmp(&rsa, &rsb, sizeof(rsa)), 0);
+	}
+	if (unique_tags) { /* with one tag per message everything must have been delivered */
+		SAME("sends left", queue.size(), 0);
+		for (const auto &q : send_reqs) {
+			SAME("send still open", q.first, -1);
+		}
+		for (const auto &q : recv_reqs) {
+			SAME("recv still open", q.first, -1);
+		}
+	}
+	oracle_send_comm_destroy(sa);
+	oracle_recv_comm_destroy(ra);
+	ofi_amd_send_comm_destroy(sb);
+	ofi_amd_recv_comm_destroy(rb);
+}
+
+/* -------------------------------------------------------- eager receive queue */
+void run_rxq(uint64_t seed)
+{
+	rng_t rng{ seed };
+	oracle_eager_rxq_t *a = oracle_eager_rxq_create();
+	ofi_amd_eager_rxq_t *b = nullptr;
+	if (!a || ofi_amd_eager_rxq_create(&b) != 0) {
+		fail("rxq create");
+	}
+	oracle_eager_tx_t tx;
+	oracle_eager_tx_init(&tx);
+	std::vector<oracle_eager_entry_t> pending;
+	uint64_t cookie = 0;
+	for (int i = 0; i < 4000; i++) {
+		if (pending.size() < 24 && rng.chance(60)) {
+			oracle_eager_hdr_t h;
+			oracle_eager_tx_assign(&tx, (int32_t)rng.below(9), &h);
+			oracle_eager_entry_t e{};
+			e.eager_offset = h.eager_offset;
+			e.prev_batch_count = h.prev_batch_count;
+			e.eager_seq = h.eager_seq;
+			e.tag = h.tag;
+			e.cookie = cookie++;
+			pending.push_back(e);
+			if (rng.chance(40)) {
+				oracle_eager_tx_advance(&tx);
+			}
+		}
+		if (!pending.empty() && rng.chance(70)) {
+			const size_t k = rng.below((uint32_t)pending.size());
+			ofi_amd_eager_entry_t eb;
+			static_assert(sizeof(eb) == sizeof(pending[k]), "entry layouts");
+			std::memcpy(&eb, &pending[k], sizeof(eb));
+			SAME("rxq insert", oracle_eager_rxq_insert(a, &pending[k]), ofi_amd_eager_rxq_insert(b, &eb));
+			pending[k] = pending.back();
+			pending.pop_back();
+			oracle_eager_entry_t oa[8];
+			ofi_amd_eager_entry_t ob[8];
+			const uint32_t na = oracle_eager_rxq_drain(a, oa, 8);
+			SAME("rxq drain", na, ofi_amd_eager_rxq_drain(b, ob, 8));
+			SAME("rxq entries", std::memcmp(oa, ob, na * sizeof(oa[0])), 0);
+			SAME("rxq pending", oracle_eager_rxq_pending(a), ofi_amd_eager_rxq_pending(b));
+		}
+	}
+	oracle_eager_rxq_destroy(a);
+	ofi_amd_eager_rxq_destroy(b);
+}
+
+/* --------------------------------------------------------------- GIN receiver */
+void run_gin_rx(uint64_t seed, uint32_t n_ops)
+{
+	rng_t rng{ seed };
+	const uint32_t comm_ids[2] = { 5, 9 };
+	oracle_gin_rx_t *a = oracle_gin_rx_create(2, comm_ids);
+	ofi_amd_gin_rx_t *b = nullptr;
+	if (!a || ofi_amd_gin_rx_create(2, comm_ids, &b) != 0) {
+		fail("gin rx create");
+	}
+	oracle_gin_mr_t mrs[3];
+	std::memset(mrs, 0, sizeof(mrs));
+	mrs[0].local_base = 0x1000000;
+	mrs[1].remote_address_offset = 0x2000000;
+	mrs[2].remote_address = 0x7F5500000000ull;
+	struct event_t {
+		uint32_t peer, is_meta, imm;
+		uint64_t meta[4];
+	};
+	std::vector<event_t> flight;
+	oracle_gin_comm_t comms[2];
+	for (int p = 0; p < 2; p++) {
+		oracle_gin_comm_init(&comms[p], comm_ids[p], 4, 131072, 64, 0);
+	}
+	auto deliver = [&](const event_t &e) {
+		if (e.is_meta) {
+			SAME("gin meta", oracle_gin_rx_metadata(a, e.peer, e.meta), ofi_amd_gin_rx_metadata(b, e.peer, e.meta));
+		} else {
+			SAME("gin write", oracle_gin_rx_write(a, e.peer, e.imm), ofi_amd_gin_rx_write_completion(b, e.peer, e.imm));
+		}
+		oracle_gin_signal_work_t wa[32];
+		ofi_amd_gin_signal_work_t wb[32];
+		static_assert(sizeof(wa[0]) == sizeof(wb[0]), "work layouts");
+		const uint32_t nw = oracle_gin_rx_take_work(a, wa, 32);
+		SAME("gin work count", nw, ofi_amd_gin_rx_take_work(b, wb, 32));
+		SAME("gin work", std::memcmp(wa, wb, nw * sizeof(wa[0])), 0);
+		oracle_gin_ack_t ka[32];
+		ofi_amd_gin_ack_t kb[32];
+		static_assert(sizeof(ka[0]) == sizeof(kb[0]), "ack layouts");
+		const uint32_t nk = oracle_gin_rx_take_acks(a, ka, 32);
+		SAME("gin ack count", nk, ofi_amd_gin_rx_take_acks(b, kb, 32));
+		SAME("gin acks", std::memcmp(ka, kb, nk * sizeof(ka[0])), 0);
+		for (uint32_t k = 0; k < nk; k++) {
+			oracle_gin_apply_ack(&comms[ka[k].peer], ka[k].rx_consumed);
+		}
+	};
+	for (uint32_t i = 0; i < n_ops; i++) {
+		const uint32_t peer = rng.below(2);
+		oracle_gin_desc_t d;
+		oracle_gin_gen_desc(seed, peer, i, 1, 3, 1 + rng.below(2), 1, &d);
+		oracle_gin_wire_t w;
+		if (oracle_gin_iput_signal(&comms[peer], mrs, &d, &w) != 0) {
+			while (!flight.empty()) { /* window full: let everything land, then go on */
+				const event_t e = flight.back();
+				flight.pop_back();
+				deliver(e);
+			}
+			continue;
+		}
+		for (uint32_t k = 0; k < w.num_writes; k++) {
+			flight.push_back(event_t{ peer, 0, w.imm, { 0, 0, 0, 0 } });
+		}
+		if (w.has_meta) {
+			flight.push_back(event_t{ peer, 1, 0, { w.meta[0], w.meta[1], w.meta[2], w.meta[3] } });
+		}
+		while (flight.size() > 40 || (!flight.empty() && rng.chance(50))) {
+			const size_t k = rng.below((uint32_t)flight.size());
+			const event_t e = flight[k];
+			flight[k] = flight.back();
+			flight.pop_back();
+			deliver(e);
+		}
+	}
+	while (!flight.empty()) {
+		const event_t e = flight.back();
+		flight.pop_back();
+		deliver(e);
+	}
+	oracle_gin_rx_destroy(a);
+	ofi_amd_gin_rx_destroy(b);
+}
+
+} // namespace
+
+int main(int argc, char **argv)
+{
+	const uint64_t seeds = argc > 1 ? std::strtoull(argv[1], nullptr, 10) : 6;
+	for (uint64_t s = 1; s <= seeds; s++) {
+		run_msgbuff(s, 4, 4, 3000);
+		run_msgbuff(s + 100, 7, 4, 3000);
+		run_msgbuff(s + 200, 256, 10, 6000);
+		run_msgbuff(s + 300, 9, 4, 10); /* rejected by both */
+		run_sendrecv(s, 60 + 20 * (uint32_t)s, true);
+		run_sendrecv(s + 1000, 60 + 20 * (uint32_t)s, false);
+		run_rxq(s);
+		run_gin_rx(s, 20000);
+	}
+	std::printf("host state machines: oracle and product agree over %llu seeds\n", (unsigned long long)seeds);
+	return 0;
+}
