@@ -1,7 +1,7 @@
 /*
  * Host-side differential driver, meant to be built with -fsanitize=address,undefined:
  * the product's plain-C++ state machines (message buffer, send/receive comms, eager receive
- * queue, GIN receiver) run side by side with the CPU oracle on random programs.  Any
+ * queue, GIN sender and receiver) run side by side with the CPU oracle on random programs.  Any
  * disagreement, and anything the sanitizers see, ends the run with a non-zero status.
  * Test infrastructure: built and run by tests/test_host_sanitizers.py, CPU only.
  */
@@ -470,6 +470,52 @@ void run_gin_rx(uint64_t seed, uint32_t n_ops)
 	ofi_amd_gin_rx_destroy(b);
 }
 
+/* ----------------------------------------------------------------- GIN sender */
+void run_gin_tx(uint64_t seed, uint32_t n_ops, uint32_t ack_model)
+{
+	rng_t rng{ seed };
+	static_assert(sizeof(oracle_gin_comm_t) == sizeof(ofi_amd_gin_comm_t), "comm layouts");
+	static_assert(sizeof(oracle_gin_wire_t) == sizeof(ofi_amd_gin_wire_t), "wire layouts");
+	static_assert(sizeof(oracle_gin_desc_t) == sizeof(ofi_amd_gin_desc_t), "descriptor layouts");
+	static_assert(sizeof(oracle_gin_mr_t) == sizeof(ofi_amd_gin_mr_t), "registration layouts");
+	oracle_gin_comm_t ca;
+	ofi_amd_gin_comm_t cb;
+	const uint32_t rails = 1 + rng.below(4);
+	oracle_gin_comm_init(&ca, 321, rails, 131072, 64, ack_model);
+	SAME("gin comm init", ofi_amd_gin_comm_init(&cb, 321, rails, 131072, 64, ack_model), 0);
+	oracle_gin_mr_t mrs[3];
+	std::memset(mrs, 0, sizeof(mrs));
+	mrs[0].local_base = 0x1000000;
+	mrs[1].remote_address_offset = 0x2000000;
+	mrs[2].remote_address = 0x7F5500000000ull;
+	for (int r = 0; r < 4; r++) {
+		mrs[1].key[r] = 0xB000 + (uint64_t)r;
+		mrs[2].key[r] = 0xC000 + (uint64_t)r;
+	}
+	ofi_amd_gin_mr_t mrs_b[3];
+	std::memcpy(mrs_b, mrs, sizeof(mrs));
+	for (uint32_t i = 0; i < n_ops; i++) {
+		oracle_gin_desc_t d;
+		oracle_gin_gen_desc(seed, 0, i, 1, 1 + rng.below(5), rng.below(4), rng.below(2), &d); /* op 3 is invalid */
+		ofi_amd_gin_desc_t db;
+		std::memcpy(&db, &d, sizeof(db));
+		oracle_gin_wire_t wa;
+		ofi_amd_gin_wire_t wb;
+		std::memset(&wa, 0, sizeof(wa));
+		std::memset(&wb, 0, sizeof(wb));
+		const int ra = oracle_gin_iput_signal(&ca, mrs, &d, &wa);
+		SAME("iput rc", ra, ofi_amd_gin_iput_signal(&cb, mrs_b, &db, &wb));
+		if (ra == 0) {
+			SAME("wire record", std::memcmp(&wa, &wb, sizeof(wa)), 0);
+		} else if (ra == -11) { /* window full: the receiver has consumed up to some point */
+			const uint32_t consumed = (ca.tx_tail + 1 + rng.below(4000)) & 0x3FFFu;
+			oracle_gin_apply_ack(&ca, consumed);
+			ofi_amd_gin_apply_ack(&cb, consumed);
+		}
+		SAME("comm state", std::memcmp(&ca, &cb, sizeof(ca)), 0);
+	}
+}
+
 } // namespace
 
 int main(int argc, char **argv)
@@ -484,6 +530,8 @@ int main(int argc, char **argv)
 		run_sendrecv(s + 1000, 60 + 20 * (uint32_t)s, false);
 		run_rxq(s);
 		run_gin_rx(s, 20000);
+		run_gin_tx(s, 30000, 0);
+		run_gin_tx(s + 50, 30000, 1);
 	}
 	std::printf("host state machines: oracle and product agree over %llu seeds\n", (unsigned long long)seeds);
 	return 0;
