@@ -120,9 +120,10 @@ __global__ __launch_bounds__(256) void region_choice_kernel(grid_dims_t g, regio
 		      pt_t{ g.log2_sizes[si], g.log2_ranks[ni * g.n_ppn + pi] }, kAllAllowed, algorithm,
 		      protocol, nchannels);
 	const uint64_t idx = (uint64_t)blockIdx.y * points_per_platform + p;
-	choice[idx * 4 + 0] = (int8_t)algorithm;
-	choice[idx * 4 + 1] = (int8_t)protocol;
-	*reinterpret_cast<int16_t *>(&choice[idx * 4 + 2]) = (int16_t)nchannels;
+	/* {int8 algorithm, int8 protocol, int16 nchannels} as one 4-byte store */
+	reinterpret_cast<uint32_t *>(choice)[idx] = ((uint32_t)(uint8_t)(int8_t)algorithm) |
+						     ((uint32_t)(uint8_t)(int8_t)protocol << 8) |
+						     ((uint32_t)(uint16_t)(int16_t)nchannels << 16);
 }
 
 /* ---- host side: building the log2-space polygon tables ---- */
@@ -470,7 +471,7 @@ int ofi_amd_tuner_region_grid(ofi_amd_tuner_plan_t *plan, const int32_t *platfor
 	if (rc != 0) {
 		return rc;
 	}
-	if (!plan || !platforms || n_platforms == 0 || !d_choice) {
+	if (!plan || !platforms || n_platforms == 0 || !d_choice || (reinterpret_cast<uintptr_t>(d_choice) & 3u) != 0) {
 		return -EINVAL;
 	}
 	for (uint32_t i = 0; i < n_platforms; i++) {

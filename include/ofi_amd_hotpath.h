@@ -534,6 +534,7 @@ int ofi_amd_tuner_model_grid(ofi_amd_tuner_plan_t *plan, const ofi_amd_tuner_var
  * Region grid for n_platforms platforms in one launch.
  *   d_choice[(p * points + point) * 4 + {0,1}] = {algo, proto} or {-1,-1} (fall back to NCCL),
  *   bytes 2..3 = int16 nChannels override, or -1 when the tuner leaves nChannels alone.
+ *   d_choice is 4-byte aligned (one record per store).
  */
 int ofi_amd_tuner_region_grid(ofi_amd_tuner_plan_t *plan, const int32_t *platforms,
 			      uint32_t n_platforms, int8_t *d_choice, void *stream);
