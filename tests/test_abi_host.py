@@ -137,3 +137,23 @@ def test_proxy_rejects_bad_arguments(lib):
     w = m.GinWire()
     assert lib.ofi_amd_gin_iput_signal(ctypes.byref(c), _oracle.default_mrs(m.GinMr), ctypes.byref(d),
                                        ctypes.byref(w)) == -errno.EINVAL
+
+
+def test_device_put_header_compiles_in_a_user_kernel(tmp_path):
+    """include/ofi_amd_gin_device.h is all a user's own kernel needs to initiate puts."""
+    import shutil
+    import subprocess
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("no hipcc")
+    obj = tmp_path / "user_put_kernel.o"
+    proc = subprocess.run([hipcc, "--offload-arch=gfx950", "-O2", "-std=c++17", "-Wall", "-Werror",
+                           "-Wno-unknown-warning-option",
+                           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                           "-I", os.path.join(ROOT, "include"), "-c",
+                           os.path.join(ROOT, "tests", "host", "user_put_kernel.hip"), "-o", str(obj)],
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    text = "\n".join(l for l in proc.stdout.splitlines()
+                     if "packed-fp32-ops" not in l and "is not a recognized feature" not in l)
+    assert proc.returncode == 0, text
+    assert obj.stat().st_size > 0
