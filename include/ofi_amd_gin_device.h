@@ -76,17 +76,49 @@ __device__ __forceinline__ int ofi_amd_gin_dev_put(const ofi_amd_gin_dev_ring_t 
 	}
 	__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
 
-	if (active) {
-		ofi_amd_u32x4 *dst = static_cast<ofi_amd_u32x4 *>(ring.records) + (uint64_t)(pos & mask) * 4u;
-		ofi_amd_u32x4 a, b, c, d; /* the descriptor is only 8-byte aligned: copy, do not cast */
-		__builtin_memcpy(&a, reinterpret_cast<const char *>(desc), 16);
-		__builtin_memcpy(&b, reinterpret_cast<const char *>(desc) + 16, 16);
-		__builtin_memcpy(&c, reinterpret_cast<const char *>(desc) + 32, 16);
-		__builtin_memcpy(&d, reinterpret_cast<const char *>(desc) + 48, 16);
-		dst[0] = a;
-		dst[1] = b;
-		dst[2] = c;
-		dst[3] = d;
+	ofi_amd_u32x4 part[4]; /* the descriptor is only 8-byte aligned: copy, do not cast */
+	__builtin_memcpy(&part[0], reinterpret_cast<const char *>(desc), 16);
+	__builtin_memcpy(&part[1], reinterpret_cast<const char *>(desc) + 16, 16);
+	__builtin_memcpy(&part[2], reinterpret_cast<const char *>(desc) + 32, 16);
+	__builtin_memcpy(&part[3], reinterpret_cast<const char *>(desc) + 48, 16);
+	ofi_amd_u32x4 *records = static_cast<ofi_amd_u32x4 *>(ring.records);
+	if (ballot == ~0ull) {
+		/* Full wavefront: lanes 4g..4g+3 hold records 4g..4g+3.  Each of the four store
+		 * instructions writes one whole record per group of four lanes -- lane 4g+p the
+		 * p-th 16 bytes of record 4g+k -- so the host link carries complete 64-byte lines
+		 * instead of four 16-byte pieces per record scattered over four instructions.
+		 * The parts travel between the four lanes through DPP quad broadcasts. */
+		const uint32_t p = lane & 3u;
+#define OFI_AMD_GIN_QUAD_BCAST(v, ctrl) \
+	((uint32_t)__builtin_amdgcn_mov_dpp((int)(v), (ctrl), 0xf, 0xf, true))
+#define OFI_AMD_GIN_STORE_COLUMN(k, ctrl)                                                              \
+	do {                                                                                           \
+		ofi_amd_u32x4 out;                                                                     \
+		ofi_amd_u32x4 q0, q1, q2, q3;                                                          \
+		q0.x = OFI_AMD_GIN_QUAD_BCAST(part[0].x, ctrl); q0.y = OFI_AMD_GIN_QUAD_BCAST(part[0].y, ctrl); \
+		q0.z = OFI_AMD_GIN_QUAD_BCAST(part[0].z, ctrl); q0.w = OFI_AMD_GIN_QUAD_BCAST(part[0].w, ctrl); \
+		q1.x = OFI_AMD_GIN_QUAD_BCAST(part[1].x, ctrl); q1.y = OFI_AMD_GIN_QUAD_BCAST(part[1].y, ctrl); \
+		q1.z = OFI_AMD_GIN_QUAD_BCAST(part[1].z, ctrl); q1.w = OFI_AMD_GIN_QUAD_BCAST(part[1].w, ctrl); \
+		q2.x = OFI_AMD_GIN_QUAD_BCAST(part[2].x, ctrl); q2.y = OFI_AMD_GIN_QUAD_BCAST(part[2].y, ctrl); \
+		q2.z = OFI_AMD_GIN_QUAD_BCAST(part[2].z, ctrl); q2.w = OFI_AMD_GIN_QUAD_BCAST(part[2].w, ctrl); \
+		q3.x = OFI_AMD_GIN_QUAD_BCAST(part[3].x, ctrl); q3.y = OFI_AMD_GIN_QUAD_BCAST(part[3].y, ctrl); \
+		q3.z = OFI_AMD_GIN_QUAD_BCAST(part[3].z, ctrl); q3.w = OFI_AMD_GIN_QUAD_BCAST(part[3].w, ctrl); \
+		out = p == 0u ? q0 : (p == 1u ? q1 : (p == 2u ? q2 : q3));                             \
+		const uint32_t rec_pos = base + (lane & ~3u) + (k);                                    \
+		records[(uint64_t)(rec_pos & mask) * 4u + p] = out;                                    \
+	} while (0)
+		OFI_AMD_GIN_STORE_COLUMN(0u, 0x00);
+		OFI_AMD_GIN_STORE_COLUMN(1u, 0x55);
+		OFI_AMD_GIN_STORE_COLUMN(2u, 0xAA);
+		OFI_AMD_GIN_STORE_COLUMN(3u, 0xFF);
+#undef OFI_AMD_GIN_STORE_COLUMN
+#undef OFI_AMD_GIN_QUAD_BCAST
+	} else if (active) {
+		ofi_amd_u32x4 *dst = records + (uint64_t)(pos & mask) * 4u;
+		dst[0] = part[0];
+		dst[1] = part[1];
+		dst[2] = part[2];
+		dst[3] = part[3];
 	}
 	__builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
 	if (active) {
