@@ -78,7 +78,8 @@ def bench_bounce(lib, oracle, torch, np, args):
     d_src = _gpu.to_dev(src)
     d_arena = torch.zeros(w["arena_bytes"], dtype=torch.uint8, device="cuda")
     d_so, d_do, d_len = _gpu.to_dev(w["src_off"]), _gpu.to_dev(w["dst_off"]), _gpu.to_dev(w["len"])
-    d_flush = torch.zeros(n, dtype=torch.int32, device="cuda")
+    # the flush words land in a host-pinned array, as a flush completion does in the reference
+    d_flush = torch.zeros(n, dtype=torch.int32).pin_memory()
     stream = _gpu.stream()
 
     def step():
@@ -608,7 +609,7 @@ def main():
         "warmup": args.warmup, "ms_per_step": bounce["ms_wall"], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": "bounce copy: 65536 eager buffers, len uniform 0..8192 B, packed source "
-                               "-> seeded 64 B-aligned offsets in a 2 GiB HBM arena, 4 B flush read each",
+                               "-> seeded 64 B-aligned offsets in a 2 GiB HBM arena, 4 B flush read each into a host-pinned array",
                    "buffers": bounce["buffers"], "payload_bytes": bounce["payload_bytes"],
                    "arena_bytes": 2 << 30},
         "roofline": {"bound": "hbm", "achieved": bounce["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
