@@ -40,12 +40,12 @@ struct pinned_t {
 };
 
 struct open_msg_t {
-	uint64_t index;
+	uint64_t index = 0;
 	int32_t send_req = -1;
 	int32_t recv_req = -1;
 	int32_t sub_idx = 0;
 	uint32_t group_size = 1;
-	ofi_amd_send_action_t action;
+	ofi_amd_send_action_t action = {};
 	bool sent = false;
 };
 
