@@ -56,7 +56,34 @@ def test_graph_of_hot_path_launches_replays_exactly(lib, oracle, gpu):
     with np.errstate(over="ignore"):
         np.add.at(per_replay, (work["offset"] // 8).astype(np.int64), work["value"])
 
+    # eager-format copy and table copy out of the same source bytes
+    n_e, stride = 512, 8320
+    e_len = rng.integers(0, 8185, n_e).astype(np.uint32)
+    e_rx = (rng.permutation(n_e).astype(np.uint64) * np.uint64(stride))
+    e_dst = (np.arange(n_e, dtype=np.uint64) * np.uint64(8192 + 64) + rng.integers(0, 16, n_e).astype(np.uint64))
+    d_earena = torch.zeros(n_e * (8192 + 64), dtype=torch.uint8, device="cuda")
+    d_erx, d_elen, d_edst = _gpu.to_dev(e_rx), _gpu.to_dev(e_len), _gpu.to_dev(e_dst)
+    d_copied = torch.zeros(n_e, dtype=torch.int32, device="cuda")
+    want_earena = np.zeros(n_e * (8192 + 64), dtype=np.uint8)
+    oracle.oracle_eager_copy_batch(_oracle.ptr(src), _oracle.ptr(e_rx), _oracle.ptr(e_len), _oracle.ptr(want_earena),
+                                   _oracle.ptr(e_dst), _oracle.ptr(e_len), n_e, None)
+    n_t = 300
+    t_len = rng.integers(1, 70000, n_t).astype(np.uint32)
+    t_src_off = rng.integers(0, w["src_bytes"] - 70000, n_t).astype(np.uint64)
+    t_dst_off = np.concatenate(([0], np.cumsum(t_len.astype(np.uint64) + np.uint64(3))[:-1])).astype(np.uint64)
+    d_tarena = torch.zeros(int(t_dst_off[-1]) + 70000, dtype=torch.uint8, device="cuda")
+    d_tsrc = _gpu.to_dev(t_src_off + np.uint64(d_src.data_ptr()))
+    d_tdst = _gpu.to_dev(t_dst_off + np.uint64(d_tarena.data_ptr()))
+    d_tlen = _gpu.to_dev(t_len)
+    want_tarena = np.zeros(d_tarena.numel(), dtype=np.uint8)
+    for a, b, l in zip(t_src_off, t_dst_off, t_len):
+        want_tarena[int(b):int(b) + int(l)] = src[int(a):int(a) + int(l)]
+
     def launches():
+        assert lib.ofi_amd_eager_copy_batch(d_src.data_ptr(), d_erx.data_ptr(), d_elen.data_ptr(),
+                                            d_earena.data_ptr(), d_edst.data_ptr(), d_elen.data_ptr(), n_e,
+                                            d_copied.data_ptr(), None, sp) == 0
+        assert lib.ofi_amd_copy_table(d_tsrc.data_ptr(), d_tdst.data_ptr(), d_tlen.data_ptr(), n_t, sp) == 0
         assert lib.ofi_amd_sched_batch(d_state.data_ptr(), d_sizes.data_ptr(), n_msg, 128, d_num.data_ptr(),
                                        d_xf.data_ptr(), sp) == 0
         assert lib.ofi_amd_bounce_scatter(d_src.data_ptr(), d_arena.data_ptr(), w["arena_bytes"],
@@ -83,6 +110,9 @@ def test_graph_of_hot_path_launches_replays_exactly(lib, oracle, gpu):
     for replay in range(4):
         # eager work and a synchronisation between replays; outputs wiped so a replay must rewrite them
         d_arena.zero_()
+        d_earena.zero_()
+        d_tarena.zero_()
+        d_copied.zero_()
         d_flush.zero_()
         d_num.fill_(-1)
         d_xf.fill_(-1)
@@ -97,6 +127,9 @@ def test_graph_of_hot_path_launches_replays_exactly(lib, oracle, gpu):
         got_state = m.SchedState.from_buffer_copy(d_state.cpu().numpy().tobytes())
         assert (got_state.rr_small_counter, got_state.rr_counter) == (ost.rr_small_counter, ost.rr_counter)
         assert np.array_equal(d_arena.cpu().numpy(), want_arena), replay
+        assert np.array_equal(d_earena.cpu().numpy(), want_earena), replay
+        assert np.array_equal(_gpu.to_host(d_copied, np.uint32), e_len), replay
+        assert np.array_equal(d_tarena.cpu().numpy(), want_tarena), replay
         assert np.array_equal(_gpu.to_host(d_flush, np.uint32), want_flush), replay
         with np.errstate(over="ignore"):
             counters += per_replay
