@@ -201,6 +201,10 @@ __global__ __launch_bounds__(kThreads) void gin_produce_seeded_kernel(
 	}
 
 	if (threadIdx.x == 0) {
+		/* the free-slot horizon of the device-side put follows the cursor: every position
+		 * this kernel filled was seen free first */
+		__hip_atomic_store(&enqueue_pos[ctx * kGinReserveStride + 1], cursor, __ATOMIC_RELAXED,
+				   __HIP_MEMORY_SCOPE_AGENT);
 		__hip_atomic_store(&enqueue_pos[ctx * kGinReserveStride], cursor, __ATOMIC_RELEASE,
 				   __HIP_MEMORY_SCOPE_AGENT);
 	}

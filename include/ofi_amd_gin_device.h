@@ -28,7 +28,8 @@
  * The wave's descriptors take consecutive positions in lane order: one atomic add on the
  * device-resident cursor per call (not per descriptor, and nothing atomic over the host
  * link), positions from a ballot and a prefix popcount.  The single consumer frees slots
- * in position order, so one lane polling the wave's last slot is enough.  Records go out
+ * in position order, so one lane checking one slot is enough, and what it learns is kept
+ * in a device-resident horizon so that most calls read nothing over the host link.  Records go out
  * as four 16-byte stores per lane, then a system-scope release fence, then the sequence
  * words: the host proxy that sees a published sequence word sees the record.
  */
@@ -47,8 +48,13 @@ __device__ __forceinline__ int ofi_amd_gin_dev_put(const ofi_amd_gin_dev_ring_t 
 	const uint32_t leader = (uint32_t)__ffsll((unsigned long long)ballot) - 1u;
 	const uint32_t mask = ring.capacity - 1u;
 
-	uint32_t base = 0;
+	/* ring.reserve[0] is the cursor; ring.reserve[1] a horizon: every position below it is
+	 * known to have been freed by the consumer.  That is a fact that stays true (a freed
+	 * slot stays free until the one producer that reserved it publishes), so a stale or
+	 * smaller value is merely conservative and plain loads and stores suffice for it. */
+	uint32_t base = 0, horizon = 0;
 	if (lane == leader) {
+		horizon = __hip_atomic_load(ring.reserve + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 		base = __hip_atomic_fetch_add(ring.reserve, count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 	}
 	base = __shfl(base, (int)leader, 64);
@@ -57,18 +63,35 @@ __device__ __forceinline__ int ofi_amd_gin_dev_put(const ofi_amd_gin_dev_ring_t 
 	int timed_out = 0;
 	if (lane == leader) {
 		const uint32_t last_pos = base + count - 1u;
-		uint64_t spins = 0;
-		while (__hip_atomic_load(&ring.sequences[last_pos & mask], __ATOMIC_RELAXED,
-					 __HIP_MEMORY_SCOPE_SYSTEM) != last_pos) {
-			if (++spins > spin_limit) {
-				timed_out = 1;
-				break;
+		if ((int32_t)(last_pos - horizon) >= 0) {
+			/* Not known to be free.  The consumer frees slots in position order, so the
+			 * slot of a position being free implies it for every position before it:
+			 * look half a lap ahead first -- when the consumer keeps up, one read over
+			 * the host link then covers the next capacity / 2 descriptors of all the
+			 * ring's producers -- and fall back to waiting for the wave's own last slot. */
+			const uint32_t far_pos = last_pos + (ring.capacity >> 1);
+			uint32_t known = 0;
+			if (__hip_atomic_load(&ring.sequences[far_pos & mask], __ATOMIC_RELAXED,
+					      __HIP_MEMORY_SCOPE_SYSTEM) == far_pos) {
+				known = far_pos + 1u;
+			} else {
+				uint64_t spins = 0;
+				while (__hip_atomic_load(&ring.sequences[last_pos & mask], __ATOMIC_RELAXED,
+							 __HIP_MEMORY_SCOPE_SYSTEM) != last_pos) {
+					if (++spins > spin_limit) {
+						timed_out = 1;
+						break;
+					}
+					__builtin_amdgcn_s_sleep(16);
+				}
+				known = last_pos + 1u;
 			}
-			__builtin_amdgcn_s_sleep(16);
-		}
-		if (timed_out) {
-			__hip_atomic_fetch_or(ring.status, OFI_AMD_GIN_DEV_TIMEOUT_BIT, __ATOMIC_RELAXED,
-					      __HIP_MEMORY_SCOPE_SYSTEM);
+			if (timed_out) {
+				__hip_atomic_fetch_or(ring.status, OFI_AMD_GIN_DEV_TIMEOUT_BIT, __ATOMIC_RELAXED,
+						      __HIP_MEMORY_SCOPE_SYSTEM);
+			} else if ((int32_t)(known - horizon) > 0) {
+				__hip_atomic_store(ring.reserve + 1, known, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+			}
 		}
 	}
 	if (__shfl(timed_out, (int)leader, 64)) {

@@ -256,7 +256,7 @@ int ofi_amd_gin_producer_status(ofi_amd_gin_rings_t *rings);
 typedef struct {
 	void *records;       /* 64-byte records, [capacity] */
 	uint32_t *sequences; /* [capacity] */
-	uint32_t *reserve;   /* next position to hand out */
+	uint32_t *reserve;   /* [0] next position to hand out, [1] positions below it are known free */
 	uint32_t *status;
 	uint32_t capacity;
 	uint32_t context;
