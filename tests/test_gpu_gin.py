@@ -178,6 +178,11 @@ def test_device_put_single_wave_keeps_table_order(lib, oracle, gpu):
     # a second launch on the same rings (seeded generator this time) continues at the cursor
     rc, stats, _d, _w = produce_and_drain(lib, rings, nctx, 500, mode=0)
     assert rc == 0 and stats.descriptors == nctx * 500
+    # and the device-side put again behind it: cursor and free-slot horizon carried over
+    assert lib.ofi_amd_gin_produce_table(rings, d_table.data_ptr(), ops, 1, 0, _gpu.stream()) == 0
+    rc, stats, got = drain_descs(lib, rings, nctx, ops)
+    assert rc == 0 and lib.ofi_amd_gin_producer_status(rings) == 0
+    assert np.array_equal(got, table)
     lib.ofi_amd_gin_rings_destroy(rings)
 
 
