@@ -262,14 +262,17 @@ __global__ __launch_bounds__(kBlock) void eager_copy_kernel(
 
 	if (flush != nullptr) {
 		__builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+		/* the first min(4, bytes) destination bytes, little-endian: lanes 0..3 read one byte
+		 * each in one instruction (the destination has no alignment to read a word from),
+		 * then the four are combined inside the quad */
+		uint32_t word = 0;
+		if (lane < min(bytes, 4u)) {
+			word = (uint32_t)__hip_atomic_load(d + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)
+			       << (8u * lane);
+		}
+		word |= __shfl_xor(word, 1, 64);
+		word |= __shfl_xor(word, 2, 64);
 		if (lane == 0) {
-			/* the first min(4, bytes) destination bytes, little-endian */
-			uint32_t word = 0;
-			for (uint32_t b = 0; b < min(bytes, 4u); b++) {
-				word |= (uint32_t)__hip_atomic_load(d + b, __ATOMIC_RELAXED,
-								    __HIP_MEMORY_SCOPE_WORKGROUP)
-					<< (8u * b);
-			}
 			flush[buf] = word;
 		}
 	}
