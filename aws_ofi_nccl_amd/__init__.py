@@ -173,7 +173,7 @@ class SendrecvLoopbackStats(ctypes.Structure):
     """ofi_amd_sendrecv_loopback_stats_t"""
     _fields_ = [("messages", c_u64), ("payload_bytes", c_u64), ("eager_messages", c_u64),
                 ("write_messages", c_u64), ("rdma_writes", c_u64), ("copy_entries", c_u64),
-                ("rounds", c_u64), ("launches", c_u64), ("send_again", c_u64),
+                ("rounds", c_u64), ("launches", c_u64), ("send_again", c_u64), ("flushes", c_u64),
                 ("seconds", ctypes.c_double)]
 
 
@@ -370,6 +370,10 @@ PROTOTYPES = {
     "ofi_amd_recv_comm_test": (ctypes.c_int, [c_vp, c_i32, ctypes.POINTER(ctypes.c_int),
                                               ctypes.POINTER(ctypes.c_int)]),
     "ofi_amd_recv_comm_state": (None, [c_vp, ctypes.POINTER(RecvState)]),
+    "ofi_amd_recv_comm_flush": (ctypes.c_int, [c_vp, ctypes.c_int, ctypes.POINTER(ctypes.c_int),
+                                               ctypes.POINTER(c_i32)]),
+    "ofi_amd_recv_comm_flush_test": (ctypes.c_int, [c_vp, c_i32, c_vp, c_u32, c_u64,
+                                                    ctypes.POINTER(ctypes.c_int)]),
     "ofi_amd_sendrecv_loopback_run": (ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_u64, c_u32, c_u32, c_u32,
                                                      c_vp, c_u64, c_u32, c_vp,
                                                      ctypes.POINTER(SendrecvLoopbackStats)]),

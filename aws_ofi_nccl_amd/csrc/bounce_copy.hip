@@ -464,20 +464,8 @@ int ofi_amd_flush_post(const void *d_flush_buf, void *slots_dev, uint32_t num_ra
 	return 0;
 }
 
-/* has_flush_completed, src/nccl_ofi_rdma.cpp:2110-2126: only the first 8 bytes of a slot count */
-int ofi_amd_flush_test(const void *slots_host, uint32_t num_rails, uint64_t sentinel)
-{
-	if (!slots_host || num_rails < 1 || num_rails > OFI_AMD_MAX_NUM_RAILS) {
-		return -EINVAL;
-	}
-	const uint64_t *slots = static_cast<const uint64_t *>(slots_host);
-	for (uint32_t r = 0; r < num_rails; r++) {
-		if (__atomic_load_n(&slots[r * 8u], __ATOMIC_ACQUIRE) != sentinel) {
-			return 0;
-		}
-	}
-	return 1;
-}
+/* ofi_amd_flush_test, the host side of the flush, lives with the other host-only wire code
+ * (wire_codec.cpp). */
 
 /* ---- nccl_ofi_device_copy (include/nccl_ofi_device_copy.h:14-69) ---- */
 

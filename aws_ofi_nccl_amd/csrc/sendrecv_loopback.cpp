@@ -106,6 +106,12 @@ extern "C" int ofi_amd_sendrecv_loopback_run(const uint64_t *src_addrs, const ui
 	if (rc == 0) rc = e_dst.alloc(sizeof(uint64_t) * inflight);
 	if (rc == 0) rc = e_cap.alloc(sizeof(uint32_t) * inflight);
 	if (rc == 0) rc = e_copied.alloc(sizeof(uint32_t) * inflight);
+	/* the receiver's flush: a 64-byte sentinel buffer on the device, one 64-byte host slot per rail */
+	pinned_t flush_slots;
+	void *d_flush_buf = nullptr;
+	if (rc == 0) rc = flush_slots.alloc(64 * OFI_AMD_WIRE_MAX_RAILS);
+	if (rc == 0) rc = ofi_amd_gpu_mem_alloc(&d_flush_buf, 64);
+	if (rc == 0) rc = ofi_amd_flush_buffer_fill(d_flush_buf, OFI_AMD_RDMA_FLUSH_SENTINEL, stream);
 	try {
 		open.reserve(inflight);
 		items.resize(inflight);
@@ -116,6 +122,8 @@ extern "C" int ofi_amd_sendrecv_loopback_run(const uint64_t *src_addrs, const ui
 		for (pinned_t *p : { &t_src, &t_dst, &t_len, &hdrs, &e_rx, &e_len, &e_dst, &e_cap, &e_copied }) {
 			p->release();
 		}
+		flush_slots.release();
+		if (d_flush_buf) (void)ofi_amd_gpu_mem_free(d_flush_buf);
 		if (sc) (void)ofi_amd_send_comm_destroy(sc);
 		if (rcv) (void)ofi_amd_recv_comm_destroy(rcv);
 	};
@@ -255,7 +263,34 @@ extern "C" int ofi_amd_sendrecv_loopback_run(const uint64_t *src_addrs, const ui
 						      static_cast<uint32_t *>(e_copied.dev), nullptr, stream);
 			st.launches++;
 		}
-		if (rc == 0) rc = ofi_amd_gpu_stream_synchronize(stream);
+		/* ---- receiver: flush, as NCCL asks for after receives into GPU memory.  The sentinel
+		 * read-back is queued behind the round's launches, so its arrival in the host slots
+		 * also says that they are done; a round that moved no byte needs no flush and just
+		 * waits for the stream. ---- */
+		if (rc == 0) {
+			int any_bytes = 0;
+			for (const open_msg_t &m : open) {
+				any_bytes |= m.action.size != 0;
+			}
+			int32_t flush_req = -1;
+			rc = ofi_amd_recv_comm_flush(rcv, 1, &any_bytes, &flush_req);
+			if (rc == 0 && flush_req >= 0) {
+				std::memset(flush_slots.host, 0, 64 * OFI_AMD_WIRE_MAX_RAILS);
+				rc = ofi_amd_flush_post(d_flush_buf, flush_slots.dev, num_rails, stream);
+				st.launches++;
+				const auto w0 = clock::now();
+				for (int done = 0; rc == 0 && !done;) {
+					rc = ofi_amd_recv_comm_flush_test(rcv, flush_req, flush_slots.host, num_rails,
+									  OFI_AMD_RDMA_FLUSH_SENTINEL, &done);
+					if (!done && std::chrono::duration<double>(clock::now() - w0).count() > 20.0) {
+						rc = -ETIMEDOUT;
+					}
+				}
+				st.flushes++;
+			} else if (rc == 0) {
+				rc = ofi_amd_gpu_stream_synchronize(stream);
+			}
+		}
 		for (uint32_t k = 0, j = 0; k < n_items && rc == 0; k++) {
 			if (!items[k].needs_copy) {
 				continue;

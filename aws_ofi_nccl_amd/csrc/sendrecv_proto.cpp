@@ -652,6 +652,7 @@ struct ofi_amd_recv_comm {
 	uint32_t inflight_reqs = 0;
 	uint64_t n_ctrl_sent = 0;
 	uint32_t num_rails = 0;
+	bool flush_live[OFI_AMD_MAX_REQUESTS] = {}; /* flush requests share the in-flight limit */
 
 	int match_arrivals();
 	RecvReq *posted(uint16_t seq, int *stat);
@@ -979,6 +980,51 @@ int ofi_amd_recv_comm_test(ofi_amd_recv_comm_t *r, int32_t id, int *done, int *s
 	r->last_completed_seq = req.msg_seq_num;
 	r->inflight_reqs--;
 	r->reqs.give(id);
+	return 0;
+}
+
+/* flush, src/nccl_ofi_rdma.cpp:4405-4510: one flush covers every buffer of the call, and a
+ * call whose receives were all empty needs none */
+int ofi_amd_recv_comm_flush(ofi_amd_recv_comm_t *r, int n, const int *sizes, int32_t *req)
+{
+	if (!r || !sizes || !req || n < 1 || n > OFI_AMD_WIRE_MAX_RECVS) {
+		return -EINVAL;
+	}
+	*req = -1;
+	if (r->inflight_reqs == OFI_AMD_MAX_REQUESTS) {
+		return -ENOSPC;
+	}
+	bool any = false;
+	for (int i = 0; i < n; i++) {
+		any = any || sizes[i] != 0;
+	}
+	if (!any) {
+		return 0;
+	}
+	for (int32_t id = 0; id < OFI_AMD_MAX_REQUESTS; id++) {
+		if (!r->flush_live[id]) {
+			r->flush_live[id] = true;
+			r->inflight_reqs++;
+			*req = id;
+			return 0;
+		}
+	}
+	return -ENOSPC;
+}
+
+/* test() of a flush request: has_flush_completed, :2110-2126 */
+int ofi_amd_recv_comm_flush_test(ofi_amd_recv_comm_t *r, int32_t req, const void *slots_host,
+				 uint32_t num_rails, uint64_t sentinel, int *done)
+{
+	if (!r || !done || req < 0 || req >= OFI_AMD_MAX_REQUESTS || !r->flush_live[req] || !slots_host ||
+	    num_rails < 1 || num_rails > OFI_AMD_WIRE_MAX_RAILS) {
+		return -EINVAL;
+	}
+	*done = ofi_amd_flush_test(slots_host, num_rails, sentinel) == 1;
+	if (*done) {
+		r->flush_live[req] = false;
+		r->inflight_reqs--;
+	}
 	return 0;
 }
 

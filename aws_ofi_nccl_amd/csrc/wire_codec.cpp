@@ -10,6 +10,7 @@
 #include <new>
 #include <vector>
 
+#include "ofi_amd_hotpath.h"
 #include "ofi_amd_wire.h"
 
 namespace {
@@ -294,6 +295,22 @@ void ofi_amd_eager_tx_advance(ofi_amd_eager_tx_t *tx)
 int ofi_amd_eager_fits(uint64_t size, int64_t eager_send_size)
 {
 	return static_cast<int64_t>(size + OFI_AMD_EAGER_HEADER_SIZE) <= eager_send_size;
+}
+
+/* has_flush_completed, src/nccl_ofi_rdma.cpp:2110-2126: one 64-byte slot per rail, only the
+ * first 8 bytes of a slot count (declared in ofi_amd_hotpath.h beside the flush kernels) */
+int ofi_amd_flush_test(const void *slots_host, uint32_t num_rails, uint64_t sentinel)
+{
+	if (!slots_host || num_rails < 1 || num_rails > OFI_AMD_WIRE_MAX_RAILS) {
+		return -EINVAL;
+	}
+	const uint64_t *slots = static_cast<const uint64_t *>(slots_host);
+	for (uint32_t r = 0; r < num_rails; r++) {
+		if (__atomic_load_n(&slots[r * 8u], __ATOMIC_ACQUIRE) != sentinel) {
+			return 0;
+		}
+	}
+	return 1;
 }
 
 } /* extern "C" */

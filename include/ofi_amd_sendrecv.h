@@ -181,6 +181,17 @@ uint32_t ofi_amd_recv_comm_take_copies(ofi_amd_recv_comm_t *r, ofi_amd_eager_cop
 int ofi_amd_recv_comm_copy_done(ofi_amd_recv_comm_t *r, int32_t req, int32_t sub_idx);
 /* *done = 1 frees the request; sizes[0] for one receive, sizes[0..n) for a grouped one. */
 int ofi_amd_recv_comm_test(ofi_amd_recv_comm_t *r, int32_t req, int *done, int *sizes);
+/* The flush NCCL asks for after a receive into GPU memory (nccl_net_ofi_rdma_recv_comm::flush,
+ * :4405-4510).  One flush covers all n buffers; when every size is 0 none is needed and *req is
+ * -1.  Otherwise *req is a flush request (its own handle space; it counts against the same
+ * OFI_AMD_MAX_REQUESTS in-flight limit as receives: -ENOSPC when full) and the caller posts the
+ * read-back: ofi_amd_flush_post of the flush buffer into one 64-byte host slot per rail.
+ * _flush_test is has_flush_completed (:2110-2126) on those slots and frees the request when
+ * every slot shows the sentinel.  (The reference keeps the request until the completions of
+ * its loop-back reads have drained as well; a read-back done by a kernel has none.) */
+int ofi_amd_recv_comm_flush(ofi_amd_recv_comm_t *r, int n, const int *sizes, int32_t *req);
+int ofi_amd_recv_comm_flush_test(ofi_amd_recv_comm_t *r, int32_t req, const void *slots_host,
+				 uint32_t num_rails, uint64_t sentinel, int *done);
 void ofi_amd_recv_comm_state(const ofi_amd_recv_comm_t *r, ofi_amd_recv_state_t *out);
 
 /* ======================================================================
@@ -196,7 +207,9 @@ void ofi_amd_recv_comm_state(const ofi_amd_recv_comm_t *r, ofi_amd_recv_state_t 
  *   `group` (1..8) consecutive messages share one grouped receive request, matched by tag
  *   (tags NULL: 1..group within each request; tags given: distinct within a request).
  *   rx_pool: device-accessible memory, inflight x 8320 bytes.  flags bit 0: the receiver
- *   posts first, so nothing goes eager.  Blocks until done;
+ *   posts first, so nothing goes eager.  Each round of `inflight` messages ends with the
+ *   receiver's flush (ofi_amd_recv_comm_flush, the sentinel read-back of ofi_amd_flush_post)
+ *   and completes when the sentinels are in the host slots.  Blocks until done;
  *   `stream` carries the launches.  -EPROTO if the state machines disagree with the wire,
  *   -EIO if a size reported back is not the size moved.
  * ====================================================================== */
@@ -210,6 +223,7 @@ typedef struct {
 	uint64_t rounds;
 	uint64_t launches;
 	uint64_t send_again;    /* isend calls answered "call again" */
+	uint64_t flushes;       /* receiver flushes (one per round that moved data) */
 	double seconds;
 } ofi_amd_sendrecv_loopback_stats_t;
 

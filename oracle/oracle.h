@@ -492,6 +492,9 @@ int oracle_recv_comm_ctrl_sent(oracle_recv_comm_t *r, int32_t req);
 uint32_t oracle_recv_comm_take_copies(oracle_recv_comm_t *r, oracle_eager_copy_item_t *out, uint32_t cap);
 int oracle_recv_comm_copy_done(oracle_recv_comm_t *r, int32_t req, int32_t sub_idx);
 int oracle_recv_comm_test(oracle_recv_comm_t *r, int32_t req, int *done, int *sizes);
+int oracle_recv_comm_flush(oracle_recv_comm_t *r, int n, const int *sizes, int32_t *req);
+int oracle_recv_comm_flush_test(oracle_recv_comm_t *r, int32_t req, const uint64_t *slots,
+				uint32_t num_rails, uint64_t sentinel, int *done);
 void oracle_recv_comm_state(const oracle_recv_comm_t *r, oracle_recv_state_t *out);
 
 #ifdef __cplusplus

@@ -598,6 +598,7 @@ struct oracle_recv_comm {
 	uint32_t num_rails;
 	oracle_eager_copy_item_t copies[COPY_RING];
 	uint32_t copy_head, copy_count;
+	int flush_live[MAX_REQUESTS];
 };
 
 static void list_init(rx_node_t *h)
@@ -1015,6 +1016,52 @@ int oracle_recv_comm_test(oracle_recv_comm_t *r, int32_t id, int *done, int *siz
 	r->last_completed_seq = req->msg_seq_num;
 	r->num_inflight_reqs--;
 	req->in_use = 0;
+	return 0;
+}
+
+/* flush, src/nccl_ofi_rdma.cpp:4405-4510 (the fabric post is the caller's) */
+int oracle_recv_comm_flush(oracle_recv_comm_t *r, int n, const int *sizes, int32_t *req)
+{
+	*req = -1;
+	if (n < 1 || n > 8) {
+		return -22;
+	}
+	if (r->num_inflight_reqs == MAX_REQUESTS) {
+		return -28;
+	}
+	int flush_n = -1;
+	for (int recv_n = 0; recv_n < n; recv_n++) {
+		if (sizes[recv_n] != 0) {
+			flush_n = recv_n;
+			break;
+		}
+	}
+	if (flush_n == -1) {
+		return 0;
+	}
+	for (uint32_t i = 0; i < MAX_REQUESTS; i++) {
+		if (!r->flush_live[i]) {
+			r->flush_live[i] = 1;
+			r->num_inflight_reqs++;
+			*req = (int32_t)i;
+			return 0;
+		}
+	}
+	return -28;
+}
+
+/* has_flush_completed, :2110-2126, then the request is released */
+int oracle_recv_comm_flush_test(oracle_recv_comm_t *r, int32_t req, const uint64_t *slots,
+				uint32_t num_rails, uint64_t sentinel, int *done)
+{
+	if (req < 0 || (uint32_t)req >= MAX_REQUESTS || !r->flush_live[req]) {
+		return -22;
+	}
+	*done = oracle_flush_completed(slots, num_rails, sentinel);
+	if (*done) {
+		r->flush_live[req] = 0;
+		r->num_inflight_reqs--;
+	}
 	return 0;
 }
 

@@ -219,6 +219,8 @@ _ORACLE_PROTOS = {
     "oracle_recv_comm_copy_done": (c_int, [c_vp, c_i32, c_i32]),
     "oracle_recv_comm_test": (c_int, [c_vp, c_i32, ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
     "oracle_recv_comm_state": (None, [c_vp, ctypes.POINTER(RecvState)]),
+    "oracle_recv_comm_flush": (c_int, [c_vp, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_i32)]),
+    "oracle_recv_comm_flush_test": (c_int, [c_vp, c_i32, c_vp, c_u32, c_u64, ctypes.POINTER(c_int)]),
     "oracle_gin_cpu_rings_run": (c_int, [c_u64, c_u32, c_u64, c_u32, c_u32, c_u32, c_u32, c_u32, c_u32,
                                          ctypes.POINTER(c_u64), ctypes.POINTER(ctypes.c_double)]),
     "oracle_model_cost": (ctypes.c_float, [c_int, c_int, c_int, c_int, c_int, c_u64, c_u64, c_u64,

@@ -49,7 +49,13 @@ def run(lib, send_sizes, recv_sizes, inflight, flags=0, dst_skew=0, seed=0, grou
         assert np.all(got[:dst_skew] == 0xCD) and np.all(got[dst_skew + k:] == 0xCD), (i, "wrote outside")
     assert stats.messages == n and stats.payload_bytes == sum(min(s, r) for s, r in zip(send_sizes, recv_sizes))
     assert stats.eager_messages + stats.write_messages == n
+    assert stats.flushes <= stats.rounds and (stats.flushes == stats.rounds or 0 in send_sizes)
     return stats
+
+
+def test_round_without_a_byte_needs_no_flush(lib, gpu):
+    st = run(lib, [0] * 64 + [8] * 64, [16] * 128, 64)
+    assert st.rounds == 2 and st.flushes == 1 and st.eager_messages == 128
 
 
 @pytest.mark.parametrize("pair", PAIRS)
