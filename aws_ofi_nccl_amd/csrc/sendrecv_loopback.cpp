@@ -5,7 +5,8 @@
  * tests/functional/nccl_message_transfer.cpp:19-56).  An eager send becomes a device copy of header
  * and payload into an rx buffer; the RDMA writes of a rendezvous become device copies stripe by
  * stripe; what the receiver decides to copy out of rx buffers goes through the batched eager
- * copy.  `inflight` messages are open at a time; each round is two launches and one wait.
+ * copy.  `inflight` messages are open at a time; each round is at most three launches (the wire's
+ * copies, the eager copies, the flush read-back) and one wait on the flush slots.
  */
 #include <cerrno>
 #include <chrono>
@@ -327,6 +328,10 @@ extern "C" int ofi_amd_sendrecv_loopback_run(const uint64_t *src_addrs, const ui
 		st.rounds++;
 	}
 	st.seconds = std::chrono::duration<double>(clock::now() - t0).count();
+	if (rc != 0) {
+		/* a round that was given up may have launches in flight that read the tables freed below */
+		(void)ofi_amd_gpu_stream_synchronize(stream);
+	}
 	release();
 	*stats = st;
 	return rc;
