@@ -428,9 +428,10 @@ int ofi_amd_sched_batch(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes,
 
 	const uint32_t passes = pick_passes(n);
 	const uint32_t tiles = (uint32_t)((n + kThreads * passes - 1) / (kThreads * passes));
-	uint32_t *totals, *prefix, *seed0;
 	hipStream_t s = as_stream(stream);
 	try {
+		/* held until the launches are queued: two threads submitting to one stream share its
+		 * scratch, and their count/emit pairs must not interleave */
 		std::lock_guard<std::mutex> g(g_ws_lock);
 		workspace_t &ws = g_ws_by_stream[stream];
 		if (tiles > ws.tiles) {
@@ -449,19 +450,16 @@ int ofi_amd_sched_batch(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes,
 			ws.prefix = b;
 			ws.tiles = want;
 		}
-		totals = ws.totals;
-		prefix = ws.prefix;
-		seed0 = ws.prefix + ws.tiles;
+		uint32_t *seed0 = ws.prefix + ws.tiles;
+		if (passes == kPassesSmall) {
+			launch_batch<kPassesSmall>(s, tiles, d_sizes, (uint32_t)n, d_state, align, ws.totals, ws.prefix,
+						   seed0, d_num_xfers, reinterpret_cast<u32x4 *>(d_xfers), err);
+		} else {
+			launch_batch<kPassesLarge>(s, tiles, d_sizes, (uint32_t)n, d_state, align, ws.totals, ws.prefix,
+						   seed0, d_num_xfers, reinterpret_cast<u32x4 *>(d_xfers), err);
+		}
 	} catch (...) {
 		return -ENOMEM;
-	}
-
-	if (passes == kPassesSmall) {
-		launch_batch<kPassesSmall>(s, tiles, d_sizes, (uint32_t)n, d_state, align, totals, prefix, seed0,
-					   d_num_xfers, reinterpret_cast<u32x4 *>(d_xfers), err);
-	} else {
-		launch_batch<kPassesLarge>(s, tiles, d_sizes, (uint32_t)n, d_state, align, totals, prefix, seed0,
-					   d_num_xfers, reinterpret_cast<u32x4 *>(d_xfers), err);
 	}
 	OFI_AMD_HIP_TRY(hipGetLastError());
 	return 0;

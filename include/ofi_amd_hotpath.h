@@ -10,6 +10,15 @@
  * memory); all others are ordinary host pointers.  Every entry point that needs
  * the GPU returns -ENODEV when no device is present; nothing falls back to the
  * CPU.
+ *
+ * Threads: the batch launches (sections 2 and 3) keep no state between calls and
+ * may be called from any thread on any stream; ofi_amd_sched_batch serialises
+ * its own per-stream scratch, the caller orders batches that share one
+ * scheduler state.  An object (tuner plan, GIN rings' consumer side, GIN
+ * receiver, send or receive comm) belongs to one thread at a time, as a comm
+ * belongs to its proxy thread in NCCL; a ring takes any number of producers;
+ * the message buffer and the tuner plugin contexts lock themselves as the
+ * reference's do.
  */
 #ifndef OFI_AMD_HOTPATH_H_
 #define OFI_AMD_HOTPATH_H_
