@@ -621,6 +621,7 @@ def main():
         "cpu_baseline": cpu,
         "parity_ok": bounce["parity_ok"],
         "gin_puts_per_s": extra.get("gin", {}).get("drain", {}).get("descs_per_s"),
+        "gin_puts_per_s_4_proxy_threads": extra.get("gin", {}).get("drain_4_proxy_threads", {}).get("descs_per_s"),
         "extra": extra,
     }
     print(json.dumps(line))
