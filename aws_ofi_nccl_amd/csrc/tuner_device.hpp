@@ -199,6 +199,7 @@ struct region_tables_t {
 	int32_t set_count[kNumPlatforms][kNumShapes][NUM_FUNCS];
 	const int32_t *poly; /* per polygon {algo, proto, first_vertex, num_vertices} */
 	const pt_t *verts;   /* log2 space */
+	const double *bbox;  /* per polygon {min_x, max_x, min_y, max_y} as is_inside_region finds them */
 	pt_t far_point;      /* log2 of (2*max size, 2*max ranks) */
 };
 
@@ -248,11 +249,73 @@ __device__ inline double seg_distance(pt_t x, pt_t y0, pt_t y1, double eps)
 	return sqrt(vdot(s, s));
 }
 
-/* is_inside_region, :159-221 */
-__device__ inline int inside_region(pt_t point, const pt_t *v, int n, pt_t far_point)
+/*
+ * Shortcuts for the two per-edge tests.  Each evaluates the quotient of `intersect` with an
+ * approximate reciprocal (hardware estimate plus one Newton step: relative error below 1e-12
+ * against the 1e-5 margins used here) and answers only when the exact code's answer is already
+ * certain; everything else -- a quotient near one of the thresholds, a degenerate edge -- goes
+ * through the exact division and square root above.  Results are therefore those of the exact
+ * code; what is saved is two or three fp64 divisions and a square root per edge.
+ */
+__device__ __forceinline__ double approx_rcp(double d)
 {
-	const double eps = 1e-10;
-	/* y bounds start from vertex 1 as in the reference (:177-178) */
+	double r = __builtin_amdgcn_rcp(d);
+	return r * (2.0 - d * r);
+}
+
+/* |a - t| far beyond what the approximate quotient can be off by */
+__device__ __forceinline__ bool clear_of(double a, double t)
+{
+	return fabs(a - t) > 1e-5 * (1.0 + fabs(a));
+}
+
+/* intersect(x0, x1, y0, y1, eps, nullptr) == 1 */
+__device__ inline bool crosses_edge(pt_t x0, pt_t x1, pt_t y0, pt_t y1, double eps)
+{
+	const pt_t dx = vsub(x1, x0);
+	const pt_t dy = vsub(y1, y0);
+	const double d = vcross(dy, dx);
+	if (fabs(d) < eps) {
+		return false;
+	}
+	const double r = approx_rcp(d);
+	const double a = (vcross(x0, dx) - vcross(y0, dx)) * r;
+	if (clear_of(a, 0.0) && clear_of(a, 1.0)) {
+		if (a < 0.0 || a > 1.0) {
+			return false; /* beyond -eps or 1 + eps */
+		}
+		const double b = (vcross(x0, dy) - vcross(y0, dy)) * r;
+		if (clear_of(b, 0.0) && clear_of(b, 1.0)) {
+			return b > 0.0 && b < 1.0;
+		}
+	}
+	return intersect(x0, x1, y0, y1, eps, nullptr) == 1;
+}
+
+/* false only when seg_distance(x, y0, y1, eps) is certainly not below eps */
+__device__ inline bool may_touch_edge(pt_t x, pt_t y0, pt_t y1, double eps)
+{
+	const pt_t dy = vsub(y1, y0);
+	pt_t x1;
+	x1.x = x.x + dy.y;
+	x1.y = x.y - dy.x;
+	const pt_t dx = vsub(x1, x);
+	const double d = vcross(dy, dx);
+	if (fabs(d) < eps) {
+		return true; /* the exact code leaves the foot point unset here */
+	}
+	const double a = (vcross(x, dx) - vcross(y0, dx)) * approx_rcp(d);
+	const pt_t s = { y0.x + a * dy.x - x.x, y0.y + a * dy.y - x.y };
+	/* the foot point computed exactly differs from this one by ~1e-12 (1 + |a|)(1 + |dy|) at most */
+	const double far = 1e-4 * (1.0 + fabs(a)) * (1.0 + fabs(dy.x) + fabs(dy.y));
+	return !(vdot(s, s) > far * far);
+}
+
+/* The bounds is_inside_region computes (:177-196): selections only, so the host can do it
+ * once per polygon with the same result.  The y bounds start from vertex 1 as in the reference
+ * (:177-178). */
+__host__ __device__ inline void region_bounds(const pt_t *v, int n, double out[4])
+{
 	double min_x = v[0].x, max_x = v[0].x, min_y = v[1].y, max_y = v[1].y;
 	for (int i = 0; i < n; i++) {
 		if (v[i].x > max_x) max_x = v[i].x;
@@ -260,6 +323,18 @@ __device__ inline int inside_region(pt_t point, const pt_t *v, int n, pt_t far_p
 		if (v[i].y > max_y) max_y = v[i].y;
 		if (v[i].y < min_y) min_y = v[i].y;
 	}
+	out[0] = min_x;
+	out[1] = max_x;
+	out[2] = min_y;
+	out[3] = max_y;
+}
+
+/* is_inside_region, :159-221; `bounds` is region_bounds of the same polygon */
+__device__ __forceinline__ int inside_region(pt_t point, const pt_t *v, int n, const double *bounds,
+					      pt_t far_point)
+{
+	const double eps = 1e-10;
+	const double min_x = bounds[0], max_x = bounds[1], min_y = bounds[2], max_y = bounds[3];
 	/* The reference looks for a point on an edge first (result 0) and rejects by bounding
 	 * box second (result -1).  A point more than 1e-6 outside the box cannot be within
 	 * 1e-10 of an edge -- edges lie inside the box, and the foot of the perpendicular may
@@ -273,7 +348,7 @@ __device__ inline int inside_region(pt_t point, const pt_t *v, int n, pt_t far_p
 	}
 	for (int i = 0; i < n; i++) {
 		int k = (i + 1) % n;
-		if (seg_distance(point, v[i], v[k], eps) < eps) {
+		if (may_touch_edge(point, v[i], v[k], eps) && seg_distance(point, v[i], v[k], eps) < eps) {
 			return 0;
 		}
 	}
@@ -283,7 +358,7 @@ __device__ inline int inside_region(pt_t point, const pt_t *v, int n, pt_t far_p
 	int crosses = 0;
 	for (int i = 0; i < n; i++) {
 		int k = (i + 1) % n;
-		if (intersect(point, far_point, v[i], v[k], eps, nullptr) == 1) {
+		if (crosses_edge(point, far_point, v[i], v[k], eps)) {
 			crosses++;
 		}
 	}
@@ -325,43 +400,53 @@ __device__ __forceinline__ int log2i_nodes(uint64_t nodes)
 	return x <= 0 ? -1 : 31 - __clz(x);
 }
 
-/* region_get_coll_info_internal_v3, :2070-2157.  Regions whose (algo, proto) bit is
- * clear in `mask` are passed over: for v3 those are the cells NCCL marked -1 or that
- * lie beyond numAlgo / numProto (:2109-2114); for v2 PAT and, without NVLS support,
- * NVLS tree (:2023-2030).  p = (log2 bytes, log2 ranks) as transform_log2 gives them. */
-__device__ inline void region_choose(const region_tables_t &t, int platform, int coll, uint64_t size,
-				     uint64_t ranks, uint64_t nodes, pt_t p, uint32_t mask,
-				     int &algorithm, int &protocol, int &nchannels)
+/* Which polygon set answers for (platform, collective, ranks per node): shape selection as in
+ * the per-platform init functions (:302,:485,:675,:768,:878,...).  count 0: no regions. */
+__device__ __forceinline__ void region_set(const region_tables_t &t, int platform, int coll, uint64_t ranks,
+					    uint64_t nodes, int &first, int &count)
 {
-	algorithm = -1;
-	protocol = -1;
-	nchannels = -1;
-	/* shape selection as in the per-platform init functions (:302,:485,:675,:768,:878,...) */
+	first = 0;
+	count = 0;
 	int shape = -1;
 	if (ranks == 8 * nodes) shape = 0;
 	else if (ranks == 2 * nodes && platform == OFI_AMD_PLATFORM_P5_P5E) shape = 1;
 	else if (ranks == nodes) shape = 2;
 	if (platform < 0 || platform >= kNumPlatforms || shape < 0 || coll < 0 || coll >= NUM_FUNCS ||
-	    t.set_count[platform][shape][coll] <= 0 || nodes <= 2) {
+	    t.set_count[platform][shape][coll] <= 0) {
 		return;
 	}
-	const int first = t.set_first[platform][shape][coll];
-	const int count = t.set_count[platform][shape][coll];
-	int in_out = -1, a = -1, pr = -1;
+	first = t.set_first[platform][shape][coll];
+	count = t.set_count[platform][shape][coll];
+}
+
+/* The loop of region_get_coll_info_internal_v3 (:2106-2128) over one set: the first polygon that
+ * holds the point (inside or on an edge) wins.  Regions whose (algo, proto) bit is clear in
+ * `mask` are passed over: for v3 those are the cells NCCL marked -1 or that lie beyond numAlgo /
+ * numProto (:2109-2114); for v2 PAT and, without NVLS support, NVLS tree (:2023-2030).
+ * poly: 4 ints per polygon, its vertex index relative to `verts`; bounds: 4 doubles per polygon.
+ * The arrays may live in global memory or in LDS. */
+__device__ __forceinline__ int region_pick(const int32_t *poly, const double *bounds, const pt_t *verts,
+					    int count, pt_t p, uint32_t mask, pt_t far_point, int &a, int &pr)
+{
+	int in_out = -1;
+	a = -1;
+	pr = -1;
 	for (int i = 0; i < count && in_out < 0; i++) {
-		const int32_t *poly = &t.poly[(first + i) * 4];
-		a = poly[0];
-		pr = poly[1];
+		a = poly[i * 4 + 0];
+		pr = poly[i * 4 + 1];
 		if (!allowed(mask, a, pr)) {
 			continue;
 		}
-		in_out = inside_region(p, &t.verts[poly[2]], poly[3], t.far_point);
+		in_out = inside_region(p, &verts[poly[i * 4 + 2]], poly[i * 4 + 3], &bounds[i * 4], far_point);
 	}
-	if (in_out < 0) {
-		return;
-	}
-	algorithm = a;
-	protocol = pr;
+	return in_out;
+}
+
+/* The nChannels override of the chosen region (:2135-2153), -1 when there is none. */
+__device__ __forceinline__ int region_channels(int platform, uint64_t size, uint64_t ranks, uint64_t nodes,
+						int algorithm, int protocol)
+{
+	int nchannels = -1;
 	if (platform == OFI_AMD_PLATFORM_P6 && size >= 4 * 1024 * 1024 && size <= 32 * 1024 * 1024 &&
 	    algorithm == ALGO_TREE && protocol == PROTO_LL128 && nodes * 8 == ranks) { /* :2140-2146 */
 		const int log2_nnodes = log2i_nodes(nodes);
@@ -384,6 +469,30 @@ __device__ inline void region_choose(const region_tables_t &t, int platform, int
 		if (size <= nodes * 65536) nchannels = 1;
 		else if (size <= nodes * 65536 * 2) nchannels = 2;
 	}
+	return nchannels;
+}
+
+/* region_get_coll_info_internal_v3, :2070-2157, for one point with the tables in global memory.
+ * p = (log2 bytes, log2 ranks) as transform_log2 gives them. */
+__device__ inline void region_choose(const region_tables_t &t, int platform, int coll, uint64_t size,
+				     uint64_t ranks, uint64_t nodes, pt_t p, uint32_t mask,
+				     int &algorithm, int &protocol, int &nchannels)
+{
+	algorithm = -1;
+	protocol = -1;
+	nchannels = -1;
+	int first, count;
+	region_set(t, platform, coll, ranks, nodes, first, count);
+	if (count <= 0 || nodes <= 2) {
+		return;
+	}
+	int a, pr;
+	if (region_pick(&t.poly[first * 4], &t.bbox[first * 4], t.verts, count, p, mask, t.far_point, a, pr) < 0) {
+		return;
+	}
+	algorithm = a;
+	protocol = pr;
+	nchannels = region_channels(platform, size, ranks, nodes, a, pr);
 }
 
 /* region_get_chunk_size_internal, :2276-2306, with chunkSizeTuningTreeLL128P5en

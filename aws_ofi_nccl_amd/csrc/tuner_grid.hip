@@ -92,33 +92,76 @@ __global__ __launch_bounds__(256) void model_grid_kernel(grid_dims_t g,
 	}
 }
 
-/* One thread per point; blockIdx.y is the platform entry. */
-__global__ __launch_bounds__(256) void region_choice_kernel(grid_dims_t g, region_tables_t t,
+constexpr int kMaxSetPolys = 8;  /* polygons of one (platform, shape, collective) set */
+constexpr int kMaxSetVerts = 64; /* their vertices together */
+constexpr uint32_t kRegionBlock = 64; /* threads per workgroup of the region kernel: one wavefront */
+static_assert(kRegionBlock >= (uint32_t)kMaxSetVerts && kRegionBlock >= (uint32_t)kMaxSetPolys * 4,
+	      "one thread per staged vertex and per staged polygon word");
+
+/*
+ * One thread per point; blockIdx.y is the platform entry.  A workgroup works on one (collective,
+ * ranks per node) pair -- `blocks_per_run` workgroups share the pair's n_sizes x n_nodes points,
+ * node count fastest -- because the polygon set depends on that pair alone: the set (at most 8
+ * polygons, 64 vertices, with their bounds) is copied into LDS once and every lane then walks
+ * the same polygons out of LDS instead of chasing them through global memory, and workgroups of
+ * pairs without regions leave after one table lookup.
+ */
+__global__ __launch_bounds__(kRegionBlock) void region_choice_kernel(grid_dims_t g, region_tables_t t,
 							    const int32_t *__restrict__ platforms,
-							    uint32_t points_per_platform,
-							    int8_t *__restrict__ choice)
+							    uint32_t points_per_platform, uint32_t blocks_per_run,
+							    uint32_t spread, int8_t *__restrict__ choice)
 {
-	const uint32_t t_idx = blockIdx.x * 256u + threadIdx.x;
-	if (t_idx >= points_per_platform) {
+	__shared__ int32_t s_poly[kMaxSetPolys * 4];
+	__shared__ double s_bounds[kMaxSetPolys * 4];
+	__shared__ pt_t s_verts[kMaxSetVerts];
+
+	/* Workgroups go to the eight XCDs in turn, and the pairs that have regions sit at a fixed
+	 * period in the run index: taken in launch order, all the long-running workgroups would land
+	 * on the same few XCDs.  `spread` is coprime to the grid width, so this is a permutation
+	 * that scatters every period over all XCDs. */
+	const uint32_t block = (uint32_t)(((uint64_t)blockIdx.x * spread) % gridDim.x);
+	const uint32_t run = block / blocks_per_run;
+	const uint32_t in_run = (block - run * blocks_per_run) * kRegionBlock + threadIdx.x;
+	const uint32_t pi = run % g.n_ppn;
+	const uint32_t ci = run / g.n_ppn;
+	const int platform = platforms[blockIdx.y];
+	const int coll = g.colls[ci];
+	const uint32_t ppn = g.ppn[pi];
+
+	/* ranks = nodes * ppn with nodes >= 1: the shape is a function of ppn */
+	int first, count;
+	region_set(t, platform, coll, ppn, 1, first, count);
+	if (count > 0) {
+		const int v0 = t.poly[first * 4 + 2];
+		const int v_end = t.poly[(first + count - 1) * 4 + 2] + t.poly[(first + count - 1) * 4 + 3];
+		if ((int)threadIdx.x < count * 4) {
+			const int32_t w = t.poly[first * 4 + threadIdx.x];
+			s_poly[threadIdx.x] = (threadIdx.x & 3u) == 2u ? w - v0 : w; /* vertex index within the set */
+			s_bounds[threadIdx.x] = t.bbox[first * 4 + threadIdx.x];
+		}
+		if ((int)threadIdx.x < v_end - v0) {
+			s_verts[threadIdx.x] = t.verts[v0 + threadIdx.x];
+		}
+		__syncthreads();
+	}
+	if (in_run >= g.n_sizes * g.n_nodes) {
 		return;
 	}
-	/* Threads are laid out with the node count fastest, then the size, then ranks per node,
-	 * then the collective -- not in output order.  Which polygon set a point is tested
-	 * against depends on (collective, ranks per node): this way the lanes of a wavefront
-	 * walk the same polygons instead of serialising over up to four different sets (and
-	 * whole wavefronts of shapes without regions leave at once). */
-	uint32_t r = t_idx;
-	const uint32_t ni = r % g.n_nodes; r /= g.n_nodes;
-	const uint32_t si = r % g.n_sizes; r /= g.n_sizes;
-	const uint32_t pi = r % g.n_ppn; r /= g.n_ppn;
-	const uint32_t ci = r;
+	const uint32_t ni = in_run % g.n_nodes;
+	const uint32_t si = in_run / g.n_nodes;
 	const uint32_t p = ((ci * g.n_sizes + si) * g.n_nodes + ni) * g.n_ppn + pi; /* output order */
 
 	const uint64_t nodes = g.nodes[ni];
-	int algorithm, protocol, nchannels;
-	region_choose(t, platforms[blockIdx.y], g.colls[ci], g.sizes[si], nodes * g.ppn[pi], nodes,
-		      pt_t{ g.log2_sizes[si], g.log2_ranks[ni * g.n_ppn + pi] }, kAllAllowed, algorithm,
-		      protocol, nchannels);
+	int algorithm = -1, protocol = -1, nchannels = -1;
+	if (count > 0 && nodes > 2) {
+		int a, pr;
+		const pt_t at = { g.log2_sizes[si], g.log2_ranks[ni * g.n_ppn + pi] };
+		if (region_pick(s_poly, s_bounds, s_verts, count, at, kAllAllowed, t.far_point, a, pr) >= 0) {
+			algorithm = a;
+			protocol = pr;
+			nchannels = region_channels(platform, g.sizes[si], nodes * ppn, nodes, a, pr);
+		}
+	}
 	const uint64_t idx = (uint64_t)blockIdx.y * points_per_platform + p;
 	/* {int8 algorithm, int8 protocol, int16 nchannels} as one 4-byte store */
 	reinterpret_cast<uint32_t *>(choice)[idx] = ((uint32_t)(uint8_t)(int8_t)algorithm) |
@@ -177,6 +220,7 @@ int build_region_tables(region_tables_t *t)
 {
 	std::vector<int32_t> poly;
 	std::vector<pt_t> verts;
+	std::vector<double> bounds;
 	for (int p = 0; p < kNumPlatforms; p++) {
 		for (int s = 0; s < kNumShapes; s++) {
 			for (int c = 0; c < NUM_FUNCS; c++) {
@@ -199,9 +243,13 @@ int build_region_tables(region_tables_t *t)
 		}
 		t->set_first[set[0]][shape][set[2]] = (int32_t)(poly.size() / 4);
 		t->set_count[set[0]][shape][set[2]] = set[4];
+		const size_t set_first_vertex = verts.size();
+		if (set[4] > kMaxSetPolys) {
+			return -EINVAL;
+		}
 		for (int q = 0; q < set[4]; q++) {
 			const int *pd = ofi_region_polys[set[3] + q];
-			if (pd[3] > kMaxVertices) {
+			if (pd[3] < 2 || pd[3] > kMaxVertices) {
 				return -EINVAL;
 			}
 			poly.push_back(pd[0]);
@@ -220,21 +268,33 @@ int build_region_tables(region_tables_t *t)
 										: ext[(kind[1] - 1) / 2].y);
 				verts.push_back(to_log2(pt)); /* set_regions, :236-247 */
 			}
+			double b[4];
+			region_bounds(&verts[verts.size() - pd[3]], pd[3], b);
+			bounds.insert(bounds.end(), b, b + 4);
+		}
+		if (verts.size() - set_first_vertex > (size_t)kMaxSetVerts) {
+			return -EINVAL; /* the grid kernel keeps one set in LDS */
 		}
 	}
 	t->far_point = to_log2(pt_t{ 2.0 * kTunerMaxSize, 2.0 * kTunerMaxRanks });
 	int32_t *d_poly = nullptr;
 	pt_t *d_verts = nullptr;
+	double *d_bounds = nullptr;
 	int rc = upload(poly, &d_poly);
 	if (rc == 0) {
 		rc = upload(verts, &d_verts);
 	}
+	if (rc == 0) {
+		rc = upload(bounds, &d_bounds);
+	}
 	if (rc != 0) {
 		(void)hipFree(d_poly);
+		(void)hipFree(d_verts);
 		return rc;
 	}
 	t->poly = d_poly;
 	t->verts = d_verts;
+	t->bbox = d_bounds;
 	return 0;
 }
 
@@ -504,8 +564,30 @@ int ofi_amd_tuner_region_grid(ofi_amd_tuner_plan_t *plan, const int32_t *platfor
 		return -EINVAL;
 	}
 	const uint32_t points = (uint32_t)plan->points;
-	hipLaunchKernelGGL(region_choice_kernel, dim3((points + 255u) / 256u, n_platforms), dim3(256), 0, s,
-			   plan->g, plan->t, plan->d_platforms, points, d_choice);
+	const uint64_t run_len = (uint64_t)plan->g.n_sizes * plan->g.n_nodes;
+	const uint64_t blocks_per_run = (run_len + kRegionBlock - 1) / kRegionBlock;
+	const uint64_t blocks = blocks_per_run * plan->g.n_colls * plan->g.n_ppn;
+	if (blocks == 0 || blocks > 0x7fffffffull) {
+		return -EINVAL;
+	}
+	/* a multiplier near blocks / golden ratio, coprime to blocks */
+	uint64_t spread = (uint64_t)((double)blocks * 0.6180339887498949);
+	spread = spread < 1 ? 1 : spread;
+	for (;;) {
+		uint64_t a = spread, b = blocks;
+		while (b != 0) {
+			const uint64_t r = a % b;
+			a = b;
+			b = r;
+		}
+		if (a == 1) {
+			break;
+		}
+		spread++;
+	}
+	hipLaunchKernelGGL(region_choice_kernel, dim3((uint32_t)blocks, n_platforms), dim3(kRegionBlock), 0, s,
+			   plan->g, plan->t, plan->d_platforms, points, (uint32_t)blocks_per_run, (uint32_t)(spread % blocks),
+			   d_choice);
 	OFI_AMD_HIP_TRY(hipGetLastError());
 	return 0;
 }
