@@ -28,8 +28,14 @@
  *   region geometry  ~70 points + 4 extend_region cases of
  *                    tests/unit/region_based_tuner.cpp
  *   region tables    re-parsed from the reference source text and compared
- *   region decisions full-grid fp bits: PARITY UNPINNED (reference object not
- *                    buildable here); pinned only through the two rows above
+ *   region decisions (algorithm, protocol) over the configured grid and random points of
+ *                    all four platforms against a textbook even-odd point-in-polygon
+ *                    rule on the same tables (another ray than the reference's), first
+ *                    polygon in table order wins; points within 1e-6 of an edge, where
+ *                    the reference's epsilon rules decide and not geometry, rest on the
+ *                    geometry row above alone.  nChannels / chunk sizes: hand-derived
+ *                    spot values only, PARITY UNPINNED beyond them (reference object
+ *                    not buildable here)
  *   model cost       exact-rational closed forms to 1e-6 rel., linearity and
  *                    protocol-ratio identities; exact fp32 bit pattern of the
  *                    reference binary: PARITY UNPINNED (not buildable here)

@@ -1,7 +1,8 @@
 """Pins the tuner oracle.
 
 Regions: the reference's own unit test (tests/unit/region_based_tuner.cpp:20-248) is replayed
-point by point, and the polygon table is re-derived from the reference source text.
+point by point, the polygon table is re-derived from the reference source text, and the
+decisions over the whole grid are compared with a textbook even-odd point-in-polygon rule.
 Model: the reference has no test of its cost function and its object does not build here, so
 the oracle is checked against the closed forms in exact rational arithmetic (1e-6 relative, the
 tolerance the task states for costs) and against identities a dropped term or a swapped
@@ -310,3 +311,68 @@ def test_channel_and_chunk_heuristics(oracle):
     assert out.value == 131072        # 1 MiB: cap step -> 512 KiB; 2 < 8 -> 256 K (4) -> 128 K (8 >= 8)
     assert oracle.oracle_region_chunk_size(0, AR, 1 << 20, TREE, LL128, 8, 8, ctypes.byref(out)) == 0
     assert oracle.oracle_region_chunk_size(1, AR, 1 << 20, TREE, LL128, 64, 8, ctypes.byref(out)) == 0
+
+
+def _independent_region_choice(polys, px, py):
+    """First polygon in table order that holds (px, py) by the even-odd rule along a horizontal ray
+    towards +x -- not the reference's ray to a far corner -- and the distance to the nearest edge of
+    any polygon of the set.  polys: [(algo, proto, [(x, y), ...]), ...] in log2 space."""
+    nearest = math.inf
+    found = None
+    for algo, proto, vs in polys:
+        crossings = 0
+        for i in range(len(vs)):
+            (x1, y1), (x2, y2) = vs[i], vs[(i + 1) % len(vs)]
+            ex, ey = x2 - x1, y2 - y1
+            ee = ex * ex + ey * ey
+            t = 0.0 if ee == 0 else max(0.0, min(1.0, ((px - x1) * ex + (py - y1) * ey) / ee))
+            nearest = min(nearest, math.hypot(px - (x1 + t * ex), py - (y1 + t * ey)))
+            if (y1 > py) != (y2 > py) and x1 + (py - y1) * ex / ey > px:
+                crossings += 1
+        if found is None and crossings % 2 == 1:
+            found = (algo, proto)
+    return found or (-1, -1), nearest
+
+
+def test_region_decisions_against_an_independent_point_in_polygon_rule(oracle):
+    """(algorithm, protocol) of the oracle's region decision over the configured grid of every
+    platform and over random (size, nodes, ranks per node) points, against a textbook even-odd test
+    on the same polygon table (itself compared with the reference text above).  Points closer than
+    1e-6 to an edge are left to the reference's own on-edge cases (its unit-test points, replayed
+    above): there the answer depends on its epsilon rules, not on geometry."""
+    colls, sizes, nodes, ppn, _ = synthetic.tuner_axes()
+    algos, protos, nv = (ctypes.c_int * 16)(), (ctypes.c_int * 16)(), (ctypes.c_int * 16)()
+    verts = (Point * (16 * 20))()
+
+    def polygons(plat, R, N, coll):
+        n = oracle.oracle_region_polys(plat, R, N, coll, algos, protos, nv, verts, 16)
+        return [(algos[q], protos[q], [(verts[q * 20 + v].x, verts[q * 20 + v].y) for v in range(nv[q])])
+                for q in range(n)]
+
+    a, p, ch = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    rng = np.random.default_rng(5)
+    checked = skipped = decided = 0
+    for plat in range(4):
+        points = [(int(c), int(s), int(n) * int(k), int(n)) for c in colls for s in sizes for n in nodes for k in ppn]
+        for _ in range(6000):
+            n = int(rng.integers(1, 3000))
+            points.append((int(rng.choice(colls)), int(2.0 ** rng.uniform(0, 37.5)), n * int(rng.choice([1, 2, 8])), n))
+        cache = {}
+        for coll, size, R, N in points:
+            key = (coll, R // N)
+            if key not in cache:
+                cache[key] = polygons(plat, R, N, coll)
+            oracle.oracle_region_decide(plat, coll, size, R, N, ctypes.byref(a), ctypes.byref(p), ctypes.byref(ch))
+            if N <= 2 or not cache[key]:
+                assert (a.value, p.value) == (-1, -1), (plat, coll, size, R, N)
+                continue
+            at = oracle.oracle_region_log2(Point(float(size), float(R)))
+            want, nearest = _independent_region_choice(cache[key], at.x, at.y)
+            if nearest < 1e-6:
+                skipped += 1
+                continue
+            assert (a.value, p.value) == want, (plat, coll, size, R, N, nearest)
+            checked += 1
+            decided += want != (-1, -1)
+    print(f"independent rule: {checked} points compared, {decided} of them inside a region, {skipped} within 1e-6 of an edge")
+    assert checked > 15000 and decided > 8000 and skipped < checked // 50, (checked, decided, skipped)
