@@ -250,12 +250,13 @@ __device__ inline double seg_distance(pt_t x, pt_t y0, pt_t y1, double eps)
 }
 
 /*
- * Shortcuts for the two per-edge tests.  Each evaluates the quotient of `intersect` with an
- * approximate reciprocal (hardware estimate plus one Newton step: relative error below 1e-12
- * against the 1e-5 margins used here) and answers only when the exact code's answer is already
- * certain; everything else -- a quotient near one of the thresholds, a degenerate edge -- goes
- * through the exact division and square root above.  Results are therefore those of the exact
- * code; what is saved is two or three fp64 divisions and a square root per edge.
+ * Certain-answer forms of the two per-edge tests.  Each evaluates the quotient of `intersect`
+ * with an approximate reciprocal (hardware estimate plus one Newton step: relative error below
+ * 1e-12 against the 1e-5 margins used here) and says whether the exact code's answer is already
+ * certain from it.  They are straight-line code -- no branch, no division, no square root -- so
+ * the walk over a polygon's edges can overlap the arithmetic of several edges; a point for which
+ * any edge is not certain (a quotient near one of the thresholds, a degenerate edge, a foot point
+ * close to the edge) is run again through the exact code above, so results are the exact code's.
  */
 __device__ __forceinline__ double approx_rcp(double d)
 {
@@ -269,31 +270,26 @@ __device__ __forceinline__ bool clear_of(double a, double t)
 	return fabs(a - t) > 1e-5 * (1.0 + fabs(a));
 }
 
-/* intersect(x0, x1, y0, y1, eps, nullptr) == 1 */
-__device__ inline bool crosses_edge(pt_t x0, pt_t x1, pt_t y0, pt_t y1, double eps)
+/* Whether intersect(x0, x0 + dx, y0, y1, eps, nullptr) == 1; `certain` is cleared when only the
+ * exact quotient can tell. */
+__device__ __forceinline__ bool crosses_edge(pt_t x0, pt_t dx, pt_t y0, pt_t y1, double eps, bool &certain)
 {
-	const pt_t dx = vsub(x1, x0);
 	const pt_t dy = vsub(y1, y0);
 	const double d = vcross(dy, dx);
-	if (fabs(d) < eps) {
-		return false;
-	}
-	const double r = approx_rcp(d);
+	const bool parallel = fabs(d) < eps; /* the exact code answers 0 */
+	const double r = approx_rcp(parallel ? 1.0 : d);
 	const double a = (vcross(x0, dx) - vcross(y0, dx)) * r;
-	if (clear_of(a, 0.0) && clear_of(a, 1.0)) {
-		if (a < 0.0 || a > 1.0) {
-			return false; /* beyond -eps or 1 + eps */
-		}
-		const double b = (vcross(x0, dy) - vcross(y0, dy)) * r;
-		if (clear_of(b, 0.0) && clear_of(b, 1.0)) {
-			return b > 0.0 && b < 1.0;
-		}
-	}
-	return intersect(x0, x1, y0, y1, eps, nullptr) == 1;
+	const double b = (vcross(x0, dy) - vcross(y0, dy)) * r;
+	const bool a_clear = clear_of(a, 0.0) && clear_of(a, 1.0);
+	const bool b_clear = clear_of(b, 0.0) && clear_of(b, 1.0);
+	const bool a_in = a > 0.0 && a < 1.0; /* with a_clear: inside (eps, 1 - eps); else beyond -eps or 1 + eps */
+	const bool b_in = b > 0.0 && b < 1.0;
+	certain &= parallel | (a_clear & (!a_in | b_clear));
+	return !parallel && a_in && b_in;
 }
 
 /* false only when seg_distance(x, y0, y1, eps) is certainly not below eps */
-__device__ inline bool may_touch_edge(pt_t x, pt_t y0, pt_t y1, double eps)
+__device__ __forceinline__ bool may_touch_edge(pt_t x, pt_t y0, pt_t y1, double eps)
 {
 	const pt_t dy = vsub(y1, y0);
 	pt_t x1;
@@ -301,14 +297,12 @@ __device__ inline bool may_touch_edge(pt_t x, pt_t y0, pt_t y1, double eps)
 	x1.y = x.y - dy.x;
 	const pt_t dx = vsub(x1, x);
 	const double d = vcross(dy, dx);
-	if (fabs(d) < eps) {
-		return true; /* the exact code leaves the foot point unset here */
-	}
-	const double a = (vcross(x, dx) - vcross(y0, dx)) * approx_rcp(d);
+	const bool degenerate = fabs(d) < eps; /* the exact code leaves the foot point unset here */
+	const double a = (vcross(x, dx) - vcross(y0, dx)) * approx_rcp(degenerate ? 1.0 : d);
 	const pt_t s = { y0.x + a * dy.x - x.x, y0.y + a * dy.y - x.y };
 	/* the foot point computed exactly differs from this one by ~1e-12 (1 + |a|)(1 + |dy|) at most */
 	const double far = 1e-4 * (1.0 + fabs(a)) * (1.0 + fabs(dy.x) + fabs(dy.y));
-	return !(vdot(s, s) > far * far);
+	return degenerate || !(vdot(s, s) > far * far);
 }
 
 /* The bounds is_inside_region computes (:177-196): selections only, so the host can do it
@@ -339,26 +333,43 @@ __device__ __forceinline__ int inside_region(pt_t point, const pt_t *v, int n, c
 	 * box second (result -1).  A point more than 1e-6 outside the box cannot be within
 	 * 1e-10 of an edge -- edges lie inside the box, and the foot of the perpendicular may
 	 * leave the segment by at most eps times its length -- so for such a point the second
-	 * answer is known without the per-edge divisions and square roots.  Most polygons are
-	 * dismissed here. */
+	 * answer is known without looking at the edges.  Most polygons are dismissed here. */
 	const double margin = 1e-6;
 	if (point.x < min_x - margin || point.x > max_x + margin || point.y < min_y - margin ||
 	    point.y > max_y + margin) {
 		return -1;
 	}
-	for (int i = 0; i < n; i++) {
-		int k = (i + 1) % n;
-		if (may_touch_edge(point, v[i], v[k], eps) && seg_distance(point, v[i], v[k], eps) < eps) {
+	/* One branch-free walk over the edges (at most 20, one bit each) serves both of the
+	 * reference's loops, the on-edge search (:168-175) and the crossing count (:207-219); the
+	 * edges whose answer it could not be certain of are then put through the exact code. */
+	const pt_t ray = vsub(far_point, point);
+	uint32_t touch = 0, unsure = 0;
+	int crosses = 0;
+	pt_t a = v[n - 1];
+#pragma unroll 4
+	for (int i = 0; i < n; i++) { /* edge (i - 1, i): the same edges, starting from the closing one */
+		const pt_t b = v[i];
+		bool certain = true;
+		const bool crossing = crosses_edge(point, ray, a, b, eps, certain);
+		touch |= (uint32_t)may_touch_edge(point, a, b, eps) << i;
+		unsure |= (uint32_t)!certain << i;
+		crosses += (crossing & certain) ? 1 : 0;
+		a = b;
+	}
+	while (touch != 0) {
+		const int i = __ffs(touch) - 1;
+		touch &= touch - 1;
+		if (seg_distance(point, v[i == 0 ? n - 1 : i - 1], v[i], eps) < eps) {
 			return 0;
 		}
 	}
 	if (point.x < min_x || point.x > max_x || point.y < min_y || point.y > max_y) {
 		return -1;
 	}
-	int crosses = 0;
-	for (int i = 0; i < n; i++) {
-		int k = (i + 1) % n;
-		if (crosses_edge(point, far_point, v[i], v[k], eps)) {
+	while (unsure != 0) {
+		const int i = __ffs(unsure) - 1;
+		unsure &= unsure - 1;
+		if (intersect(point, far_point, v[i == 0 ? n - 1 : i - 1], v[i], eps, nullptr) == 1) {
 			crosses++;
 		}
 	}
