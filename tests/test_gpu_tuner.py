@@ -161,6 +161,25 @@ def test_region_dense_sizes_near_edges(lib, oracle, gpu):
     lib.ofi_amd_tuner_plan_destroy(plan)
 
 
+@pytest.mark.parametrize("n_sizes,n_nodes", [(1, 1), (9, 7), (8, 8), (13, 5), (43, 3), (1, 200)])
+def test_region_grid_shapes_around_the_workgroup_size(lib, oracle, gpu, n_sizes, n_nodes):
+    """Sizes x nodes per (collective, ranks per node) pair of 1, 63, 64, 65, 129 and 200 points:
+    workgroups of 64 with a short or an empty tail, one pair only, platform lists with repeats."""
+    rng = np.random.default_rng(n_sizes * 1000 + n_nodes)
+    sizes = np.sort(np.unique(np.floor(2.0 ** rng.uniform(0, 37, 4 * n_sizes)).astype(np.uint64)))[:n_sizes]
+    assert len(sizes) == n_sizes
+    nodes = np.sort(rng.choice(np.arange(1, 3000), n_nodes, replace=False)).astype(np.uint64)
+    for colls, ppn, platforms in (([2], [8], [1]), ([4, 3], [1, 8, 2], [3, 0, 0, 2, 1])):
+        colls, ppn = np.array(colls, dtype=np.int32), np.array(ppn, dtype=np.uint32)
+        plan = make_plan(lib, colls, sizes, nodes, ppn, np.array([1], dtype=np.int32))
+        want = oracle_region_grid(oracle, platforms, colls, sizes, nodes, ppn)
+        got = run_region(lib, plan, platforms, (len(platforms), len(colls), n_sizes, n_nodes, len(ppn)))
+        mism = np.argwhere((got != want).any(axis=-1))
+        assert len(mism) == 0, mism[:10]
+        assert n_nodes < 3 or (want[..., 0] >= 0).any()
+        lib.ofi_amd_tuner_plan_destroy(plan)
+
+
 def test_bad_arguments(lib, gpu):
     colls, sizes, nodes, ppn, algos = synthetic.tuner_axes()
     plan = ctypes.c_void_p()
