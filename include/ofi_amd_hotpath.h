@@ -38,15 +38,15 @@ extern "C" {
  *    (include/nccl_ofi_cuda.h:34-139).
  * ====================================================================== */
 
-/* nccl_net_ofi_gpu_init, include/nccl_ofi_rocm.h:12 */
+/* nccl_net_ofi_gpu_init, include/nccl_ofi_rocm.h:11 */
 int ofi_amd_gpu_init(void);
-/* nccl_net_ofi_get_gpu_device_for_addr, :25.  Unlike the ROCm stub of the
+/* nccl_net_ofi_get_gpu_device_for_addr, :24.  Unlike the ROCm stub of the
  * reference (src/nccl_ofi_rocm.cpp:58-76, always -1) this reports the ordinal. */
 int ofi_amd_gpu_get_device_for_addr(void *data, int *dev_id);
-/* nccl_net_ofi_gpu_flush_gpudirect_rdma_writes, :32.  -EPERM: not available,
+/* nccl_net_ofi_gpu_flush_gpudirect_rdma_writes, :31.  -EPERM: not available,
  * callers use the read-back flush (ofi_amd_flush_read) instead. */
 int ofi_amd_gpu_flush_gpudirect_rdma_writes(void);
-/* nccl_net_ofi_gpu_mem_alloc / _free / _copy_host_to_device, :39-53 */
+/* nccl_net_ofi_gpu_mem_alloc / _free / _copy_host_to_device, :38-52 */
 int ofi_amd_gpu_mem_alloc(void **ptr, size_t size);
 int ofi_amd_gpu_mem_free(void *ptr);
 int ofi_amd_gpu_mem_copy_host_to_device(void *dst, const void *src, size_t size);
@@ -55,21 +55,23 @@ int ofi_amd_gpu_get_dma_buf_fd(void *aligned_ptr, size_t aligned_size, int *fd, 
 /* nccl_net_ofi_gpu_have_dma_buf_attr / _have_gdr_support_attr, :62-63 (1/0) */
 int ofi_amd_gpu_have_dma_buf_attr(void);
 int ofi_amd_gpu_have_gdr_support_attr(void);
-/* nccl_net_ofi_gpu_set/get_current_context, include/nccl_ofi_cuda.h:50-60.
+/* nccl_net_ofi_gpu_set/get_current_context, include/nccl_ofi_cuda.h:34-39.
  * HIP has no driver contexts; the "context" is the device ordinal. */
 int ofi_amd_gpu_set_current_device(int dev_id);
 int ofi_amd_gpu_get_current_device(int *dev_id);
-/* nccl_net_ofi_gpu_get_address_range, include/nccl_ofi_cuda.h:71 */
+/* nccl_net_ofi_gpu_get_address_range, include/nccl_ofi_cuda.h:46 */
 int ofi_amd_gpu_get_address_range(void *ptr, void **base_out, size_t *size_out);
-/* nccl_net_ofi_gpu_seg_is_host, include/nccl_ofi_cuda.h:82 */
+/* nccl_net_ofi_gpu_seg_is_host, include/nccl_ofi_cuda.h:54 */
 int ofi_amd_gpu_seg_is_host(void *seg_base, int *is_host_out);
 /* Pinned host memory the GPU can address.  Stands in for
  * nccl_net_ofi_gpu_host_register_iomem / _host_unregister
- * (include/nccl_ofi_cuda.h:107-113): memory is allocated pinned rather than
- * registered after the fact. */
+ * (include/nccl_ofi_cuda.h:91-98): memory is allocated pinned rather than
+ * registered after the fact.  nccl_net_ofi_gpu_vmm_alloc / _vmm_free (:131-139) have no
+ * counterpart: they serve the GDAKI device queues, which are outside this path, and
+ * ofi_amd_gpu_mem_alloc covers what the path itself allocates. */
 int ofi_amd_gpu_host_alloc(void **ptr, size_t size);
 int ofi_amd_gpu_host_free(void *ptr);
-/* nccl_net_ofi_gpu_host_get_device_pointer, include/nccl_ofi_cuda.h:121 */
+/* nccl_net_ofi_gpu_host_get_device_pointer, include/nccl_ofi_cuda.h:106 */
 int ofi_amd_gpu_host_get_device_pointer(void **dev_ptr, void *host_ptr);
 int ofi_amd_gpu_mem_copy_device_to_host(void *dst, const void *src, size_t size);
 int ofi_amd_gpu_stream_synchronize(void *stream);
