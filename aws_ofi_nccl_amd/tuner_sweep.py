@@ -1,7 +1,7 @@
 """Tuner decision sweep: where, along the message-size axis, the tuner changes its answer.
 
 Host-side counterpart of the reference's `show-tuner-decisions` tool
-(contrib/python/ofi_nccl/tuner/cli/wrapper.py:55-230, main.py:13-69), same classes, method
+(contrib/python/ofi_nccl/tuner/cli/wrapper.py:57-229, main.py:13-69), same classes, method
 names, defaults and output columns.  The reference asks the plugin one (collective, size)
 question per ctypes call and bisects the size range recursively; here every round of the
 bisection -- for all collectives, shapes and platforms at once -- is one batched GPU query
@@ -74,7 +74,7 @@ def gpu_backend(questions):
 
 
 class Tuner:
-    """One communicator shape on one platform (wrapper.py:55-230).  Answers come from a
+    """One communicator shape on one platform (wrapper.py:57-229).  Answers come from a
     cache that `Sweep` fills in batches; `get_coll_info` on its own asks for one."""
 
     def __init__(self, nranks, nnodes, platform, backend=gpu_backend):
