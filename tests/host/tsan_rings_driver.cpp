@@ -1,5 +1,6 @@
 /*
- * Host producers and proxy threads on the GIN descriptor rings under ThreadSanitizer.
+ * Host producers and proxy threads on the GIN descriptor rings, and threads sharing one message
+ * buffer, under ThreadSanitizer.
  *
  * The rings are built here from ordinary host memory (the product puts them in pinned host memory,
  * which needs a device); push, pop and the proxy loop are the product's own
@@ -18,6 +19,7 @@
 #include <vector>
 
 #include "gin_rings.hpp"
+#include "ofi_amd_sendrecv.h"
 
 namespace {
 
@@ -213,6 +215,64 @@ void phase_pop(uint64_t per_producer)
 	free_rings(r);
 }
 
+/*
+ * The message buffer locks itself, as the reference's does (src/nccl_ofi_msgbuff.cpp): several
+ * threads draw sequence numbers from one counter and each inserts, reads back and completes its
+ * own.  A number beyond the window is refused (INVALID_IDX / UNAVAILABLE) until the older ones
+ * have completed, so the threads advance the window together.
+ */
+void phase_msgbuff(uint64_t total)
+{
+	ofi_amd_msgbuff_t *mb = nullptr;
+	if (ofi_amd_msgbuff_create(256, 10, 1, &mb) != 0) {
+		fail("msgbuff create", 0, 0);
+	}
+	std::atomic<uint64_t> next{ 0 }, refused{ 0 };
+	std::vector<uint64_t> cookies(total);
+	auto work = [&]() {
+		uint64_t not_yet = 0;
+		for (;;) {
+			const uint64_t k = next.fetch_add(1);
+			if (k >= total) {
+				break;
+			}
+			const uint16_t seq = (uint16_t)((1 + k) & 1023u);
+			int status = -1;
+			for (;;) {
+				const int rc = ofi_amd_msgbuff_insert(mb, seq, &cookies[k], OFI_AMD_MSGBUFF_REQ, &status);
+				if (rc == OFI_AMD_MSGBUFF_SUCCESS) {
+					break;
+				}
+				if (rc != OFI_AMD_MSGBUFF_INVALID_IDX || status != OFI_AMD_MSGBUFF_UNAVAILABLE) {
+					fail("msgbuff insert", k, (uint64_t)status);
+				}
+				not_yet++;
+				std::this_thread::yield();
+			}
+			void *elem = nullptr;
+			int type = -1;
+			if (ofi_amd_msgbuff_retrieve(mb, seq, &elem, &type, &status) != OFI_AMD_MSGBUFF_SUCCESS ||
+			    elem != &cookies[k] || type != OFI_AMD_MSGBUFF_REQ || status != OFI_AMD_MSGBUFF_INPROGRESS) {
+				fail("msgbuff retrieve", k, (uint64_t)status);
+			}
+			if (ofi_amd_msgbuff_complete(mb, seq, &status) != OFI_AMD_MSGBUFF_SUCCESS) {
+				fail("msgbuff complete", k, (uint64_t)status);
+			}
+		}
+		refused.fetch_add(not_yet);
+	};
+	std::vector<std::thread> threads;
+	for (int t = 0; t < 4; t++) {
+		threads.emplace_back(work);
+	}
+	for (auto &t : threads) {
+		t.join();
+	}
+	std::printf("message buffer: %llu sequence numbers on 4 threads, %llu inserts refused beyond the window\n",
+		    (unsigned long long)total, (unsigned long long)refused.load());
+	ofi_amd_msgbuff_destroy(mb);
+}
+
 } // namespace
 
 int main(int argc, char **argv)
@@ -220,6 +280,7 @@ int main(int argc, char **argv)
 	const uint64_t per_producer = argc > 1 ? std::strtoull(argv[1], nullptr, 10) : 20000;
 	phase_proxy_threads(per_producer);
 	phase_pop(per_producer);
+	phase_msgbuff(per_producer * 4);
 	std::printf("rings clean with %u producers per ring\n", kProducers);
 	return 0;
 }

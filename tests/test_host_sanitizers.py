@@ -47,14 +47,16 @@ def test_host_state_machines_clean_under_sanitizers_and_equal_to_the_oracle(driv
 
 def test_ring_push_pop_and_proxy_threads_clean_under_thread_sanitizer(tmp_path):
     """Three host producers per ring against two proxy threads, then against one popping thread per
-    ring (tests/host/tsan_rings_driver.cpp): every descriptor once, per-producer order, no data race."""
+    ring; four threads inserting, reading back and completing sequence numbers in one message buffer
+    (tests/host/tsan_rings_driver.cpp): every descriptor once, per-producer order, no data race."""
     if not shutil.which("g++"):
         pytest.skip("no host compiler")
     exe = os.path.join(tmp_path, "tsan_rings")
     subprocess.run(["g++", "-std=c++17", "-pthread", "-fsanitize=thread", "-static-libtsan", "-O1", "-g",
                     "-I", os.path.join(ROOT, "include"), "-I", CSRC,
                     os.path.join(ROOT, "tests", "host", "tsan_rings_driver.cpp"),
-                    *[os.path.join(CSRC, s) for s in ("gin_proxy.cpp", "gin_wire.cpp", "sched_host.cpp")],
+                    *[os.path.join(CSRC, s) for s in ("gin_proxy.cpp", "gin_wire.cpp", "sched_host.cpp", "sendrecv_proto.cpp",
+                                                      "wire_codec.cpp")],
                     "-o", exe], check=True)
     env = dict(os.environ, TSAN_OPTIONS="halt_on_error=1:exitcode=66")
     proc = subprocess.run([exe, "20000"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env,
@@ -63,3 +65,4 @@ def test_ring_push_pop_and_proxy_threads_clean_under_thread_sanitizer(tmp_path):
         pytest.skip("ThreadSanitizer cannot map its shadow memory on this kernel")
     assert proc.returncode == 0, proc.stdout[-4000:]
     assert "rings clean with 3 producers per ring" in proc.stdout
+    assert "message buffer: 80000 sequence numbers on 4 threads" in proc.stdout
