@@ -259,6 +259,7 @@ PROTOTYPES = {
     "ofi_amd_gpu_host_free": (ctypes.c_int, [c_vp]),
     "ofi_amd_gpu_host_get_device_pointer": (ctypes.c_int, [ctypes.POINTER(c_vp), c_vp]),
     "ofi_amd_sched_batch": (ctypes.c_int, [c_vp, c_vp, c_u64, c_u64, c_vp, c_vp, c_vp]),
+    "ofi_amd_sched_batch_noalloc": (ctypes.c_int, [c_vp, c_vp, c_u64, c_u64, c_vp, c_vp, c_vp]),
     "ofi_amd_sched_get_schedule": (ctypes.c_int, [ctypes.POINTER(SchedState), c_u64, c_u64,
                                                   ctypes.POINTER(XferInfo)]),
     "ofi_amd_bounce_scatter": (ctypes.c_int, [c_vp, c_vp, c_u64, c_vp, c_vp, c_vp, c_u32, c_vp,

@@ -44,6 +44,13 @@ int require_device();
 /* Device-visible error word (pinned host memory): kernels OR a bit into it when
  * they skip work because a documented precondition does not hold. */
 uint32_t *async_error_word();
+/* The same word if ofi_amd_gpu_init() or an earlier call has already allocated it, else
+ * NULL: for entry points that must not allocate. */
+uint32_t *async_error_word_if_ready();
+
+/* Looks up, for every GPU, the device address of the striping scratch that
+ * ofi_amd_sched_batch_noalloc uses.  Called by ofi_amd_gpu_init(). */
+int sched_noalloc_setup();
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 

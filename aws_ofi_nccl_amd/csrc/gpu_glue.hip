@@ -27,18 +27,26 @@ int require_device()
 	return status;
 }
 
+namespace {
+std::atomic<uint32_t *> g_async_error_word{nullptr};
+}
+
 uint32_t *async_error_word()
 {
 	static std::once_flag once;
-	static uint32_t *word = nullptr;
 	std::call_once(once, [] {
 		void *p = nullptr;
 		if (hipHostMalloc(&p, 64, hipHostMallocMapped) == hipSuccess) {
 			std::memset(p, 0, 64);
-			word = static_cast<uint32_t *>(p);
+			g_async_error_word.store(static_cast<uint32_t *>(p), std::memory_order_release);
 		}
 	});
-	return word;
+	return g_async_error_word.load(std::memory_order_acquire);
+}
+
+uint32_t *async_error_word_if_ready()
+{
+	return g_async_error_word.load(std::memory_order_acquire);
 }
 
 } // namespace ofi_amd
@@ -56,7 +64,10 @@ int ofi_amd_gpu_init(void)
 	int driver = -1, runtime = -1;
 	OFI_AMD_HIP_TRY(hipDriverGetVersion(&driver));
 	OFI_AMD_HIP_TRY(hipRuntimeGetVersion(&runtime));
-	return async_error_word() ? 0 : -ENOMEM;
+	if (!async_error_word()) {
+		return -ENOMEM;
+	}
+	return sched_noalloc_setup();
 }
 
 int ofi_amd_async_error_fetch(uint32_t *bits)

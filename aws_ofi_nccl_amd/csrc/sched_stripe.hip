@@ -374,6 +374,43 @@ struct workspace_t {
 std::mutex g_ws_lock;
 std::unordered_map<void *, workspace_t> g_ws_by_stream;
 
+/*
+ * The same scratch for callers that may not allocate: one array per GPU, part of the loaded
+ * code object, held until the process ends.  Layout in 32-bit words:
+ * [0, kNoAllocTiles) tile totals, [kNoAllocTiles, 2 * kNoAllocTiles) tile prefixes, then the
+ * seed word.  kNoAllocMaxBatch messages need kNoAllocTiles tiles of 2048.  In host code the
+ * array's name is only a handle for hipGetSymbolAddress; kernels get the address it returns.
+ */
+constexpr uint64_t kNoAllocMaxBatch = 1ull << 26;
+constexpr uint32_t kNoAllocTiles = (uint32_t)(kNoAllocMaxBatch / (kThreads * kPassesLarge));
+static_assert(kNoAllocTiles >= kInlineTiles, "small batches use up to kInlineTiles tiles of 512");
+static __device__ __align__(256) __attribute__((used)) uint32_t scratch[2 * kNoAllocTiles + 64];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_lock;
+uint32_t *g_scratch_ptr[kMaxDevices]; /* device address of `scratch` on each GPU, once looked up */
+
+/* Device address of the current GPU's copy of `scratch` (each GPU has its own). */
+int scratch_of_current_device(uint32_t **out)
+{
+	int dev = -1;
+	OFI_AMD_HIP_TRY(hipGetDevice(&dev));
+	if (dev < 0 || dev >= kMaxDevices) {
+		return -ENODEV;
+	}
+	std::lock_guard<std::mutex> g(g_scratch_lock);
+	if (!g_scratch_ptr[dev]) {
+		void *p = nullptr;
+		OFI_AMD_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+		if (!p) {
+			return -EIO;
+		}
+		g_scratch_ptr[dev] = static_cast<uint32_t *>(p);
+	}
+	*out = g_scratch_ptr[dev];
+	return 0;
+}
+
 uint32_t pick_passes(uint64_t n)
 {
 	return n <= kSmallBatch ? kPassesSmall : kPassesLarge;
@@ -398,6 +435,28 @@ void launch_batch(hipStream_t s, uint32_t tiles, const uint64_t *d_sizes, uint32
 }
 
 } // namespace
+
+namespace ofi_amd {
+
+int sched_noalloc_setup()
+{
+	int count = 0, before = -1;
+	OFI_AMD_HIP_TRY(hipGetDeviceCount(&count));
+	OFI_AMD_HIP_TRY(hipGetDevice(&before));
+	int rc = 0;
+	for (int dev = 0; dev < count && dev < kMaxDevices && rc == 0; dev++) {
+		uint32_t *p = nullptr;
+		if (hipSetDevice(dev) != hipSuccess) {
+			rc = -ENODEV;
+			break;
+		}
+		rc = scratch_of_current_device(&p);
+	}
+	(void)hipSetDevice(before);
+	return rc;
+}
+
+} // namespace ofi_amd
 
 using namespace ofi_amd;
 
@@ -460,6 +519,51 @@ int ofi_amd_sched_batch(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes,
 		}
 	} catch (...) {
 		return -ENOMEM;
+	}
+	OFI_AMD_HIP_TRY(hipGetLastError());
+	return 0;
+}
+
+int ofi_amd_sched_batch_noalloc(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes, uint64_t n,
+				uint64_t align, uint32_t *d_num_xfers, ofi_amd_xfer_info_t *d_xfers,
+				void *stream)
+{
+	int rc = require_device();
+	if (rc != 0) {
+		return rc;
+	}
+	if (!d_state || align == 0) {
+		return -EINVAL;
+	}
+	if (n > kNoAllocMaxBatch) {
+		return -E2BIG; /* more messages than the fixed scratch has tiles for */
+	}
+	if (n == 0) {
+		return 0;
+	}
+	if (!d_sizes || !d_num_xfers || !d_xfers) {
+		return -EINVAL;
+	}
+	uint32_t *err = async_error_word_if_ready();
+	if (!err) {
+		return -ENXIO; /* ofi_amd_gpu_init() allocates it; this call must not */
+	}
+	uint32_t *base = nullptr;
+	rc = scratch_of_current_device(&base);
+	if (rc != 0) {
+		return rc;
+	}
+	uint32_t *totals = base, *prefix = base + kNoAllocTiles, *seed0 = base + 2 * kNoAllocTiles;
+
+	const uint32_t passes = pick_passes(n);
+	const uint32_t tiles = (uint32_t)((n + kThreads * passes - 1) / (kThreads * passes));
+	hipStream_t s = as_stream(stream);
+	if (passes == kPassesSmall) {
+		launch_batch<kPassesSmall>(s, tiles, d_sizes, (uint32_t)n, d_state, align, totals, prefix, seed0,
+					   d_num_xfers, reinterpret_cast<u32x4 *>(d_xfers), err);
+	} else {
+		launch_batch<kPassesLarge>(s, tiles, d_sizes, (uint32_t)n, d_state, align, totals, prefix, seed0,
+					   d_num_xfers, reinterpret_cast<u32x4 *>(d_xfers), err);
 	}
 	OFI_AMD_HIP_TRY(hipGetLastError());
 	return 0;

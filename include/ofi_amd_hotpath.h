@@ -121,6 +121,22 @@ int ofi_amd_sched_batch(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes,
 			uint64_t align, uint32_t *d_num_xfers, ofi_amd_xfer_info_t *d_xfers,
 			void *stream);
 
+/*
+ * ofi_amd_sched_batch for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments, same results and the same kernels; the tile totals and prefixes
+ * that ofi_amd_sched_batch keeps in a per-stream allocation live here in a fixed array inside
+ * the library's device code (about 256 KiB per GPU, held until the process ends), so the call
+ * allocates and frees nothing.  n <= 2^26 messages per call, -E2BIG beyond.  Call
+ * ofi_amd_gpu_init() once beforehand (it allocates the asynchronous error word and looks up
+ * the array's address on every GPU); -ENXIO otherwise.  All calls on one GPU share that GPU's
+ * array: calls that overlap there -- different streams, or two threads -- race; order them.
+ * Nothing in the array has to start at zero: a call writes every word before it reads it.
+ */
+int ofi_amd_sched_batch_noalloc(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes, uint64_t n,
+				uint64_t align, uint32_t *d_num_xfers, ofi_amd_xfer_info_t *d_xfers,
+				void *stream);
+
 /* Host-side single-message form with the reference's semantics, for per-op
  * callers (the GIN proxy).  `state` is a host struct. Returns the stripe count. */
 int ofi_amd_sched_get_schedule(ofi_amd_sched_state_t *state, uint64_t size, uint64_t align,

@@ -1,0 +1,56 @@
+"""GPU parity of the striping entry point that allocates nothing (ofi_amd_sched_batch_noalloc)
+against ofi_amd_sched_batch and the CPU oracle: two calls in a row on the same scratch, the
+second with a smaller input, then a batch large enough for the separate scan launch."""
+import numpy as np
+import pytest
+import torch
+
+import _gpu
+import _oracle
+import aws_ofi_nccl_amd as m
+from aws_ofi_nccl_amd import synthetic
+
+pytestmark = pytest.mark.gpu
+
+
+def dev_state(rails, min_stripe, max_small, seeds):
+    st = m.SchedState(seeds[0], seeds[1], max_small, min_stripe, rails, 0)
+    return _gpu.to_dev(np.frombuffer(bytes(st), dtype=np.uint8).copy())
+
+
+def run(fn, d_state, d_sizes, n):
+    d_num = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+    d_xf = torch.full((n * 12,), -1, dtype=torch.int64, device="cuda")
+    rc = fn(d_state.data_ptr(), d_sizes.data_ptr(), n, 128, d_num.data_ptr(), d_xf.data_ptr(), _gpu.stream())
+    _gpu.sync()
+    assert rc == 0
+    return _gpu.to_host(d_num, np.uint32), _gpu.to_host(d_xf, np.uint64).reshape(n, 4, 3), \
+        d_state.cpu().numpy().tobytes()
+
+
+def test_noalloc_matches_allocating_entry_point(lib, oracle, gpu):
+    assert lib.ofi_amd_gpu_init() == 0
+    # second call smaller than the first (stale totals of the first stay in the scratch),
+    # third call beyond 4096 tiles of 2048 messages: the scan launch and the prefix half
+    for seed, n in ((11, 300007), (12, 1234), (13, (1 << 23) + 4099)):
+        sizes = synthetic.stripe_sizes(seed, n)
+        sizes[::7] = sizes[::7] % np.uint64(150)
+        d_sizes = _gpu.to_dev(sizes)
+        got = run(lib.ofi_amd_sched_batch_noalloc, dev_state(4, 131072, 64, (3, 1)), d_sizes, n)
+        ref = run(lib.ofi_amd_sched_batch, dev_state(4, 131072, 64, (3, 1)), d_sizes, n)
+        assert np.array_equal(got[0], ref[0]) and np.array_equal(got[1], ref[1]) and got[2] == ref[2], n
+        if n <= 400000:
+            want_num, want_xf, ost = _oracle.sched_batch(oracle, sizes, 4, 131072, 64, (3, 1))
+            assert np.array_equal(got[0], want_num) and np.array_equal(got[1], want_xf)
+            st = m.SchedState.from_buffer_copy(got[2])
+            assert (st.rr_small_counter, st.rr_counter) == (ost.rr_small_counter, ost.rr_counter)
+        assert _gpu.fetch_async_errors(lib) == 0
+
+
+def test_noalloc_rejects_oversized_batch(lib, gpu):
+    assert lib.ofi_amd_gpu_init() == 0
+    d = torch.zeros(16, dtype=torch.int64, device="cuda")
+    rc = lib.ofi_amd_sched_batch_noalloc(d.data_ptr(), d.data_ptr(), (1 << 26) + 1, 128, d.data_ptr(),
+                                         d.data_ptr(), _gpu.stream())
+    assert rc == -7                                            # -E2BIG, nothing launched
+    _gpu.sync()
