@@ -307,6 +307,9 @@ int oracle_region_polys(int platform, uint64_t num_ranks, uint64_t num_nodes, in
 int oracle_region_chunk_size(int platform, int coll, uint64_t size, int algo, int proto,
 			     uint64_t num_ranks, uint64_t num_nodes, uint64_t *chunk);
 uint64_t oracle_chunk_tree_ll128(uint64_t message_size, int nchannels, int log2_nnodes);
+/* calculateBestNChannelTree / calculateBestNChannelPat, :1943-1971 */
+int oracle_best_nchannel_tree(uint64_t message_size, int log2_nnodes);
+int oracle_best_nchannel_pat(uint64_t message_size, uint64_t num_nodes);
 
 /* Whole-grid loops over the functions above.  point = ((coll*n_sizes + size)*n_nodes +
  * node)*n_ppn + ppn; cost[point*n_algos*3 + a*3 + proto]; choice[point*2 + {algo, proto}];

@@ -454,7 +454,7 @@ uint64_t oracle_chunk_tree_ll128(uint64_t message_size, int nChannels, int log2_
 }
 
 /* calculateBestNChannelPat, :1943-1953 */
-static int best_nchannel_pat(uint64_t message_size, uint64_t num_nodes)
+int oracle_best_nchannel_pat(uint64_t message_size, uint64_t num_nodes)
 {
 	int best = 0;
 	if (message_size <= (num_nodes * 65536)) {
@@ -466,7 +466,7 @@ static int best_nchannel_pat(uint64_t message_size, uint64_t num_nodes)
 }
 
 /* calculateBestNChannelTree, :1955-1971 */
-static int best_nchannel_tree(uint64_t message_size, int log2_nnodes)
+int oracle_best_nchannel_tree(uint64_t message_size, int log2_nnodes)
 {
 	const int channels[] = { 16, 24, 32 };
 	int best = 0;
@@ -535,11 +535,11 @@ void oracle_region_decide_masked(int platform, int coll, uint64_t size, uint64_t
 	int log2_nnodes = log2i((int)num_nodes); /* :2340 */
 	if (platform == ORACLE_PLAT_P6 && size >= 4 * 1024 * 1024 && size <= 32 * 1024 * 1024 &&
 	    algorithm == ALGO_TREE && protocol == PROTO_LL128 && num_nodes * 8 == num_ranks) {
-		*nchannels = best_nchannel_tree(size, log2_nnodes);
+		*nchannels = oracle_best_nchannel_tree(size, log2_nnodes);
 	}
 	if (platform == ORACLE_PLAT_P6 && size <= 32 * 1024 * 1024 && algorithm == ALGO_PAT &&
 	    protocol == PROTO_SIMPLE && num_nodes == num_ranks) {
-		*nchannels = best_nchannel_pat(size, num_nodes);
+		*nchannels = oracle_best_nchannel_pat(size, num_nodes);
 	}
 }
 

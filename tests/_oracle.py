@@ -238,6 +238,8 @@ _ORACLE_PROTOS = {
     "oracle_region_chunk_size": (c_int, [c_int, c_int, c_u64, c_int, c_int, c_u64, c_u64,
                                          ctypes.POINTER(c_u64)]),
     "oracle_chunk_tree_ll128": (c_u64, [c_u64, c_int, c_int]),
+    "oracle_best_nchannel_tree": (c_int, [c_u64, c_int]),
+    "oracle_best_nchannel_pat": (c_int, [c_u64, c_u64]),
     "oracle_model_decide_v2": (None, [c_int, c_int, c_int, c_u64, c_u64, c_u64, c_int, c_int, c_int,
                                       ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
     "oracle_region_decide_masked": (None, [c_int, c_int, c_u64, c_u64, c_u64, c_u32,

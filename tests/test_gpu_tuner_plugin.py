@@ -224,3 +224,44 @@ def test_plugin_v6_chunk_size(lib, oracle, gpu, clean_env):
         assert v6.getCollInfo(ctx, 4, 4096, 1, table.ctypes.data, 7, 3, 1, ctypes.byref(nch)) == 0
         assert v6.finalize(ctx) == 0
     assert hits > 100
+
+
+def test_query_heuristic_breakpoints_by_hand(lib, gpu):
+    """The hand-derived breakpoints of the nChannels and chunk-size ladders
+    (tests/test_oracle_tuner_heuristics.py) asked of the GPU through the point-query C ABI:
+    both sides of every breakpoint, no oracle in between."""
+    import test_oracle_tuner_heuristics as h
+    qs, want = [], []
+
+    def ask(plat, kind, coll, size, ranks, nodes, algo, proto, expect):
+        qs.append(m.TunerQuery(plat, kind, coll, 1, 8, 3, algo, proto, ALL, 0, size, ranks, nodes))
+        want.append(expect)
+
+    for nodes, log2_nodes in ((8, 3), (32, 5)):
+        before = 32
+        for cut, after in h.BEST_TREE[log2_nodes]:
+            ask(h.P6, 0, h.AR, cut - 1, 8 * nodes, nodes, 0, 0, (h.TREE, h.LL128, before, 0))
+            ask(h.P6, 0, h.AR, cut, 8 * nodes, nodes, 0, 0, (h.TREE, h.LL128, after, 0))
+            before = after
+    for size, ch in ((4 * h.MIB - 1, -1), (4 * h.MIB, 32), (32 * h.MIB, 32), (32 * h.MIB + 1, -1)):
+        ask(h.P6, 0, h.AR, size, 64, 8, 0, 0, (h.TREE, h.LL128, ch, 0))
+    for nodes in (8, 16, 64):
+        for size, ch in ((nodes * 65536, 1), (nodes * 65536 + 1, 2), (nodes * 131072, 2), (nodes * 131072 + 1, 0)):
+            ask(h.P6, 0, h.AG, size, nodes, nodes, 0, 0, (h.PAT, h.SIMPLE, ch, 0))
+    ask(h.P6, 0, h.AG, 32 * h.MIB, 512, 512, 0, 0, (h.PAT, h.SIMPLE, 1, 0))
+    ask(h.P6, 0, h.AG, 32 * h.MIB + 1, 512, 512, 0, 0, (h.PAT, h.SIMPLE, -1, 0))
+    for table, coll, algo, proto, floor in ((h.PAT_LADDERS, h.AG, h.PAT, h.SIMPLE, 32768),
+                                            (h.TREE_P5EN_LADDERS, h.AR, h.TREE, h.LL128, 18000)):
+        for nodes, ladder in table.items():
+            before = floor
+            for cut, after in ladder:
+                ask(h.P5EN, 2, coll, cut - 1, nodes, nodes, algo, proto, (-1, -1, -1, before))
+                ask(h.P5EN, 2, coll, cut, nodes, nodes, algo, proto, (-1, -1, -1, after))
+                before = after
+    n = len(qs)
+    ans = (m.TunerAnswer * n)()
+    assert lib.ofi_amd_tuner_query((m.TunerQuery * n)(*qs), n, ans) == 0
+    got = [(x.algo, x.proto, x.nchannels, x.chunk_size) for x in ans]
+    bad = [i for i in range(n) if got[i] != want[i]]
+    assert not bad, [(qs[i].nbytes, qs[i].num_nodes, got[i], want[i]) for i in bad[:5]]
+    assert n > 150

@@ -286,14 +286,11 @@ def test_channel_and_chunk_heuristics(oracle):
     assert oracle.oracle_chunk_tree_ll128(8 << 20, 16, 2) == 36864
     a, p, ch = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(-1)
     # P6, 1 rank per node, PAT/Simple region: nChannels 1 up to nodes*64 KiB, 2 up to twice that, else 0
-    found = 0
+    # (every breakpoint of these ladders is pinned in test_oracle_tuner_heuristics.py)
     for size, want in [(8 * 65536, 1), (8 * 65536 + 1, 2), (8 * 131072, 2), (8 * 131072 + 1, 0)]:
         ch.value = -1
         oracle.oracle_region_decide(2, AG, size, 8, 8, ctypes.byref(a), ctypes.byref(p), ctypes.byref(ch))
-        if (a.value, p.value) == (PAT, SIMPLE):
-            assert ch.value == want
-            found += 1
-    assert found >= 1
+        assert (a.value, p.value, ch.value) == (PAT, SIMPLE, want)
     out = ctypes.c_uint64(0)
     # chunkSizeTuningTreeLL128P5en (:2211-2274): 8 nodes -> nsteps 4; 64 MiB per channel keeps 288000
     assert oracle.oracle_region_chunk_size(1, AR, 64 << 20, TREE, LL128, 8, 8, ctypes.byref(out)) == 1
