@@ -306,6 +306,7 @@ extern "C" int ofi_amd_sendrecv_loopback_run(const uint64_t *src_addrs, const ui
 		}
 
 		/* ---- both ranks test their requests: all of the round must be complete ---- */
+		uint64_t group_moved = 0;
 		for (open_msg_t &m : open) {
 			if (rc != 0) {
 				break;
@@ -322,6 +323,16 @@ extern "C" int ofi_amd_sendrecv_loopback_run(const uint64_t *src_addrs, const ui
 			}
 			const uint64_t moved = sizes[m.index] < dst_sizes[m.index] ? sizes[m.index] : dst_sizes[m.index];
 			if (rc == 0 && ssize != moved) rc = -EIO;
+			group_moved += moved;
+			if (m.sub_idx == static_cast<int32_t>(m.group_size) - 1) {
+				/* the receiver reports, per sub-receive, the bytes that landed in it */
+				uint64_t reported = 0;
+				for (uint32_t j = 0; j < m.group_size; j++) {
+					reported += static_cast<uint64_t>(static_cast<uint32_t>(rsizes[j]));
+				}
+				if (rc == 0 && reported != group_moved) rc = -EIO;
+				group_moved = 0;
+			}
 			st.payload_bytes += moved;
 			st.messages++;
 		}

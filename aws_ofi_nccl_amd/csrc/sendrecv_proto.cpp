@@ -737,7 +737,11 @@ int ofi_amd_recv_comm::match_arrivals()
 					}
 				} else {
 					sr.copy_posted = true;
-					sr.eager_len = a.e.recv_len;
+					/* the copy is cut to the receive buffer (rdma_eager_copy_req::post,
+					 * src/nccl_ofi_rdma.cpp:2738-2743) and its completion counts the
+					 * bytes copied (:2936-2937) */
+					sr.eager_len = a.e.recv_len < sr.dst_len ? a.e.recv_len
+										: static_cast<uint32_t>(sr.dst_len);
 				}
 				try {
 					copies.push_back(item);

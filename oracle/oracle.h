@@ -15,15 +15,20 @@
  *                    side by side; behaviour cases of tests/unit/mpsc_ring.cpp
  *   gin imm/meta/ack reference macros + bit-field structs compiled as-is
  *                    (oracle/_ref), encode/decode cross-checked field by field
- *   gin iputSignal   state machine (window, pin, FI_MORE flags): PARITY UNPINNED
- *                    beyond the encoders above -- the reference has no
- *                    wire-level test for it and its source does not build here
+ *   gin iputSignal   state machine (window, ACK hysteresis, pin / defer, FI_MORE): a
+ *                    known answer worked out by hand for every branch (first ACK
+ *                    request at op 4160, period 4161; window closed at 8192
+ *                    outstanding; 15 + 1 doorbell batches; pin redirect cases).  The
+ *                    reference has no wire-level test and its source does not build
+ *                    here, so nothing beyond those cases and the encoders pins it
  *   gin receiver     end values of tests/functional/rma.cpp (64 put-signals -> 64)
  *                    and rma_multiseg_signal.cpp (two slots, each its count)
  *                    under arbitrary arrival orders; hand-derived fold runs;
- *                    exactly-once in-order delivery; ACK cursor + encoding.  The
- *                    work-item / ACK streams themselves: PARITY UNPINNED (no
- *                    reference test observes them; source does not build here)
+ *                    exactly-once in-order delivery; ACK cursor + encoding; the ACK
+ *                    cadence (one ACK per retire walk, carrying the cursor after the
+ *                    walk) worked out by hand on literal wire words for in-order,
+ *                    reversed and swapped arrivals, either submission path, folded
+ *                    runs, the 14-bit cursor wrap and per-peer comm ids
  *   gin signal apply per-slot sums against a plain scatter-add (mod 2^64)
  *   region geometry  ~70 points + 4 extend_region cases of
  *                    tests/unit/region_based_tuner.cpp
@@ -33,9 +38,12 @@
  *                    rule on the same tables (another ray than the reference's), first
  *                    polygon in table order wins; points within 1e-6 of an edge, where
  *                    the reference's epsilon rules decide and not geometry, rest on the
- *                    geometry row above alone.  nChannels / chunk sizes: hand-derived
- *                    spot values only, PARITY UNPINNED beyond them (reference object
- *                    not buildable here)
+ *                    geometry row above alone.
+ *   nChannels /      every breakpoint of calculateChunkSizeTreeLL128, calculateBestNChannel
+ *   chunk sizes      Tree / Pat and the two P5en chunk ladders worked out on paper from
+ *                    the reference's thresholds, both sides of each asserted, for several
+ *                    (channels, nodes) shapes; tie-break, window ends, dispatch
+ *                    conditions; monotonicity / rung-set / grain invariants
  *   model cost       exact-rational closed forms to 1e-6 rel., linearity and
  *                    protocol-ratio identities; exact fp32 bit pattern of the
  *                    reference binary: PARITY UNPINNED (not buildable here)
@@ -45,15 +53,17 @@
  *                    full groups, sorted insert 1-7, chain decisions, wrap
  *                    regression) and the static_asserts of include/nccl_ofi_rdma.h
  *                    (8 / 64 / 512 / 560 bytes); sender numbering -> reordered
- *                    delivery -> chain drain returns send order
+ *                    delivery -> chain drain returns send order; header bytes of a
+ *                    three-batch example and the 16-bit wrap worked out by hand
  *   message buffer   the scenario of tests/unit/msgbuff.cpp:42-122 (4 in flight, 4-bit
  *                    numbers, four rounds) plus wrap, skip and out-of-order cases
  *   send/recv state  who-receives-what and reported sizes of the scenarios of
  *   machines         tests/functional/eager_multirecv.cpp (T5-T19, T21-T25) replayed with
  *                    the test as the wire; per-tag order under random interleavings
- *                    with unique tags.  The decision stream itself (which call returns
- *                    "again", eager header values beyond ctrl_msg.cpp's): PARITY UNPINNED
- *                    (no reference test observes it; the source does not build here)
+ *                    with unique tags; the sender's decision stream call by call
+ *                    (again / eager + header / writes + immediate data, schedule,
+ *                    size, state) worked out on paper for a single-receive program, a
+ *                    truncating rendezvous and a grouped receive
  */
 #ifndef ORACLE_H_
 #define ORACLE_H_

@@ -716,7 +716,11 @@ static int eager_copy_to_sub_recv(oracle_recv_comm_t *r, int req_id, rx_node_t *
 		}
 	} else {
 		req->recvs[sub_idx].has_eager_copy = 1;
-		req->recvs[sub_idx].eager_len = entry->recv_len;
+		/* rdma_eager_copy_req::post, :2738-2743, cuts the rx buffer's recv_len to the
+		 * sub-receive's length before the read; the completion (:2936-2937) counts that */
+		req->recvs[sub_idx].eager_len = entry->recv_len < req->recvs[sub_idx].dst_len
+							? entry->recv_len
+							: (uint32_t)req->recvs[sub_idx].dst_len;
 	}
 	return push_copy(r, &it);
 }

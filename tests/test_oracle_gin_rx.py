@@ -192,6 +192,160 @@ def test_ack_carries_the_cursor_and_decodes_with_reference_bitfields(oracle, ref
         assert msg == oracle.oracle_gin_ack_msg(7, rx_consumed)
 
 
+# ---- ACK emission cadence, worked out by hand from retire_completed_peer_iput_ops ----
+#
+# src/rdma/gin/nccl_ofi_gin.cpp:1622-1790: one retire call walks every op that is complete and next
+# in sequence, ORs their ack-request bits, advances rx_consumed (a 14-bit cursor) once per op, and
+# at its end (maybe_send_ack, :1608-1620) sends at most ONE standalone ACK carrying the cursor as it
+# stands then -- not one per asking op, and not the cursor at the asking op.  A retire call happens
+# only when an arriving completion makes its own op complete (:1843-1846, :1913-1921).
+# Events below are built from literal wire words: imm = ack << 28 | nseg << 24 | seq << 11 | comm << 1
+# (include/rdma/gin/nccl_ofi_gin_types.h:55-79), so seq 3 / one segment / comm 5 / ack is
+# 0x1000000 | 0x1800 | 0xA | 0x10000000 = 0x1100180A.
+
+def _imm(seq, nseg=1, ack=0, comm=5):
+    return (ack << 28) | (nseg << 24) | (seq << 11) | (comm << 1)
+
+
+def _meta(seq, nseg, ack, base, off, val, comm=5):
+    # header bit-field (:128-159): type 2 bits = 0, comm 10 bits, seq 13 bits, segment count 4 bits, ack 1 bit
+    return [(comm << 2) | (seq << 12) | (nseg << 25) | (ack << 29), base, off, val]
+
+
+class _Rx:
+    """The oracle's or the product's receiver behind one set of calls."""
+
+    def __init__(self, which, oracle, lib):
+        self.product = which == "product"
+        if self.product:
+            import aws_ofi_nccl_amd as m
+            self.lib, self.pre, self.Ack, self.Work = lib, "ofi_amd_gin_rx_", m.GinAck, m.GinSignalWork
+            self.api = (lib.ofi_amd_gin_rx_write_completion, lib.ofi_amd_gin_rx_metadata)
+        else:
+            self.lib, self.pre, self.Ack, self.Work = oracle, "oracle_gin_rx_", GinAck, GinSignalWork
+            self.api = oracle_api(oracle)
+
+    def call(self, name):
+        return getattr(self.lib, self.pre + name)
+
+    def create(self, comm_ids):
+        ids = (c_u32 * len(comm_ids))(*comm_ids)
+        if self.product:
+            rx = ctypes.c_void_p()
+            assert self.lib.ofi_amd_gin_rx_create(len(comm_ids), ids, ctypes.byref(rx)) == 0
+            return rx
+        return self.lib.oracle_gin_rx_create(len(comm_ids), ids)
+
+
+@pytest.fixture(params=["oracle", "product"])
+def rxside(request, oracle, lib):
+    return _Rx(request.param, oracle, lib)
+
+
+def _run_events(side, events, comm_ids=(7,), peer=0):
+    rx = side.create(list(comm_ids))
+    acks_after = []
+    buf = (side.Ack * 16)()
+    for ev in events:
+        G.feed(side.api, rx, peer, [ev])
+        n = side.call("take_acks")(rx, buf, 16)
+        acks_after.append([(buf[i].peer, buf[i].rx_consumed, buf[i].msg) for i in range(n)])
+    work = G.take_all(side.call("take_work"), rx, side.Work)
+    cons, nxt = c_u32(), c_u32()
+    side.call("cursors")(rx, peer, ctypes.byref(cons), ctypes.byref(nxt))
+    side.call("destroy")(rx)
+    return acks_after, work, cons.value, nxt.value
+
+
+def _ack_word(comm, rx_consumed):
+    # gin_ack_msg_t (:170-181): type 2 bits = 1, comm 10 bits, rx_consumed 14 bits
+    return 1 | (comm << 2) | (rx_consumed << 12)
+
+
+def test_hand_built_wire_words_agree_with_the_pinned_encoders(oracle):
+    assert _imm(3, 1, 1) == 0x1100180A == oracle.oracle_gin_imm(5, 3, 1, 1)
+    assert _meta(3, 2, 1, 0, 0, 0)[0] == oracle.oracle_gin_meta_header(5, 3, 2, 1)
+    assert _ack_word(7, 6) == 0x601D == oracle.oracle_gin_ack_msg(7, 6)
+
+
+def test_ack_cadence_in_order_one_ack_per_asking_op(rxside):
+    # six one-segment puts, seq 1 and 4 ask: each arrival retires exactly its own op
+    ev = [(k, "w", _imm(k, ack=int(k in (1, 4)))) for k in range(6)]
+    acks, work, cons, nxt = _run_events(rxside, ev)
+    assert acks == [[], [(0, 2, _ack_word(7, 2))], [], [], [(0, 5, _ack_word(7, 5))], []]
+    assert work == [] and (cons, nxt) == (6, 6)
+
+
+def test_ack_cadence_reversed_arrival_one_ack_for_the_whole_walk(rxside):
+    # same ops, arriving 5, 4, 3, 2, 1, 0: nothing can retire before seq 0 is there; that arrival
+    # walks all six in one call -> a single ACK with the cursor after the walk (6, not 2 or 5)
+    ev = [(k, "w", _imm(k, ack=int(k in (1, 4)))) for k in reversed(range(6))]
+    acks, _work, cons, _nxt = _run_events(rxside, ev)
+    assert acks == [[], [], [], [], [], [(0, 6, _ack_word(7, 6))]]
+    assert cons == 6
+
+
+def test_ack_cadence_pairwise_swapped(rxside):
+    # arrival 1, 0, 3, 2, 5, 4; asks on 1 and 4.  Walks: {0, 1} -> ACK 2; {2, 3} -> none; {4, 5} -> ACK 6
+    ev = [(k, "w", _imm(k, ack=int(k in (1, 4)))) for k in (1, 0, 3, 2, 5, 4)]
+    acks, _work, _cons, _nxt = _run_events(rxside, ev)
+    assert acks == [[], [(0, 2, _ack_word(7, 2))], [], [], [], [(0, 6, _ack_word(7, 6))]]
+
+
+def test_ack_cursor_is_the_end_of_the_walk_not_the_asking_op(rxside):
+    # arrival 2, 1, 0 with only seq 0 asking: one ACK, cursor 3
+    ev = [(k, "w", _imm(k, ack=int(k == 0))) for k in (2, 1, 0)]
+    acks, _work, _cons, _nxt = _run_events(rxside, ev)
+    assert acks == [[], [], [(0, 3, _ack_word(7, 3))]]
+
+
+def test_ack_request_is_honoured_from_either_submission_path(rxside):
+    """:1817-1828 and :1893-1900: the bit may come with the write's immediate data or with the
+    metadata header; the op asks if either did.  Two-segment put-signals (one write + metadata)."""
+    base = SIG_BASE
+    for imm_ack, meta_ack in ((1, 0), (0, 1), (1, 1), (0, 0)):
+        for order in ("wm", "mw"):
+            w = (0, "w", _imm(0, nseg=2, ack=imm_ack))
+            mm = (0, "m", _meta(0, 2, meta_ack, base, 8, 1))
+            ev = [w, mm] if order == "wm" else [mm, w]
+            acks, work, cons, _nxt = _run_events(rxside, ev)
+            want = [(0, 1, _ack_word(7, 1))] if (imm_ack or meta_ack) else []
+            assert acks == [[], want], (imm_ack, meta_ack, order)
+            assert [(x[1], x[2], x[4], x[5]) for x in work] == [(8, 1, 0, 1)] and cons == 1
+
+
+def test_ack_with_a_folded_run(rxside):
+    # three put-signals to one slot arrive last-first, the middle one asks: one work item of run
+    # length 3 (gate = seq 2) and one ACK with cursor 3
+    ev = []
+    for k in (2, 1, 0):
+        ev.append((k, "w", _imm(k, nseg=2, ack=int(k == 1))))
+        ev.append((k, "m", _meta(k, 2, 0, SIG_BASE, 16, 1)))
+    acks, work, cons, nxt = _run_events(rxside, ev)
+    assert acks[:-1] == [[]] * 5 and acks[-1] == [(0, 3, _ack_word(7, 3))]
+    assert work == [(SIG_BASE, 16, 3, 0, 2, 3)] and (cons, nxt) == (3, 3)
+
+
+def test_ack_cursor_is_fourteen_bits_while_sequence_numbers_are_thirteen(rxside):
+    """rx_consumed counts modulo 16,384 (gin_cursor_inc, include/rdma/gin/nccl_ofi_gin.h:155-158),
+    sequence numbers modulo 8,192 (GIN_IMM_SEQ_MASK).  16,386 in-order puts; op 16,383 asks: the
+    cursor it reports is (16,383 + 1) mod 16,384 = 0; op 16,385 asks: 2.  Op k travels as seq k mod 8,192."""
+    total = 16386
+    ev = [(k, "w", _imm(k & 0x1FFF, ack=int(k in (8191, 16383, 16385)))) for k in range(total)]
+    acks, _work, cons, nxt = _run_events(rxside, ev)
+    said = [(k, a) for k, a in enumerate(acks) if a]
+    assert said == [(8191, [(0, 8192, _ack_word(7, 8192))]), (16383, [(0, 0, _ack_word(7, 0))]),
+                    (16385, [(0, 2, _ack_word(7, 2))])]
+    assert (cons, nxt) == (2, 2)
+
+
+def test_ack_names_the_comm_id_the_peer_expects(rxside):
+    # two peers with their own comm ids; completions of peer 1 only: its ACK carries id 33
+    ev = [(0, "w", _imm(0, ack=1))]
+    acks, _w, _c, _n = _run_events(rxside, ev, comm_ids=(21, 33), peer=1)
+    assert acks == [[(1, 1, _ack_word(33, 1))]]
+
+
 def test_closed_loop_never_stalls(oracle):
     """Sender and receiver wired back to back for four trips round the 13-bit sequence
     space: the ACKs the receiver produces keep the sender's window open."""

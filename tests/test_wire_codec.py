@@ -208,6 +208,62 @@ def test_wrap_collision_regression(side):
     side.eager_rxq_destroy(q)
 
 
+# ---- sender numbering by hand ----
+
+def test_sender_numbering_three_batches_by_hand(side):
+    """send(), src/nccl_ofi_rdma.cpp:5783-5806, with the batch close of :5594-5598 / :5863-5866,
+    from a fresh send comm (all four fields zero, :6324-6326).  Worked out on paper:
+      batch 1, three eager sends (tags 10, 11, -2): the first finds eager_offset_next == 0 and takes
+        eager_seq 0; offsets 0, 1, 2; prev_batch_count 0 (nothing before)
+      msg_seq_num advances: prev_eager_batch_count = 3, eager_offset_next = 0
+      msg_seq_num advances again with no eager send in between (rendezvous traffic): no change
+      batch 2, one send (tag 20): eager_seq 1, offset 0, prev_batch_count 3
+      advance: prev = 1
+      batch 3, two sends (tags 30, 31): eager_seq 2, offsets 0 and 1; BOTH carry prev_batch_count 1
+        (the field is copied from the comm on every send, the receiver only reads it at offset 0)
+    Header bytes, little-endian {u8 offset, u8 prev, u16 seq, i32 tag}
+    (include/nccl_ofi_rdma.h:217-226)."""
+    tx = side.mod.EagerTx()
+    side.eager_tx_init(ctypes.byref(tx))
+
+    def send(tag):
+        h = side.mod.EagerHdr()
+        side.eager_tx_assign(ctypes.byref(tx), tag, ctypes.byref(h))
+        return bytes(h)
+
+    assert send(10) == bytes([0, 0, 0, 0, 10, 0, 0, 0])
+    assert send(11) == bytes([1, 0, 0, 0, 11, 0, 0, 0])
+    assert send(-2) == bytes([2, 0, 0, 0, 0xFE, 0xFF, 0xFF, 0xFF])
+    side.eager_tx_advance(ctypes.byref(tx))
+    assert (tx.eager_seq_next, tx.cur_eager_seq, tx.eager_offset_next, tx.prev_eager_batch_count) == (1, 0, 0, 3)
+    side.eager_tx_advance(ctypes.byref(tx))
+    assert (tx.eager_seq_next, tx.cur_eager_seq, tx.eager_offset_next, tx.prev_eager_batch_count) == (1, 0, 0, 3)
+    assert send(20) == bytes([0, 3, 1, 0, 20, 0, 0, 0])
+    side.eager_tx_advance(ctypes.byref(tx))
+    assert send(30) == bytes([0, 1, 2, 0, 30, 0, 0, 0])
+    assert send(31) == bytes([1, 1, 2, 0, 31, 0, 0, 0])
+    assert (tx.eager_seq_next, tx.cur_eager_seq, tx.eager_offset_next, tx.prev_eager_batch_count) == (3, 2, 2, 1)
+    # a batch is only closed by an advance: without one the next send continues batch 3
+    assert send(32) == bytes([2, 1, 2, 0, 32, 0, 0, 0])
+
+
+def test_sender_numbering_wraps_at_sixteen_bits(side):
+    """eager_seq_next is a uint16 that wraps naturally (:5792): batch number 65,536 is numbered
+    0 again, batch 65,537 (two sends) announces the single send of the batch before it."""
+    tx = side.mod.EagerTx()
+    side.eager_tx_init(ctypes.byref(tx))
+    h = side.mod.EagerHdr()
+    for batch in range(65536):
+        side.eager_tx_assign(ctypes.byref(tx), 7, ctypes.byref(h))
+        assert h.eager_seq == batch
+        side.eager_tx_advance(ctypes.byref(tx))
+    assert bytes(h) == bytes([0, 1, 0xFF, 0xFF, 7, 0, 0, 0])       # batch 65,535
+    side.eager_tx_assign(ctypes.byref(tx), 8, ctypes.byref(h))
+    assert bytes(h) == bytes([0, 1, 0, 0, 8, 0, 0, 0])
+    side.eager_tx_assign(ctypes.byref(tx), 9, ctypes.byref(h))
+    assert bytes(h) == bytes([1, 1, 0, 0, 9, 0, 0, 0])
+
+
 # ---- sender numbering -> network reordering -> receiver chain ----
 
 @pytest.mark.parametrize("seed", [1, 2, 3])
