@@ -30,10 +30,14 @@ inline int errno_of(hipError_t e)
 	}
 }
 
+/* A failed call is reported through the return value only: the runtime's per-thread
+ * "last error" is cleared so that it does not surface in an unrelated later call of the
+ * application (hipGetLastError / hipPeekAtLastError users). */
 #define OFI_AMD_HIP_TRY(expr)                                                           \
 	do {                                                                            \
 		hipError_t e_ = (expr);                                                 \
 		if (e_ != hipSuccess) {                                                 \
+			(void)hipGetLastError();                                        \
 			return ::ofi_amd::errno_of(e_);                                 \
 		}                                                                       \
 	} while (0)

@@ -222,6 +222,52 @@ def test_gpu_glue(lib, gpu):
     assert lib.ofi_amd_gpu_get_device_for_addr(host.ctypes.data, ctypes.byref(dev)) < 0 and dev.value == -1
 
 
+def test_dma_buf_export_of_device_memory(lib, gpu):
+    """nccl_net_ofi_gpu_get_dma_buf_fd (src/nccl_ofi_rocm.cpp:129-139), called as the reference
+    calls it for its flush buffer (src/nccl_ofi_rdma.cpp:3842-3845: a page-aligned address, one
+    system page) and for a whole registration: a dma-buf file descriptor and offset 0.  Where the
+    device cannot export (have_dma_buf_attr 0) the call fails with a negative errno instead."""
+    import os
+    page = os.sysconf("SC_PAGE_SIZE")
+    p = ctypes.c_void_p()
+    assert lib.ofi_amd_gpu_mem_alloc(ctypes.byref(p), 4 << 20) == 0 and p.value % page == 0
+    have = lib.ofi_amd_gpu_have_dma_buf_attr()
+    assert have in (0, 1)
+    for addr, size in ((p.value, page), (p.value + 16 * page, 1 << 20), (p.value, 4 << 20)):
+        fd, off = ctypes.c_int(-1), ctypes.c_size_t(99)
+        rc = lib.ofi_amd_gpu_get_dma_buf_fd(ctypes.c_void_p(addr), size, ctypes.byref(fd), ctypes.byref(off))
+        if not have:
+            assert rc < 0
+            continue
+        assert rc == 0 and fd.value >= 0 and off.value == 0
+        st = os.fstat(fd.value)                                  # a live descriptor of this process
+        assert st.st_ino > 0
+        link = os.readlink("/proc/self/fd/%d" % fd.value)
+        assert "dmabuf" in link, link                            # an anonymous dma-buf inode
+        try:
+            end = os.lseek(fd.value, 0, os.SEEK_END)             # dma-buf files report their size
+            assert end >= size, (end, size)
+        except OSError:
+            pass
+        os.close(fd.value)
+        with pytest.raises(OSError):
+            os.fstat(fd.value)                                   # the caller owns the descriptor: closed means gone
+    # the exported memory is untouched and still usable
+    data = np.arange(256, dtype=np.uint8)
+    back = np.zeros(256, dtype=np.uint8)
+    assert lib.ofi_amd_gpu_mem_copy_host_to_device(p, data.ctypes.data, 256) == 0
+    assert lib.ofi_amd_gpu_mem_copy_device_to_host(back.ctypes.data, p, 256) == 0 and np.array_equal(back, data)
+    # a pointer the runtime does not know as device memory, and missing outputs
+    host = np.zeros(2 * page, dtype=np.uint8)
+    aligned = (host.ctypes.data + page - 1) // page * page
+    fd, off = ctypes.c_int(-1), ctypes.c_size_t(0)
+    assert lib.ofi_amd_gpu_get_dma_buf_fd(ctypes.c_void_p(aligned), page, ctypes.byref(fd), ctypes.byref(off)) < 0
+    assert lib.ofi_amd_gpu_get_dma_buf_fd(p, page, None, ctypes.byref(off)) == -22
+    assert lib.ofi_amd_gpu_get_dma_buf_fd(p, page, ctypes.byref(fd), None) == -22
+    assert lib.ofi_amd_gpu_mem_free(p) == 0
+    assert _gpu.fetch_async_errors(lib) == 0
+
+
 @pytest.mark.parametrize("sentinel", [0x00000000FFFFFFFF, 0xDEADBEEFDEADBEEF])
 def test_sentinel_flush_reaches_every_rail_slot(lib, oracle, gpu, sentinel):
     """GPU flush buffer -> one 64-byte pinned host slot per rail; complete when each slot's

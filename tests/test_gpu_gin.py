@@ -249,6 +249,20 @@ def test_configured_shape_checksum(lib, oracle, gpu):
     lib.ofi_amd_gin_rings_destroy(rings)
 
 
+def test_configured_shape_full_size(lib, oracle, gpu):
+    """The configured run in full: 256 contexts x 1,000,000 put ops (a put-signal every 64th)
+    into 4096-entry rings drained by one proxy thread; the order-sensitive checksum of all
+    256,000,000 descriptors against the oracle's."""
+    nctx, cap, ops = 256, 4096, 1_000_000
+    rings = make_rings(lib, nctx, cap)
+    rc, stats, _, _ = produce_and_drain(lib, rings, nctx, ops, mode=0)
+    assert rc == 0 and lib.ofi_amd_gin_producer_status(rings) == 0
+    assert stats.descriptors == nctx * ops and stats.signals == nctx * (ops // 64)
+    assert stats.checksum == oracle.oracle_gin_stream_checksum(SEED, nctx, ops, 1, 64, 1, 1, 0, 4, 131072,
+                                                                64, 1, None)
+    lib.ofi_amd_gin_rings_destroy(rings)
+
+
 def test_producer_gives_up_when_nobody_drains(lib, gpu):
     """Failure path forced from the host: more ops than slots, no consumer, a tiny spin limit.
     Every wave reaches its exit, the kernel ends, the status word reports the timeout."""

@@ -4,7 +4,8 @@ copy, rendezvous as striped device copies.  Checked byte for byte against the so
 
 Sizes: the ten (send, receive) pairs of the reference's tests/functional/
 nccl_message_transfer.cpp:44-56 with NCCL_NET_MAX_REQUESTS = 32 requests each, and the
-powers of two of the configured sweep (8 B up; 64 MiB here) with 64 in flight."""
+powers of two of the configured sweep, 8 B to 1 GiB: 64 in flight up to 1 MiB, then as many as
+128 MiB hold, and 4 / 4 / 2 / 2 messages of 128 MiB / 256 MiB / 512 MiB / 1 GiB."""
 import ctypes
 
 import numpy as np
@@ -76,6 +77,35 @@ def test_power_of_two_sweep_sixty_four_in_flight(lib, gpu):
         stripes = 1 if size <= 131072 else (2 if size <= 262144 else 4)
         if size + 8 > 8192:
             assert st.rdma_writes == count * stripes
+
+
+@pytest.mark.parametrize("size,count", [(128 << 20, 4), (256 << 20, 4), (512 << 20, 2), (1 << 30, 2)])
+def test_power_of_two_sweep_large_messages(lib, gpu, size, count):
+    """The top of the configured sweep.  Payloads are random 16-bit words (bf16 bit patterns)
+    generated on the device; every received byte, and the guard bytes behind each receive
+    buffer, are compared on the device."""
+    gen = torch.Generator(device="cuda").manual_seed(size + count)
+    srcs = [torch.randint(-32768, 32768, (size // 2,), dtype=torch.int16, device="cuda", generator=gen)
+            for _ in range(count)]
+    dsts = [torch.full((size // 2 + 32,), 0x4DCD, dtype=torch.int16, device="cuda") for _ in range(count)]
+    pool = torch.zeros(64 * RX_STRIDE, dtype=torch.uint8, device="cuda")
+    a_src = np.array([t.data_ptr() for t in srcs], dtype=np.uint64)
+    a_dst = np.array([t.data_ptr() for t in dsts], dtype=np.uint64)
+    a_size = np.array([size] * count, dtype=np.uint64)
+    stats = m.SendrecvLoopbackStats()
+    torch.cuda.synchronize()
+    rc = lib.ofi_amd_sendrecv_loopback_run(a_src.ctypes.data, a_dst.ctypes.data, a_size.ctypes.data,
+                                           a_size.ctypes.data, None, count, 64, 4, 1, pool.data_ptr(),
+                                           pool.numel(), 0, _gpu.stream(), ctypes.byref(stats))
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    for i in range(count):
+        assert torch.equal(dsts[i][:size // 2], srcs[i]), (i, size)
+        assert bool((dsts[i][size // 2:] == 0x4DCD).all()), (i, "wrote past the receive buffer")
+    assert stats.messages == count and stats.payload_bytes == size * count
+    assert stats.write_messages == count and stats.rdma_writes == 4 * count and stats.eager_messages == 0
+    # every stripe is cut into 256 KiB table entries: size / 4 rails / 256 KiB each
+    assert stats.copy_entries == count * 4 * (size // 4 // (256 << 10))
 
 
 def test_receiver_first_sends_everything_as_writes(lib, gpu):

@@ -264,4 +264,4 @@ def test_query_heuristic_breakpoints_by_hand(lib, gpu):
     got = [(x.algo, x.proto, x.nchannels, x.chunk_size) for x in ans]
     bad = [i for i in range(n) if got[i] != want[i]]
     assert not bad, [(qs[i].nbytes, qs[i].num_nodes, got[i], want[i]) for i in bad[:5]]
-    assert n > 150
+    assert n >= 150
