@@ -267,7 +267,7 @@ PROTOTYPES = {
     "ofi_amd_eager_copy_batch": (ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_u32, c_vp, c_vp,
                                                 c_vp]),
     "ofi_amd_copy_table": (ctypes.c_int, [c_vp, c_vp, c_vp, c_u32, c_vp]),
-    "ofi_amd_gin_loopback_run": (ctypes.c_int, [c_vp, c_u64, c_vp, c_vp, ctypes.POINTER(GinSignalRegion), c_u32,
+    "ofi_amd_gin_loopback_run": (ctypes.c_int, [c_vp, c_u64, c_vp, c_vp, c_u32, ctypes.POINTER(GinSignalRegion), c_u32,
                                                 c_u32, c_u32, c_u32, c_vp, ctypes.POINTER(GinLoopbackStats)]),
     "ofi_amd_flush_buffer_fill": (ctypes.c_int, [c_vp, c_u64, c_vp]),
     "ofi_amd_flush_post": (ctypes.c_int, [c_vp, c_vp, c_u32, c_vp]),
@@ -292,15 +292,15 @@ PROTOTYPES = {
     "ofi_amd_gin_ring_pop": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(GinDesc)]),
     "ofi_amd_gin_comm_init": (ctypes.c_int, [ctypes.POINTER(GinComm), c_u32, c_u32, c_u64, c_u64,
                                              c_u32]),
-    "ofi_amd_gin_iput_signal": (ctypes.c_int, [ctypes.POINTER(GinComm), ctypes.POINTER(GinMr),
+    "ofi_amd_gin_iput_signal": (ctypes.c_int, [ctypes.POINTER(GinComm), ctypes.POINTER(GinMr), c_u32,
                                                ctypes.POINTER(GinDesc), ctypes.POINTER(GinWire)]),
     "ofi_amd_gin_apply_ack": (None, [ctypes.POINTER(GinComm), c_u32]),
     "ofi_amd_gin_imm": (c_u32, [c_u32, c_u32, c_u32, c_u32]),
     "ofi_amd_gin_meta_header": (c_u64, [c_u32, c_u32, c_u32, c_u32]),
     "ofi_amd_gin_ack_msg": (c_u64, [c_u32, c_u32]),
-    "ofi_amd_gin_proxy_drain": (ctypes.c_int, [c_vp, c_u64, ctypes.c_int, c_vp, c_vp, c_vp, c_vp,
+    "ofi_amd_gin_proxy_drain": (ctypes.c_int, [c_vp, c_u64, ctypes.c_int, c_vp, c_vp, c_vp, c_u32, c_vp,
                                                c_u32, ctypes.POINTER(GinProxyStats)]),
-    "ofi_amd_gin_proxy_drain_mt": (ctypes.c_int, [c_vp, c_u64, ctypes.c_int, c_vp, c_vp, c_vp, c_vp,
+    "ofi_amd_gin_proxy_drain_mt": (ctypes.c_int, [c_vp, c_u64, ctypes.c_int, c_vp, c_vp, c_vp, c_u32, c_vp,
                                                   c_u32, c_u32, ctypes.POINTER(GinProxyStats)]),
     "ofi_amd_gin_rx_create": (ctypes.c_int, [c_u32, ctypes.POINTER(c_u32), ctypes.POINTER(c_vp)]),
     "ofi_amd_gin_rx_destroy": (ctypes.c_int, [c_vp]),

@@ -83,12 +83,12 @@ struct lcg_t {
 } // namespace
 
 extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per_context,
-					ofi_amd_gin_comm_t *comms, const ofi_amd_gin_mr_t *mrs,
+					ofi_amd_gin_comm_t *comms, const ofi_amd_gin_mr_t *mrs, uint32_t n_mrs,
 					const ofi_amd_gin_signal_region_t *regions, uint32_t n_regions,
 					uint32_t reorder_window, uint32_t batch_writes, uint32_t timeout_ms,
 					void *stream, ofi_amd_gin_loopback_stats_t *stats)
 {
-	if (!r || !comms || !mrs || !regions || n_regions == 0 || batch_writes == 0 ||
+	if (!r || !comms || !mrs || n_mrs == 0 || !regions || n_regions == 0 || batch_writes == 0 ||
 	    batch_writes > (1u << 24) || reorder_window > 2048) {
 		return -EINVAL;
 	}
@@ -243,12 +243,12 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 					break;
 				}
 				ofi_amd_gin_wire_t wire;
-				rc = ofi_amd_gin_iput_signal(&comms[c], mrs, &d, &wire);
+				rc = ofi_amd_gin_iput_signal(&comms[c], mrs, n_mrs, &d, &wire);
 				if (rc == -EAGAIN) {
 					/* window closed: let everything in flight arrive, which brings the ACKs */
 					rc = deliver_some(0);
 					if (rc == 0) {
-						rc = ofi_amd_gin_iput_signal(&comms[c], mrs, &d, &wire);
+						rc = ofi_amd_gin_iput_signal(&comms[c], mrs, n_mrs, &d, &wire);
 					}
 				}
 				if (rc != 0) {

@@ -85,7 +85,7 @@ int ofi_amd_gin_ring_pop(ofi_amd_gin_rings_t *r, uint32_t context, ofi_amd_gin_d
 /* One proxy thread's share: contexts [c_begin, c_end). */
 static int drain_contexts(ofi_amd_gin_rings_t *r, uint32_t c_begin, uint32_t c_end,
 			  uint64_t ops_per_context, int mode, ofi_amd_gin_desc_t *out_desc,
-			  ofi_amd_gin_comm_t *comms, const ofi_amd_gin_mr_t *mrs,
+			  ofi_amd_gin_comm_t *comms, const ofi_amd_gin_mr_t *mrs, uint32_t n_mrs,
 			  ofi_amd_gin_wire_t *out_wire, uint32_t timeout_ms,
 			  ofi_amd_gin_proxy_stats_t *stats)
 {
@@ -135,19 +135,21 @@ static int drain_contexts(ofi_amd_gin_rings_t *r, uint32_t c_begin, uint32_t c_e
 				st.signals += d->signal_op != 0;
 				if (mode == 1) {
 					out_desc[(size_t)c * ops_per_context + i] = *d;
-				} else if (mode == 2) {
-					ofi_amd_gin_wire_t wire;
-					ofi_amd_gin_desc_t copy = *d; /* the slot is recycled below */
-					int e = ofi_amd_gin_iput_signal(&comms[c], mrs, &copy, &wire);
+				} else if (mode >= 2) {
+					/* the slot is handed back only after this burst, so the record is
+					 * read in place; the wire record goes straight to its output slot */
+					ofi_amd_gin_wire_t local;
+					ofi_amd_gin_wire_t *wire =
+						out_wire ? &out_wire[(size_t)c * ops_per_context + i] : &local;
+					int e = ofi_amd_gin_iput_signal(&comms[c], mrs, n_mrs, d, wire);
 					if (e != 0) {
 						rc = e;
 						break;
 					}
-					st.writes += wire.num_writes;
-					h = fold_words(h, reinterpret_cast<const uint64_t *>(&wire),
-						       (int)(sizeof(wire) / 8));
-					if (out_wire) {
-						out_wire[(size_t)c * ops_per_context + i] = wire;
+					st.writes += wire->num_writes;
+					if (mode == 3) {
+						h = fold_words(h, reinterpret_cast<const uint64_t *>(wire),
+							       (int)(sizeof(*wire) / 8));
 					}
 				}
 				pos++;
@@ -198,10 +200,11 @@ static int drain_contexts(ofi_amd_gin_rings_t *r, uint32_t c_begin, uint32_t c_e
 
 int ofi_amd_gin_proxy_drain_mt(ofi_amd_gin_rings_t *r, uint64_t ops_per_context, int mode,
 			       ofi_amd_gin_desc_t *out_desc, ofi_amd_gin_comm_t *comms,
-			       const ofi_amd_gin_mr_t *mrs, ofi_amd_gin_wire_t *out_wire,
+			       const ofi_amd_gin_mr_t *mrs, uint32_t n_mrs, ofi_amd_gin_wire_t *out_wire,
 			       uint32_t timeout_ms, uint32_t n_threads, ofi_amd_gin_proxy_stats_t *stats)
 {
-	if (!r || mode < 0 || mode > 2 || (mode == 1 && !out_desc) || (mode == 2 && (!comms || !mrs)) ||
+	if (!r || mode < 0 || mode > 3 || (mode == 1 && !out_desc) ||
+	    (mode >= 2 && (!comms || !mrs || n_mrs == 0)) ||
 	    n_threads < 1 || n_threads > 64) {
 		return -EINVAL;
 	}
@@ -214,7 +217,7 @@ int ofi_amd_gin_proxy_drain_mt(ofi_amd_gin_rings_t *r, uint64_t ops_per_context,
 		/* contiguous ranges of contexts, sizes differing by at most one */
 		const uint32_t lo = (uint32_t)((uint64_t)nctx * w / workers);
 		const uint32_t hi = (uint32_t)((uint64_t)nctx * (w + 1) / workers);
-		rcs[w] = drain_contexts(r, lo, hi, ops_per_context, mode, out_desc, comms, mrs, out_wire,
+		rcs[w] = drain_contexts(r, lo, hi, ops_per_context, mode, out_desc, comms, mrs, n_mrs, out_wire,
 					timeout_ms, &part[w]);
 	};
 	try {
@@ -251,10 +254,10 @@ int ofi_amd_gin_proxy_drain_mt(ofi_amd_gin_rings_t *r, uint64_t ops_per_context,
 
 int ofi_amd_gin_proxy_drain(ofi_amd_gin_rings_t *r, uint64_t ops_per_context, int mode,
 			    ofi_amd_gin_desc_t *out_desc, ofi_amd_gin_comm_t *comms,
-			    const ofi_amd_gin_mr_t *mrs, ofi_amd_gin_wire_t *out_wire,
+			    const ofi_amd_gin_mr_t *mrs, uint32_t n_mrs, ofi_amd_gin_wire_t *out_wire,
 			    uint32_t timeout_ms, ofi_amd_gin_proxy_stats_t *stats)
 {
-	return ofi_amd_gin_proxy_drain_mt(r, ops_per_context, mode, out_desc, comms, mrs, out_wire,
+	return ofi_amd_gin_proxy_drain_mt(r, ops_per_context, mode, out_desc, comms, mrs, n_mrs, out_wire,
 					  timeout_ms, 1, stats);
 }
 

@@ -372,8 +372,13 @@ def bench_gin(lib, oracle, torch, np, args):
     nctx, cap, ops = 256, 4096, args.gin_ops
     out = {"contexts": nctx, "ring_capacity": cap, "ops_per_context": ops}
     # NCCL runs up to NCCL_GIN_MAX_CONNECTIONS = 4 GIN proxy threads (nccl/net.h:38)
+    # mode 2 is the product's work per descriptor (pop, derive the wire record); mode 3 is the same
+    # with every wire record folded into the checksum: the parity check of the derived stream at the
+    # full size, reported beside the timed figure and never as it
     for mode, threads, key in ((0, 1, "drain"), (0, 4, "drain_4_proxy_threads"), (2, 1, "drain_and_derive_wire"),
-                               (2, 4, "drain_and_derive_wire_4_proxy_threads")):
+                               (2, 4, "drain_and_derive_wire_4_proxy_threads"),
+                               (3, 1, "drain_derive_and_check_wire"),
+                               (3, 4, "drain_derive_and_check_wire_4_proxy_threads")):
         rings = ctypes.c_void_p()
         m.check(lib.ofi_amd_gin_rings_create(nctx, cap, ctypes.byref(rings)), "rings_create")
         comms = (m.GinComm * nctx)()
@@ -384,7 +389,7 @@ def bench_gin(lib, oracle, torch, np, args):
         t0 = time.perf_counter()
         m.check(lib.ofi_amd_gin_produce_seeded(rings, SEED, ops, 1, 64, 1, 1, 0, _gpu.stream()), "produce")
         rc = lib.ofi_amd_gin_proxy_drain_mt(rings, ops, mode, None, ctypes.cast(comms, ctypes.c_void_p),
-                                            ctypes.cast(mrs, ctypes.c_void_p), None, 20000, threads,
+                                            ctypes.cast(mrs, ctypes.c_void_p), len(mrs), None, 20000, threads,
                                             ctypes.byref(stats))
         torch.cuda.synchronize()
         secs = time.perf_counter() - t0
@@ -407,7 +412,7 @@ def bench_gin(lib, oracle, torch, np, args):
         t0 = time.perf_counter()
         m.check(lib.ofi_amd_gin_produce_table(rings, d_table.data_ptr(), t_ops, waves, 0, _gpu.stream()),
                 "produce_table")
-        rc = lib.ofi_amd_gin_proxy_drain_mt(rings, t_ops, 0, None, None, None, None, 20000, 4,
+        rc = lib.ofi_amd_gin_proxy_drain_mt(rings, t_ops, 0, None, None, None, 0, None, 20000, 4,
                                             ctypes.byref(stats))
         torch.cuda.synchronize()
         secs = time.perf_counter() - t0
@@ -440,7 +445,7 @@ def bench_gin(lib, oracle, torch, np, args):
     t0 = time.perf_counter()
     m.check(lib.ofi_amd_gin_produce_seeded(rings, SEED, l_ops, 1, 64, 1, 1, 0, _gpu.stream()), "produce")
     rc = lib.ofi_amd_gin_loopback_run(rings, l_ops, ctypes.cast(comms, ctypes.c_void_p),
-                                      ctypes.cast(mrs, ctypes.c_void_p), regions, 1, 32, 4096, 20000,
+                                      ctypes.cast(mrs, ctypes.c_void_p), 3, regions, 1, 32, 4096, 20000,
                                       ctypes.c_void_p(side.cuda_stream), ctypes.byref(lstats))
     torch.cuda.synchronize()
     secs = time.perf_counter() - t0
@@ -484,9 +489,12 @@ def bench_gin(lib, oracle, torch, np, args):
             ck = oracle.oracle_gin_stream_checksum(SEED, nctx, ops, 1, 64, 1, 1, 0, 4, 131072, 64, 1, omrs)
         ck_wire = oracle.oracle_gin_stream_checksum(SEED, nctx, ops, 1, 64, 1, 1, 1, 4, 131072, 64, 1, omrs)
         out["parity_ok"] = (out["drain"]["checksum"] == "%016x" % ck and
-                            out["drain_and_derive_wire"]["checksum"] == "%016x" % ck_wire)
+                            out["drain_and_derive_wire"]["checksum"] == "%016x" % ck and
+                            out["drain_derive_and_check_wire"]["checksum"] == "%016x" % ck_wire)
     out["derive_checksums_agree_across_thread_counts"] = (
-        out["drain_and_derive_wire"]["checksum"] == out["drain_and_derive_wire_4_proxy_threads"]["checksum"])
+        out["drain_derive_and_check_wire"]["checksum"] ==
+        out["drain_derive_and_check_wire_4_proxy_threads"]["checksum"] and
+        out["drain_and_derive_wire"]["rdma_writes"] == out["drain_derive_and_check_wire"]["rdma_writes"])
     return out
 
 

@@ -363,9 +363,11 @@ typedef struct {
 
 int ofi_amd_gin_comm_init(ofi_amd_gin_comm_t *c, uint32_t comm_id, uint32_t num_rails,
 			  uint64_t min_stripe, uint64_t max_small, uint32_t ack_model);
-/* iputSignal's derivation for one descriptor.  0, -EINVAL (signal op),
- * -EAGAIN (TX window full; the reference blocks in await_tx_window). */
-int ofi_amd_gin_iput_signal(ofi_amd_gin_comm_t *c, const ofi_amd_gin_mr_t *mrs,
+/* iputSignal's derivation for one descriptor.  mrs[0..n_mrs) is the registration table the
+ * descriptor's 16-bit handles index.  0; -EINVAL (a NULL argument, a signal op other than
+ * 0/INC/ADD, a handle >= n_mrs -- sig_mr 0xffff means "no signal handle"); -EAGAIN (TX window
+ * full; the reference blocks in await_tx_window).  *out is all-zero on failure. */
+int ofi_amd_gin_iput_signal(ofi_amd_gin_comm_t *c, const ofi_amd_gin_mr_t *mrs, uint32_t n_mrs,
 			    const ofi_amd_gin_desc_t *d, ofi_amd_gin_wire_t *out);
 /* apply_rx_consumed, include/rdma/gin/nccl_ofi_gin.h:535-543 */
 void ofi_amd_gin_apply_ack(ofi_amd_gin_comm_t *c, uint32_t wire_rx_consumed);
@@ -389,13 +391,17 @@ typedef struct {
  * progress (-ETIMEDOUT).
  *   mode 0: pop + fold every descriptor into the checksum;
  *   mode 1: also store the descriptors: out_desc[c * ops_per_context + i];
- *   mode 2: also run the iputSignal derivation per context (comms[c], mrs) and
- *           fold the wire records into the checksum; out_wire (may be NULL)
- *           receives them at [c * ops_per_context + i].
+ *   mode 2: also run the iputSignal derivation per context (comms[c], mrs[0..n_mrs));
+ *           out_wire (may be NULL) receives the wire records at
+ *           [c * ops_per_context + i].  The checksum is that of mode 0: what a proxy
+ *           does with a record (the posts) is not this library's, and checking is
+ *   mode 3: mode 2, and every wire record is folded into the checksum after its
+ *           descriptor (the parity check of the derived stream at any size).
+ * A descriptor whose handles lie outside mrs ends the call with -EINVAL.
  */
 int ofi_amd_gin_proxy_drain(ofi_amd_gin_rings_t *rings, uint64_t ops_per_context, int mode,
 			    ofi_amd_gin_desc_t *out_desc, ofi_amd_gin_comm_t *comms,
-			    const ofi_amd_gin_mr_t *mrs, ofi_amd_gin_wire_t *out_wire,
+			    const ofi_amd_gin_mr_t *mrs, uint32_t n_mrs, ofi_amd_gin_wire_t *out_wire,
 			    uint32_t timeout_ms, ofi_amd_gin_proxy_stats_t *stats);
 
 /*
@@ -406,7 +412,7 @@ int ofi_amd_gin_proxy_drain(ofi_amd_gin_rings_t *rings, uint64_t ops_per_context
  */
 int ofi_amd_gin_proxy_drain_mt(ofi_amd_gin_rings_t *rings, uint64_t ops_per_context, int mode,
 			       ofi_amd_gin_desc_t *out_desc, ofi_amd_gin_comm_t *comms,
-			       const ofi_amd_gin_mr_t *mrs, ofi_amd_gin_wire_t *out_wire,
+			       const ofi_amd_gin_mr_t *mrs, uint32_t n_mrs, ofi_amd_gin_wire_t *out_wire,
 			       uint32_t timeout_ms, uint32_t n_threads, ofi_amd_gin_proxy_stats_t *stats);
 
 /* ---- receiver side: completions -> in-order retire -> signal counters in HBM ---- */
@@ -505,7 +511,7 @@ typedef struct {
 } ofi_amd_gin_loopback_stats_t;
 
 int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *rings, uint64_t ops_per_context,
-			     ofi_amd_gin_comm_t *comms, const ofi_amd_gin_mr_t *mrs,
+			     ofi_amd_gin_comm_t *comms, const ofi_amd_gin_mr_t *mrs, uint32_t n_mrs,
 			     const ofi_amd_gin_signal_region_t *regions, uint32_t n_regions,
 			     uint32_t reorder_window, uint32_t batch_writes, uint32_t timeout_ms,
 			     void *stream, ofi_amd_gin_loopback_stats_t *stats);

@@ -504,7 +504,7 @@ void run_gin_tx(uint64_t seed, uint32_t n_ops, uint32_t ack_model)
 		std::memset(&wa, 0, sizeof(wa));
 		std::memset(&wb, 0, sizeof(wb));
 		const int ra = oracle_gin_iput_signal(&ca, mrs, &d, &wa);
-		SAME("iput rc", ra, ofi_amd_gin_iput_signal(&cb, mrs_b, &db, &wb));
+		SAME("iput rc", ra, ofi_amd_gin_iput_signal(&cb, mrs_b, 3, &db, &wb));
 		if (ra == 0) {
 			SAME("wire record", std::memcmp(&wa, &wb, sizeof(wa)), 0);
 		} else if (ra == -11) { /* window full: the receiver has consumed up to some point */

@@ -137,7 +137,7 @@ void phase_proxy_threads(uint64_t per_producer)
 		}
 	}
 	ofi_amd_gin_proxy_stats_t st;
-	const int rc = ofi_amd_gin_proxy_drain_mt(&r, per_context, 1, out.data(), nullptr, nullptr, nullptr, 60000, 2, &st);
+	const int rc = ofi_amd_gin_proxy_drain_mt(&r, per_context, 1, out.data(), nullptr, nullptr, 0, nullptr, 60000, 2, &st);
 	for (auto &t : producers) {
 		t.join();
 	}

@@ -114,7 +114,7 @@ def test_proxy_derivation_matches_oracle(lib, oracle, ack_model, agg_mask, signa
             od.size = 0                                # signal-only / empty ops now and then
         pd = m.GinDesc.from_buffer_copy(bytes(od))
         orc = oracle.oracle_gin_iput_signal(ctypes.byref(oc), omrs, ctypes.byref(od), ctypes.byref(ow))
-        prc = lib.ofi_amd_gin_iput_signal(ctypes.byref(pc), pmrs, ctypes.byref(pd), ctypes.byref(pw))
+        prc = lib.ofi_amd_gin_iput_signal(ctypes.byref(pc), pmrs, 3, ctypes.byref(pd), ctypes.byref(pw))
         assert (orc, prc) in ((0, 0), (-11, -errno.EAGAIN))
         assert bytes(ow) == bytes(pw), i
         assert bytes(oc) == bytes(pc), i
@@ -124,7 +124,7 @@ def test_proxy_derivation_matches_oracle(lib, oracle, ack_model, agg_mask, signa
         assert pc.tx_tail == 100
         lib.ofi_amd_gin_apply_ack(ctypes.byref(pc), 50)          # older ACK: ignored
         assert pc.tx_tail == 100
-        assert lib.ofi_amd_gin_iput_signal(ctypes.byref(pc), pmrs, ctypes.byref(pd), ctypes.byref(pw)) == 0
+        assert lib.ofi_amd_gin_iput_signal(ctypes.byref(pc), pmrs, 3, ctypes.byref(pd), ctypes.byref(pw)) == 0
 
 
 def test_proxy_rejects_bad_arguments(lib):
@@ -135,8 +135,27 @@ def test_proxy_rejects_bad_arguments(lib):
     assert lib.ofi_amd_gin_comm_init(ctypes.byref(c), 1, 4, 131072, 64, 1) == 0
     d = m.GinDesc(0, 0, 8, 0, 0, 1, 7, 0, 0, 0, 1, 2, 2)
     w = m.GinWire()
-    assert lib.ofi_amd_gin_iput_signal(ctypes.byref(c), _oracle.default_mrs(m.GinMr), ctypes.byref(d),
-                                       ctypes.byref(w)) == -errno.EINVAL
+    mrs = _oracle.default_mrs(m.GinMr)
+    assert lib.ofi_amd_gin_iput_signal(ctypes.byref(c), mrs, 3, ctypes.byref(d), ctypes.byref(w)) == -errno.EINVAL
+    # handles outside the registration table: the record comes from device code and is not trusted
+    state = bytes(c)
+    for src_mr, dst_mr, sig_mr, sig_op, size, n_mrs, want in [
+            (0, 1, 2, 1, 8, 3, 0), (3, 1, 2, 1, 8, 3, -errno.EINVAL), (0, 3, 2, 1, 8, 3, -errno.EINVAL),
+            (0, 1, 3, 1, 8, 3, -errno.EINVAL), (0, 1, 0xFFFF, 1, 8, 3, 0), (0, 1, 2, 1, 8, 2, -errno.EINVAL),
+            (0, 1, 9, 0, 8, 3, 0),               # no signal: the signal handle is not looked at
+            (9, 9, 2, 1, 0, 3, 0),               # no payload: the data handles are not looked at
+            (0, 1, 2, 1, 8, 0, -errno.EINVAL)]:
+        c2 = m.GinComm.from_buffer_copy(state)
+        d = m.GinDesc(0, 0, size, 8, 0, 1, sig_op, 0, 0, src_mr, dst_mr, sig_mr, 2 if sig_op else 1)
+        w.imm = 77
+        rc = lib.ofi_amd_gin_iput_signal(ctypes.byref(c2), mrs, n_mrs, ctypes.byref(d), ctypes.byref(w))
+        assert rc == want, (src_mr, dst_mr, sig_mr, sig_op, size, n_mrs)
+        if want != 0:
+            assert bytes(w) == bytes(224) and bytes(c2) == state     # nothing derived, state untouched
+    assert lib.ofi_amd_gin_iput_signal(None, mrs, 3, ctypes.byref(d), ctypes.byref(w)) == -errno.EINVAL
+    assert lib.ofi_amd_gin_iput_signal(ctypes.byref(c), None, 3, ctypes.byref(d), ctypes.byref(w)) == -errno.EINVAL
+    assert lib.ofi_amd_gin_iput_signal(ctypes.byref(c), mrs, 3, None, ctypes.byref(w)) == -errno.EINVAL
+    assert lib.ofi_amd_gin_iput_signal(ctypes.byref(c), mrs, 3, ctypes.byref(d), None) == -errno.EINVAL
 
 
 def test_device_put_header_compiles_in_a_user_kernel(tmp_path):

@@ -43,7 +43,7 @@ def produce_and_drain(lib, rings, nctx, ops, mode, signal_every=64, signal_op=1,
                                           _gpu.stream()) == 0
     rc = lib.ofi_amd_gin_proxy_drain(rings, ops, mode, ctypes.cast(descs, ctypes.c_void_p) if descs else None,
                                      ctypes.cast(comms, ctypes.c_void_p) if comms else None,
-                                     ctypes.cast(mrs, ctypes.c_void_p) if mrs else None,
+                                     ctypes.cast(mrs, ctypes.c_void_p) if mrs else None, len(mrs) if mrs else 0,
                                      ctypes.cast(wires, ctypes.c_void_p) if wires else None,
                                      timeout_ms, ctypes.byref(stats))
     _gpu.sync()
@@ -92,7 +92,7 @@ def test_second_launch_continues_ring_positions(lib, oracle, gpu):
 
 @pytest.mark.parametrize("signal_every,signal_op,agg_mask", [(64, 1, 1), (3, 2, 1), (0, 0, 0)])
 def test_wire_records_bit_exact(lib, oracle, gpu, signal_every, signal_op, agg_mask):
-    """Proxy mode 2: sequence numbers, segment counts, immediate data, stripes, doorbell flags and
+    """Proxy mode 3: sequence numbers, segment counts, immediate data, stripes, doorbell flags and
     metadata messages derived from the GPU-produced stream equal the oracle's iputSignal."""
     nctx, cap, ops = 6, 512, 12000
     rings = make_rings(lib, nctx, cap)
@@ -100,7 +100,7 @@ def test_wire_records_bit_exact(lib, oracle, gpu, signal_every, signal_op, agg_m
     for c in range(nctx):
         assert lib.ofi_amd_gin_comm_init(ctypes.byref(comms[c]), c, 4, 131072, 64, 1) == 0
     pmrs, omrs = _oracle.default_mrs(m.GinMr), _oracle.default_mrs()
-    rc, stats, _, wires = produce_and_drain(lib, rings, nctx, ops, mode=2, signal_every=signal_every,
+    rc, stats, _, wires = produce_and_drain(lib, rings, nctx, ops, mode=3, signal_every=signal_every,
                                             signal_op=signal_op, agg_mask=agg_mask, comms=comms, mrs=pmrs,
                                             want_wire=True)
     assert rc == 0
@@ -122,6 +122,52 @@ def test_wire_records_bit_exact(lib, oracle, gpu, signal_every, signal_op, agg_m
     lib.ofi_amd_gin_rings_destroy(rings)
 
 
+def test_proxy_mode_two_derives_without_folding_the_wire_records(lib, oracle, gpu):
+    """Mode 2 is mode 3 without the check: the same wire records and comm state, the checksum of
+    the descriptor stream alone."""
+    nctx, cap, ops = 5, 512, 7000
+    pmrs = _oracle.default_mrs(m.GinMr)
+    out = []
+    for mode in (2, 3):
+        rings = make_rings(lib, nctx, cap)
+        comms = (m.GinComm * nctx)()
+        for c in range(nctx):
+            assert lib.ofi_amd_gin_comm_init(ctypes.byref(comms[c]), c, 4, 131072, 64, 1) == 0
+        rc, stats, _, wires = produce_and_drain(lib, rings, nctx, ops, mode=mode, comms=comms, mrs=pmrs,
+                                                want_wire=True)
+        assert rc == 0
+        out.append((bytes(wires), bytes(comms), stats.writes, stats.checksum))
+        lib.ofi_amd_gin_rings_destroy(rings)
+    assert out[0][:3] == out[1][:3]
+    assert out[0][3] == oracle.oracle_gin_stream_checksum(SEED, nctx, ops, 1, 64, 1, 1, 0, 4, 131072, 64, 1, None)
+    assert out[1][3] == oracle.oracle_gin_stream_checksum(SEED, nctx, ops, 1, 64, 1, 1, 1, 4, 131072, 64, 1,
+                                                          _oracle.default_mrs())
+
+
+def test_proxy_stops_at_a_descriptor_with_a_handle_outside_the_table(lib, gpu):
+    """The handle indices of a record are written by device code; the proxy checks them against the
+    registration table it was given and ends the drain with -EINVAL instead of reading past it."""
+    ops, cap = 200, 256
+    table = np.zeros((1, ops, 8), dtype=np.uint64)
+    table[0, :, 2] = 4096                                        # size
+    table[0, :, 5] = 1                                           # rank 1, no signal
+    table[0, :, 7] = (1 << 16) | (0xFFFF << 32) | (1 << 48)      # src 0, dst 1, no signal handle, kind 1
+    table[0, 150, 7] = 7 | (1 << 16) | (0xFFFF << 32) | (1 << 48)    # source handle 7 of a table of 3
+    d_table = _gpu.to_dev(table)
+    for n_mrs, want_rc, want_done in ((3, -errno.EINVAL, 150), (8, 0, ops)):
+        rings = make_rings(lib, 1, cap)
+        comms = (m.GinComm * 1)()
+        assert lib.ofi_amd_gin_comm_init(ctypes.byref(comms[0]), 1, 4, 131072, 64, 1) == 0
+        mrs = (m.GinMr * 8)()
+        assert lib.ofi_amd_gin_produce_table(rings, d_table.data_ptr(), ops, 1, 0, _gpu.stream()) == 0
+        _gpu.sync()                                              # 200 records fit the ring: the producer is done
+        stats = m.GinProxyStats()
+        rc = lib.ofi_amd_gin_proxy_drain(rings, ops, 2, None, ctypes.cast(comms, ctypes.c_void_p),
+                                         ctypes.cast(mrs, ctypes.c_void_p), n_mrs, None, 2000, ctypes.byref(stats))
+        assert rc == want_rc and comms[0].tx_head == want_done
+        lib.ofi_amd_gin_rings_destroy(rings)
+
+
 def test_proxy_thread_count_does_not_change_the_result(lib, oracle, gpu):
     """Several proxy threads, each owning a range of contexts: wire records, per-context comm
     state and the checksum equal the single-thread run (and so the oracle's)."""
@@ -137,8 +183,8 @@ def test_proxy_thread_count_does_not_change_the_result(lib, oracle, gpu):
         wires = (m.GinWire * (nctx * ops))()
         stats = m.GinProxyStats()
         assert lib.ofi_amd_gin_produce_seeded(rings, SEED, ops, 1, 5, 2, 1, 0, _gpu.stream()) == 0
-        rc = lib.ofi_amd_gin_proxy_drain_mt(rings, ops, 2, None, ctypes.cast(comms, ctypes.c_void_p),
-                                            ctypes.cast(pmrs, ctypes.c_void_p),
+        rc = lib.ofi_amd_gin_proxy_drain_mt(rings, ops, 3, None, ctypes.cast(comms, ctypes.c_void_p),
+                                            ctypes.cast(pmrs, ctypes.c_void_p), 3,
                                             ctypes.cast(wires, ctypes.c_void_p), 10000, threads,
                                             ctypes.byref(stats))
         _gpu.sync()
@@ -148,15 +194,15 @@ def test_proxy_thread_count_does_not_change_the_result(lib, oracle, gpu):
         lib.ofi_amd_gin_rings_destroy(rings)
     assert all(r == results[0] for r in results[1:])
     rings = make_rings(lib, 2, 256)
-    assert lib.ofi_amd_gin_proxy_drain_mt(rings, 0, 0, None, None, None, None, 10, 0, None) == -22
-    assert lib.ofi_amd_gin_proxy_drain_mt(rings, 0, 0, None, None, None, None, 10, 65, None) == -22
+    assert lib.ofi_amd_gin_proxy_drain_mt(rings, 0, 0, None, None, None, 0, None, 10, 0, None) == -22
+    assert lib.ofi_amd_gin_proxy_drain_mt(rings, 0, 0, None, None, None, 0, None, 10, 65, None) == -22
     lib.ofi_amd_gin_rings_destroy(rings)
 
 
 def drain_descs(lib, rings, nctx, ops, timeout_ms=10000):
     descs = (m.GinDesc * (nctx * ops))()
     stats = m.GinProxyStats()
-    rc = lib.ofi_amd_gin_proxy_drain(rings, ops, 1, ctypes.cast(descs, ctypes.c_void_p), None, None, None,
+    rc = lib.ofi_amd_gin_proxy_drain(rings, ops, 1, ctypes.cast(descs, ctypes.c_void_p), None, None, 0, None,
                                      timeout_ms, ctypes.byref(stats))
     _gpu.sync()
     return rc, stats, np.frombuffer(descs, dtype=np.uint64).reshape(nctx, ops, 8)
@@ -272,9 +318,9 @@ def test_producer_gives_up_when_nobody_drains(lib, gpu):
     assert lib.ofi_amd_gin_producer_status(rings) == -errno.ETIMEDOUT
     stats = m.GinProxyStats()
     # the first lap (256 per ring) was published before the producers ran out of slots
-    rc = lib.ofi_amd_gin_proxy_drain(rings, 256, 0, None, None, None, None, 2000, ctypes.byref(stats))
+    rc = lib.ofi_amd_gin_proxy_drain(rings, 256, 0, None, None, None, 0, None, 2000, ctypes.byref(stats))
     assert rc == 0 and stats.descriptors == 512
-    rc = lib.ofi_amd_gin_proxy_drain(rings, 1, 0, None, None, None, None, 200, ctypes.byref(stats))
+    rc = lib.ofi_amd_gin_proxy_drain(rings, 1, 0, None, None, None, 0, None, 200, ctypes.byref(stats))
     assert rc == -errno.ETIMEDOUT                    # nothing more will come
     lib.ofi_amd_gin_rings_destroy(rings)
 
@@ -321,7 +367,7 @@ def test_host_producers_threaded(lib, gpu):
         t.start()
     out = (m.GinDesc * (per * producers))()
     stats = m.GinProxyStats()
-    rc = lib.ofi_amd_gin_proxy_drain(rings, per * producers, 1, ctypes.cast(out, ctypes.c_void_p), None, None,
+    rc = lib.ofi_amd_gin_proxy_drain(rings, per * producers, 1, ctypes.cast(out, ctypes.c_void_p), None, None, 0,
                                      None, 20000, ctypes.byref(stats))
     for t in threads:
         t.join()
@@ -339,6 +385,6 @@ def test_bad_arguments(lib, gpu):
         assert lib.ofi_amd_gin_rings_create(nctx, cap, ctypes.byref(r)) == -errno.EINVAL
     rings = make_rings(lib, 1, 256)
     assert lib.ofi_amd_gin_produce_seeded(rings, 1, 10, 1, 64, 3, 1, 0, None) == -errno.EINVAL
-    assert lib.ofi_amd_gin_proxy_drain(rings, 1, 1, None, None, None, None, 10, None) == -errno.EINVAL
-    assert lib.ofi_amd_gin_proxy_drain(rings, 1, 2, None, None, None, None, 10, None) == -errno.EINVAL
+    assert lib.ofi_amd_gin_proxy_drain(rings, 1, 1, None, None, None, 0, None, 10, None) == -errno.EINVAL
+    assert lib.ofi_amd_gin_proxy_drain(rings, 1, 2, None, None, None, 0, None, 10, None) == -errno.EINVAL
     lib.ofi_amd_gin_rings_destroy(rings)

@@ -85,7 +85,7 @@ def test_puts_and_signals_arrive_bit_exact(lib, gpu, nctx, ops, waves, reorder, 
     # the copies and signal updates go on their own stream: the producer kernel occupies the first
     side = torch.cuda.Stream()
     rc = lib.ofi_amd_gin_loopback_run(rings, ops, ctypes.cast(comms, ctypes.c_void_p),
-                                      ctypes.cast(mrs, ctypes.c_void_p), regions, 1, reorder, batch, 20000,
+                                      ctypes.cast(mrs, ctypes.c_void_p), len(mrs), regions, 1, reorder, batch, 20000,
                                       ctypes.c_void_p(side.cuda_stream), ctypes.byref(stats))
     torch.cuda.synchronize()
     assert rc == 0 and lib.ofi_amd_gin_producer_status(rings) == 0
@@ -153,7 +153,7 @@ def test_bad_arguments(lib, gpu):
     mrs = (m.GinMr * 3)()
     regions = (m.GinSignalRegion * 1)()
     stats = m.GinLoopbackStats()
-    args = (ctypes.cast(comms, ctypes.c_void_p), ctypes.cast(mrs, ctypes.c_void_p), regions)
+    args = (ctypes.cast(comms, ctypes.c_void_p), ctypes.cast(mrs, ctypes.c_void_p), 3, regions)
     assert lib.ofi_amd_gin_loopback_run(None, 1, *args, 1, 0, 64, 10, None, ctypes.byref(stats)) == -22
     assert lib.ofi_amd_gin_loopback_run(rings, 1, *args, 0, 0, 64, 10, None, ctypes.byref(stats)) == -22
     assert lib.ofi_amd_gin_loopback_run(rings, 1, *args, 1, 0, 0, 10, None, ctypes.byref(stats)) == -22
