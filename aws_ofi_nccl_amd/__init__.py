@@ -59,6 +59,29 @@ class GinWire(ctypes.Structure):
                 ("ack_req", c_u32), ("writes", GinWrite * 4), ("meta", c_u64 * 4)]
 
 
+class GinPost(ctypes.Structure):
+    """ofi_amd_gin_post_t (88 bytes)"""
+    _fields_ = [("kind", c_u32), ("rail", c_u32), ("more", c_u32), ("context", c_u32), ("peer", c_u32),
+                ("imm", c_u32), ("src", c_u64), ("len", c_u64), ("dest", c_u64), ("key", c_u64),
+                ("msg", c_u64 * 4)]
+
+
+FABRIC_POST_FN = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(GinPost))
+FABRIC_CQ_READ_FN = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, c_u32, ctypes.POINTER(c_u32), c_u32)
+
+
+class GinFabricOps(ctypes.Structure):
+    """ofi_amd_gin_fabric_ops_t"""
+    _fields_ = [("post", FABRIC_POST_FN), ("cq_read", FABRIC_CQ_READ_FN), ("fabric", ctypes.c_void_p)]
+
+
+class GinTxStats(ctypes.Structure):
+    """ofi_amd_gin_tx_stats_t"""
+    _fields_ = [("posts", c_u64), ("refused", c_u64), ("retries", c_u64), ("retried_ok", c_u64),
+                ("completions", c_u64), ("pending", c_u32), ("pending_max", c_u32), ("requests", c_u32),
+                ("requests_max", c_u32), ("outstanding_acks", c_u32), ("pad", c_u32)]
+
+
 class GinComm(ctypes.Structure):
     """ofi_amd_gin_comm_t"""
     _fields_ = [("sched", SchedState), ("comm_id", c_u32), ("num_rails", c_u32),
@@ -84,7 +107,8 @@ class GinLoopbackStats(ctypes.Structure):
     """ofi_amd_gin_loopback_stats_t"""
     _fields_ = [("descriptors", c_u64), ("writes", c_u64), ("copy_entries", c_u64), ("bytes", c_u64),
                 ("signals", c_u64), ("work_items", c_u64), ("acks", c_u64), ("launches", c_u64),
-                ("seconds", ctypes.c_double)]
+                ("seconds", ctypes.c_double), ("posts_refused", c_u64), ("post_retries", c_u64),
+                ("tx_completions", c_u64), ("pending_max", c_u32), ("requests_max", c_u32)]
 
 
 class GinSignalWork(ctypes.Structure):
@@ -268,7 +292,9 @@ PROTOTYPES = {
                                                 c_vp]),
     "ofi_amd_copy_table": (ctypes.c_int, [c_vp, c_vp, c_vp, c_u32, c_vp]),
     "ofi_amd_gin_loopback_run": (ctypes.c_int, [c_vp, c_u64, c_vp, c_vp, c_u32, ctypes.POINTER(GinSignalRegion), c_u32,
-                                                c_u32, c_u32, c_u32, c_vp, ctypes.POINTER(GinLoopbackStats)]),
+                                                c_u32, c_u32, c_u32, c_u32, c_u32, c_vp,
+                                                ctypes.POINTER(GinLoopbackStats)]),
+    "ofi_amd_loopfab_ring_all": (ctypes.c_int, [c_vp]),
     "ofi_amd_flush_buffer_fill": (ctypes.c_int, [c_vp, c_u64, c_vp]),
     "ofi_amd_flush_post": (ctypes.c_int, [c_vp, c_vp, c_u32, c_vp]),
     "ofi_amd_flush_test": (ctypes.c_int, [c_vp, c_u32, c_u64]),
@@ -302,6 +328,19 @@ PROTOTYPES = {
                                                c_u32, ctypes.POINTER(GinProxyStats)]),
     "ofi_amd_gin_proxy_drain_mt": (ctypes.c_int, [c_vp, c_u64, ctypes.c_int, c_vp, c_vp, c_vp, c_u32, c_vp,
                                                   c_u32, c_u32, ctypes.POINTER(GinProxyStats)]),
+    "ofi_amd_gin_tx_create": (ctypes.c_int, [c_u32, c_u32, c_u32, c_u32, ctypes.POINTER(GinFabricOps),
+                                             ctypes.POINTER(c_vp)]),
+    "ofi_amd_gin_tx_destroy": (ctypes.c_int, [c_vp]),
+    "ofi_amd_gin_tx_iput_signal": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(GinWire),
+                                                  ctypes.POINTER(c_i32)]),
+    "ofi_amd_gin_tx_send_ack": (ctypes.c_int, [c_vp, c_u32, c_u64]),
+    "ofi_amd_gin_tx_progress": (ctypes.c_int, [c_vp]),
+    "ofi_amd_gin_tx_test": (ctypes.c_int, [c_vp, c_i32, ctypes.POINTER(ctypes.c_int)]),
+    "ofi_amd_gin_tx_stats": (ctypes.c_int, [c_vp, ctypes.POINTER(GinTxStats)]),
+    "ofi_amd_loopfab_create": (ctypes.c_int, [c_u32, c_u32, ctypes.POINTER(c_vp)]),
+    "ofi_amd_loopfab_destroy": (ctypes.c_int, [c_vp]),
+    "ofi_amd_loopfab_ops": (ctypes.c_int, [c_vp, ctypes.POINTER(GinFabricOps)]),
+    "ofi_amd_loopfab_take_transmitted": (c_u32, [c_vp, ctypes.POINTER(GinPost), c_u32]),
     "ofi_amd_gin_rx_create": (ctypes.c_int, [c_u32, ctypes.POINTER(c_u32), ctypes.POINTER(c_vp)]),
     "ofi_amd_gin_rx_destroy": (ctypes.c_int, [c_vp]),
     "ofi_amd_gin_rx_write_completion": (ctypes.c_int, [c_vp, c_u32, c_u32]),

@@ -10,6 +10,7 @@
 #include <cerrno>
 #include <chrono>
 #include <cstring>
+#include <deque>
 #include <new>
 #include <vector>
 
@@ -85,11 +86,12 @@ struct lcg_t {
 extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per_context,
 					ofi_amd_gin_comm_t *comms, const ofi_amd_gin_mr_t *mrs, uint32_t n_mrs,
 					const ofi_amd_gin_signal_region_t *regions, uint32_t n_regions,
-					uint32_t reorder_window, uint32_t batch_writes, uint32_t timeout_ms,
-					void *stream, ofi_amd_gin_loopback_stats_t *stats)
+					uint32_t reorder_window, uint32_t batch_writes, uint32_t sq_depth,
+					uint32_t progress_interval, uint32_t timeout_ms, void *stream,
+					ofi_amd_gin_loopback_stats_t *stats)
 {
 	if (!r || !comms || !mrs || n_mrs == 0 || !regions || n_regions == 0 || batch_writes == 0 ||
-	    batch_writes > (1u << 24) || reorder_window > 2048) {
+	    batch_writes > (1u << 24) || reorder_window > 2048 || sq_depth > (1u << 20)) {
 		return -EINVAL;
 	}
 	using clock = std::chrono::steady_clock;
@@ -102,6 +104,10 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 	std::memset(&st, 0, sizeof(st));
 	batch_t batches[2];
 	ofi_amd_gin_rx_t *rx = nullptr;
+	ofi_amd_loopfab_t *fab = nullptr;
+	ofi_amd_gin_tx_t *tx = nullptr;
+	std::deque<int32_t> open_ops; /* operations whose posts have not all completed, oldest first */
+	constexpr uint32_t kPool = 1u << 16;
 	std::vector<uint32_t> comm_ids;
 	std::vector<event_t> in_flight;
 	std::vector<uint64_t> done;
@@ -113,8 +119,13 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 	} catch (...) {
 		return -ENOMEM;
 	}
+	uint32_t num_rails = 1;
 	for (uint32_t c = 0; c < nctx; c++) {
 		comm_ids[c] = comms[c].comm_id;
+		if (comms[c].num_rails < 1 || comms[c].num_rails > OFI_AMD_MAX_NUM_RAILS) {
+			return -EINVAL;
+		}
+		num_rails = comms[c].num_rails > num_rails ? comms[c].num_rails : num_rails;
 	}
 	/* completion of a batch is observed the reference's way: a sentinel flush read back into a
 	 * host slot behind the batch's launches (iflush, src/rdma/gin/nccl_ofi_gin.cpp:941-1003) */
@@ -125,11 +136,21 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 	}
 	if (rc == 0) rc = ofi_amd_gpu_mem_alloc(&d_flush_buf, 64);
 	if (rc == 0) rc = ofi_amd_flush_buffer_fill(d_flush_buf, kSentinel, stream);
+	/* the initiator's posts go through the progress engine into a fabric with bounded send
+	 * queues; the reference's defaults for the CQ drain (include/nccl_ofi_param.h:104-109) */
+	if (rc == 0) rc = ofi_amd_loopfab_create(num_rails, sq_depth ? sq_depth : 4096, &fab);
+	if (rc == 0) {
+		ofi_amd_gin_fabric_ops_t ops;
+		rc = ofi_amd_loopfab_ops(fab, &ops);
+		if (rc == 0) rc = ofi_amd_gin_tx_create(num_rails, 4, 4, kPool, &ops, &tx);
+	}
 	auto release = [&]() {
 		free_batch(batches[0]);
 		free_batch(batches[1]);
 		if (d_flush_buf) (void)ofi_amd_gpu_mem_free(d_flush_buf);
 		if (rx) (void)ofi_amd_gin_rx_destroy(rx);
+		if (tx) (void)ofi_amd_gin_tx_destroy(tx);
+		if (fab) (void)ofi_amd_loopfab_destroy(fab);
 	};
 	if (rc != 0) {
 		release();
@@ -192,11 +213,14 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 			return e;
 		}
 		for (;;) {
+			/* the target sends its ACKs back through the same endpoint (send_ack, :267-315) */
 			const uint32_t n = ofi_amd_gin_rx_take_acks(rx, acks, 64);
-			for (uint32_t i = 0; i < n; i++) {
-				ofi_amd_gin_apply_ack(&comms[acks[i].peer], acks[i].rx_consumed);
+			for (uint32_t i = 0; i < n && e == 0; i++) {
+				e = ofi_amd_gin_tx_send_ack(tx, acks[i].peer, acks[i].msg);
 			}
-			st.acks += n;
+			if (e != 0) {
+				return e;
+			}
 			if (n < 64) {
 				break;
 			}
@@ -230,10 +254,75 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 		return 0;
 	};
 
+	/* The wire and the initiator's progress: what the fabric has transmitted is executed (a write
+	 * becomes table entries of the next copy launch and a completion event for the target, a
+	 * metadata message an event, an ACK moves the sender's window), then one progress call of
+	 * the engine (bounded CQ drain, retry of the refused posts), then test() of the oldest
+	 * operations. */
+	ofi_amd_gin_post_t wire_posts[64];
+	auto pump = [&]() -> int {
+		for (;;) {
+			const uint32_t n = ofi_amd_loopfab_take_transmitted(fab, wire_posts, 64);
+			for (uint32_t i = 0; i < n; i++) {
+				const ofi_amd_gin_post_t &p = wire_posts[i];
+				event_t ev;
+				std::memset(&ev, 0, sizeof(ev));
+				ev.peer = p.peer;
+				if (p.kind == OFI_AMD_GIN_POST_WRITE) {
+					const uint64_t pieces = (p.len + kPiece - 1) / kPiece;
+					if (pieces > cap_copy) {
+						return -EMSGSIZE; /* a write larger than the table: raise batch_writes */
+					}
+					if (batches[cur].n_copy + pieces > cap_copy) {
+						int e = flush();
+						if (e != 0) {
+							return e;
+						}
+					}
+					batch_t &b = batches[cur];
+					for (uint64_t off = 0; off < p.len; off += kPiece) {
+						const uint64_t len = p.len - off < kPiece ? p.len - off : kPiece;
+						b.src[b.n_copy] = p.src + off;
+						b.dst[b.n_copy] = p.dest + off;
+						b.len[b.n_copy] = (uint32_t)len;
+						b.n_copy++;
+					}
+					st.bytes += p.len;
+					st.writes++;
+					ev.imm = p.imm;
+					in_flight.push_back(ev);
+				} else if (p.kind == OFI_AMD_GIN_POST_META) {
+					ev.is_meta = 1;
+					std::memcpy(ev.meta, p.msg, sizeof(ev.meta));
+					in_flight.push_back(ev);
+				} else {
+					/* gin_ack_msg_t: rx_consumed in bits 12..25 (handle_ack_completion, :1843-1869) */
+					ofi_amd_gin_apply_ack(&comms[p.peer], (uint32_t)(p.msg[0] >> 12) & 0x3fffu);
+					st.acks++;
+				}
+			}
+			if (n < 64) {
+				break;
+			}
+		}
+		int e = ofi_amd_gin_tx_progress(tx);
+		while (e == 0 && !open_ops.empty()) {
+			int done = 0;
+			e = ofi_amd_gin_tx_test(tx, open_ops.front(), &done);
+			if (e != 0 || !done) {
+				break;
+			}
+			open_ops.pop_front();
+		}
+		return e;
+	};
+
 	const auto t0 = clock::now();
 	auto last_progress = t0;
 	uint64_t remaining = (uint64_t)nctx * ops_per_context;
 	uint32_t idle = 0;
+	ofi_amd_gin_tx_stats_t ts;
+	uint32_t since_progress = 0;
 	while (remaining > 0 && rc == 0) {
 		bool progressed = false;
 		for (uint32_t c = 0; c < nctx && rc == 0; c++) {
@@ -244,57 +333,51 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 				}
 				ofi_amd_gin_wire_t wire;
 				rc = ofi_amd_gin_iput_signal(&comms[c], mrs, n_mrs, &d, &wire);
-				if (rc == -EAGAIN) {
-					/* window closed: let everything in flight arrive, which brings the ACKs */
-					rc = deliver_some(0);
-					if (rc == 0) {
-						rc = ofi_amd_gin_iput_signal(&comms[c], mrs, n_mrs, &d, &wire);
+				const auto w0 = clock::now();
+				while (rc == -EAGAIN) {
+					/* window closed (await_tx_window, :518-537, progresses until it opens): let
+					 * everything in flight arrive, which brings the ACKs */
+					rc = pump();
+					if (rc == 0) rc = deliver_some(0);
+					if (rc == 0) rc = pump();
+					if (rc == 0) rc = ofi_amd_gin_iput_signal(&comms[c], mrs, n_mrs, &d, &wire);
+					if (rc == -EAGAIN &&
+					    std::chrono::duration_cast<std::chrono::milliseconds>(clock::now() - w0).count() >
+						    (long long)timeout_ms) {
+						rc = -ETIMEDOUT;
 					}
 				}
-				if (rc != 0) {
-					break;
-				}
-				if (batches[cur].n_copy + 4u * (uint32_t)(((uint64_t)d.size >> 16) + 2u) > cap_copy) {
-					rc = flush();
-					if (rc != 0) {
+				/* room in the request pool for this operation and the ACKs it may trigger */
+				while (rc == 0) {
+					(void)ofi_amd_gin_tx_stats(tx, &ts);
+					if (ts.requests + 64 <= kPool) {
 						break;
 					}
-				}
-				batch_t &b = batches[cur];
-				for (uint32_t k = 0; k < wire.num_writes; k++) {
-					const ofi_amd_gin_write_t &w = wire.writes[k];
-					for (uint64_t off = 0; off < w.len; off += kPiece) {
-						if (b.n_copy == cap_copy) {
-							rc = -EMSGSIZE; /* an op larger than the table: raise batch_writes */
-							break;
-						}
-						const uint64_t n = w.len - off < kPiece ? w.len - off : kPiece;
-						b.src[b.n_copy] = w.src + off;
-						b.dst[b.n_copy] = w.dest + off;
-						b.len[b.n_copy] = (uint32_t)n;
-						b.n_copy++;
-					}
-					st.bytes += w.len;
-					event_t ev;
-					std::memset(&ev, 0, sizeof(ev));
-					ev.peer = c;
-					ev.imm = wire.imm;
-					in_flight.push_back(ev);
+					rc = pump();
+					if (rc == 0) rc = deliver_some(0);
 				}
 				if (rc != 0) {
 					break;
 				}
-				st.writes += wire.num_writes;
-				if (wire.has_meta) {
-					event_t ev;
-					std::memset(&ev, 0, sizeof(ev));
-					ev.peer = c;
-					ev.is_meta = 1;
-					std::memcpy(ev.meta, wire.meta, sizeof(ev.meta));
-					in_flight.push_back(ev);
-					st.signals++;
+				int32_t req = -1;
+				rc = ofi_amd_gin_tx_iput_signal(tx, c, &wire, &req);
+				if (rc != 0) {
+					break;
 				}
-				rc = deliver_some(reorder_window);
+				try {
+					open_ops.push_back(req);
+				} catch (...) {
+					rc = -ENOMEM;
+					break;
+				}
+				st.signals += wire.has_meta;
+				/* NCCL's proxy submits what it has and then calls ginProgress: a progress call
+				 * every progress_interval operations */
+				if (++since_progress >= progress_interval) {
+					since_progress = 0;
+					rc = pump();
+				}
+				if (rc == 0) rc = deliver_some(reorder_window);
 				if (rc == 0 && batches[cur].n_copy >= batch_writes) {
 					rc = flush();
 				}
@@ -315,12 +398,36 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 			}
 		}
 	}
-	if (rc == 0) {
-		rc = deliver_some(0);
+	/* The stream may end on operations whose doorbell was deferred for a successor that never
+	 * came (NCCL sets the aggregate hint only when more operations follow): ring them.  Then
+	 * run the wire, the target and the engine until nothing is left anywhere. */
+	const auto d0 = clock::now();
+	while (rc == 0) {
+		ofi_amd_loopfab_ring_all(fab);
+		rc = pump();
+		if (rc == 0) rc = deliver_some(0);
+		if (rc == 0) rc = pump();
+		if (rc != 0) {
+			break;
+		}
+		(void)ofi_amd_gin_tx_stats(tx, &ts);
+		if (open_ops.empty() && in_flight.empty() && ts.requests == 0) {
+			break;
+		}
+		if (std::chrono::duration_cast<std::chrono::milliseconds>(clock::now() - d0).count() >
+		    (long long)timeout_ms) {
+			rc = -ETIMEDOUT;
+		}
 	}
 	if (rc == 0) {
 		rc = flush();
 	}
+	(void)ofi_amd_gin_tx_stats(tx, &ts);
+	st.posts_refused = ts.refused;
+	st.post_retries = ts.retries;
+	st.tx_completions = ts.completions;
+	st.pending_max = ts.pending_max;
+	st.requests_max = ts.requests_max;
 	int sync_rc = ofi_amd_gpu_stream_synchronize(stream);
 	if (rc == 0) {
 		rc = sync_rc;

@@ -445,7 +445,7 @@ def bench_gin(lib, oracle, torch, np, args):
     t0 = time.perf_counter()
     m.check(lib.ofi_amd_gin_produce_seeded(rings, SEED, l_ops, 1, 64, 1, 1, 0, _gpu.stream()), "produce")
     rc = lib.ofi_amd_gin_loopback_run(rings, l_ops, ctypes.cast(comms, ctypes.c_void_p),
-                                      ctypes.cast(mrs, ctypes.c_void_p), 3, regions, 1, 32, 4096, 20000,
+                                      ctypes.cast(mrs, ctypes.c_void_p), 3, regions, 1, 32, 4096, 0, 1, 20000,
                                       ctypes.c_void_p(side.cuda_stream), ctypes.byref(lstats))
     torch.cuda.synchronize()
     secs = time.perf_counter() - t0

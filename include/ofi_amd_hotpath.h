@@ -415,6 +415,99 @@ int ofi_amd_gin_proxy_drain_mt(ofi_amd_gin_rings_t *rings, uint64_t ops_per_cont
 			       const ofi_amd_gin_mr_t *mrs, uint32_t n_mrs, ofi_amd_gin_wire_t *out_wire,
 			       uint32_t timeout_ms, uint32_t n_threads, ofi_amd_gin_proxy_stats_t *stats);
 
+/* ---- initiator side, below the derivation: request pool, posts, pending retry, bounded CQ drain ----
+ *
+ * What nccl_ofi_rdma_gin_put_comm::iputSignal does with the records it has derived
+ * (src/rdma/gin/nccl_ofi_gin.cpp:737-864), send_ack (:267-315), and the progress engine of
+ * nccl_ofi_gin_resources (src/rdma/gin/nccl_ofi_gin_resources.cpp:89-166 process_cq,
+ * :574-599 progress / retry_pending_reqs): every RDMA write, metadata send and ACK send is a
+ * request from one pool; a post that the fabric refuses with -EAGAIN (send queue full) goes
+ * to the back of one pending list and is posted again, without FI_MORE, by the next progress
+ * call; a progress call reads at most cq_read_count x cq_process_max_iter completions per
+ * rail (OFI_NCCL_CQ_READ_COUNT and OFI_NCCL_GIN_CQ_PROCESS_MAX_ITER, both 4 by default,
+ * include/nccl_ofi_param.h:104-109), then retries the pending list in order and stops at the
+ * first request the fabric still refuses.  The fabric is reached through two callbacks, which
+ * is where libfabric's fi_writemsg / fi_sendmsg / fi_send and fi_cq_readfrom go.
+ */
+#define OFI_AMD_GIN_POST_WRITE 1 /* fi_writemsg with FI_REMOTE_CQ_DATA */
+#define OFI_AMD_GIN_POST_META 2  /* fi_sendmsg of the 32-byte metadata message */
+#define OFI_AMD_GIN_POST_ACK 3   /* fi_send of the 8-byte ACK */
+
+typedef struct {
+	uint32_t kind;
+	uint32_t rail;
+	uint32_t more;    /* FI_MORE: this post does not ring the rail's doorbell */
+	uint32_t context; /* completion context: the fabric returns it through cq_read */
+	uint32_t peer;
+	uint32_t imm;     /* write: immediate data */
+	uint64_t src;     /* write */
+	uint64_t len;
+	uint64_t dest;
+	uint64_t key;
+	uint64_t msg[4];  /* metadata message, or msg[0] = the ACK word */
+} ofi_amd_gin_post_t; /* 88 bytes */
+
+typedef struct {
+	/* 0, -EAGAIN (send queue full: the engine queues the request), any other negative errno */
+	int (*post)(void *fabric, const ofi_amd_gin_post_t *post);
+	/* completions of rail `rail`: writes up to `max` contexts, returns how many (0: none now) or a
+	 * negative errno */
+	int (*cq_read)(void *fabric, uint32_t rail, uint32_t *contexts, uint32_t max);
+	void *fabric;
+} ofi_amd_gin_fabric_ops_t;
+
+typedef struct {
+	uint64_t posts;          /* accepted by the fabric at the first attempt */
+	uint64_t refused;        /* first attempts answered -EAGAIN (queued) */
+	uint64_t retries;        /* posts of queued requests, accepted or not */
+	uint64_t retried_ok;     /* of which accepted */
+	uint64_t completions;    /* read from the CQs */
+	uint32_t pending;        /* queued now */
+	uint32_t pending_max;
+	uint32_t requests;       /* pool entries in use now */
+	uint32_t requests_max;
+	uint32_t outstanding_acks;
+	uint32_t pad;
+} ofi_amd_gin_tx_stats_t;
+
+typedef struct ofi_amd_gin_tx ofi_amd_gin_tx_t;
+
+/* max_requests: size of the request pool (an operation takes one entry plus one per write and
+ * one for its metadata message until each completes; an ACK takes one). */
+int ofi_amd_gin_tx_create(uint32_t num_rails, uint32_t cq_read_count, uint32_t cq_process_max_iter,
+			  uint32_t max_requests, const ofi_amd_gin_fabric_ops_t *ops,
+			  ofi_amd_gin_tx_t **out);
+int ofi_amd_gin_tx_destroy(ofi_amd_gin_tx_t *tx);
+/* Posts the writes of *wire in stripe order and then its metadata message; *request is the
+ * handle for ofi_amd_gin_tx_test.  0 also when posts were queued; -ENOMEM when the pool cannot
+ * hold the operation (nothing is posted then); another negative errno when the fabric fails a
+ * post (the operation is given up as the reference does: what was posted completes unobserved). */
+int ofi_amd_gin_tx_iput_signal(ofi_amd_gin_tx_t *tx, uint32_t peer, const ofi_amd_gin_wire_t *wire,
+			       int32_t *request);
+/* send_ack: one ACK send on rail 0. */
+int ofi_amd_gin_tx_send_ack(ofi_amd_gin_tx_t *tx, uint32_t peer, uint64_t ack_msg);
+/* nccl_ofi_gin_resources::progress. */
+int ofi_amd_gin_tx_progress(ofi_amd_gin_tx_t *tx);
+/* nccl_ofi_rdma_gin_iputsignal_req::test: *done = 1 (and the request is freed) once every post
+ * of the operation has completed.  It does not progress. */
+int ofi_amd_gin_tx_test(ofi_amd_gin_tx_t *tx, int32_t request, int *done);
+int ofi_amd_gin_tx_stats(const ofi_amd_gin_tx_t *tx, ofi_amd_gin_tx_stats_t *out);
+
+/* The in-process fabric of the loop-back runs: per rail a send queue of sq_depth entries and a
+ * completion queue.  A post is refused with -EAGAIN while the rail's send queue is full; an
+ * entry leaves the send queue when its completion is read.  Entries are transmitted in post
+ * order per rail once the rail's doorbell rings: by a post without FI_MORE, or by the queue
+ * filling up.  ofi_amd_loopfab_take_transmitted hands the transmitted posts, in the order
+ * their doorbells rang, to the caller, who plays the wire and the target; a taken post's
+ * completion becomes readable at once. */
+typedef struct ofi_amd_loopfab ofi_amd_loopfab_t;
+int ofi_amd_loopfab_create(uint32_t num_rails, uint32_t sq_depth, ofi_amd_loopfab_t **out);
+int ofi_amd_loopfab_destroy(ofi_amd_loopfab_t *f);
+int ofi_amd_loopfab_ops(ofi_amd_loopfab_t *f, ofi_amd_gin_fabric_ops_t *ops);
+uint32_t ofi_amd_loopfab_take_transmitted(ofi_amd_loopfab_t *f, ofi_amd_gin_post_t *out, uint32_t cap);
+/* Rings every rail's doorbell: posts still waiting behind FI_MORE are transmitted. */
+int ofi_amd_loopfab_ring_all(ofi_amd_loopfab_t *f);
+
 /* ---- receiver side: completions -> in-order retire -> signal counters in HBM ---- */
 
 /* One folded signal delivery: add `value` to the 8-byte counter at base + offset
@@ -483,13 +576,19 @@ int ofi_amd_gin_signal_apply(const ofi_amd_gin_signal_work_t *d_work, uint32_t n
  * In-process loop-back of the whole GIN path on one GPU: initiator and target are the same
  * device, the "network" is this call.  For every descriptor drained from the rings it
  *   1. derives the wire record (ofi_amd_gin_iput_signal on comms[context], ack_model 0),
- *   2. queues each RDMA write as a (source, destination, length) copy -- source
- *      mrs[src_mr].local_base + src_off, destination the write's `dest` (give the
- *      destination MR's remote_address_offset the device address of the target buffer) --
- *      long writes cut into 64 KiB pieces,
- *   3. delivers the write completions and the metadata message to a receiver
- *      (ofi_amd_gin_rx_*, one peer per context), up to reorder_window events out of order,
- *   4. returns the receiver's ACKs to the sender (ofi_amd_gin_apply_ack),
+ *   2. posts it through the progress engine (ofi_amd_gin_tx_*) into the in-process fabric
+ *      (ofi_amd_loopfab_*, sq_depth entries per rail; 0 = 4096): refused posts are queued and
+ *      retried by the engine's progress calls -- one every progress_interval operations (0
+ *      or 1: after each), as NCCL's proxy alternates between submitting and ginProgress --
+ *      and completions are drained 16 per rail and call,
+ *   3. executes what the fabric transmits: each RDMA write as a (source, destination, length)
+ *      copy -- source mrs[src_mr].local_base + src_off, destination the write's `dest` (give
+ *      the destination MR's remote_address_offset the device address of the target buffer) --
+ *      long writes cut into 64 KiB pieces; the write completions and the metadata message go
+ *      to a receiver (ofi_amd_gin_rx_*, one peer per context), up to reorder_window events
+ *      out of order,
+ *   4. sends the receiver's ACKs back through the same engine and fabric; an ACK that arrives
+ *      moves the sender's window (ofi_amd_gin_apply_ack),
  * and every batch_writes queued copies (and at the end) launches, in this order on `stream`,
  * ofi_amd_copy_table for the copies and ofi_amd_gin_signal_apply for the signals the
  * receiver has released: a signal is applied after the payloads it covers.  `stream` must
@@ -508,13 +607,19 @@ typedef struct {
 	uint64_t acks;            /* ACKs returned to the senders */
 	uint64_t launches;        /* copy + apply launch pairs */
 	double seconds;
+	uint64_t posts_refused;   /* posts the fabric answered -EAGAIN (send queue full) */
+	uint64_t post_retries;    /* posts of queued requests by progress calls */
+	uint64_t tx_completions;  /* initiator completions read from the CQs */
+	uint32_t pending_max;     /* longest the pending list got */
+	uint32_t requests_max;    /* most request-pool entries in use */
 } ofi_amd_gin_loopback_stats_t;
 
 int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *rings, uint64_t ops_per_context,
 			     ofi_amd_gin_comm_t *comms, const ofi_amd_gin_mr_t *mrs, uint32_t n_mrs,
 			     const ofi_amd_gin_signal_region_t *regions, uint32_t n_regions,
-			     uint32_t reorder_window, uint32_t batch_writes, uint32_t timeout_ms,
-			     void *stream, ofi_amd_gin_loopback_stats_t *stats);
+			     uint32_t reorder_window, uint32_t batch_writes, uint32_t sq_depth,
+			     uint32_t progress_interval, uint32_t timeout_ms, void *stream,
+			     ofi_amd_gin_loopback_stats_t *stats);
 
 /* ======================================================================
  * 5. Tuner: batched cost model and region lookup.

@@ -29,6 +29,9 @@
  *                    walk) worked out by hand on literal wire words for in-order,
  *                    reversed and swapped arrivals, either submission path, folded
  *                    runs, the 14-bit cursor wrap and per-peer comm ids
+ *   gin tx engine    post / retry / completion orders worked out by hand against scripted
+ *                    fabrics (full send queues, FI_MORE dropped on retry, head-of-line stop of
+ *                    the retry, 16 completions per rail per progress call)
  *   gin signal apply per-slot sums against a plain scatter-add (mod 2^64)
  *   region geometry  ~70 points + 4 extend_region cases of
  *                    tests/unit/region_based_tuner.cpp
@@ -231,6 +234,36 @@ void oracle_gin_comm_init(oracle_gin_comm_t *c, uint32_t comm_id, uint32_t num_r
 int oracle_gin_iput_signal(oracle_gin_comm_t *c, const oracle_gin_mr_t *mrs,
 			   const oracle_gin_desc_t *d, oracle_gin_wire_t *out);
 void oracle_gin_apply_ack(oracle_gin_comm_t *c, uint32_t wire_rx_consumed);
+
+/* ---- initiator below the derivation (oracle_gin_tx.c): posts, pending retry, CQ drain ---- */
+#define ORACLE_GIN_POST_WRITE 1
+#define ORACLE_GIN_POST_META 2
+#define ORACLE_GIN_POST_ACK 3
+typedef struct {
+	uint32_t kind, rail, more, context, peer, imm;
+	uint64_t src, len, dest, key;
+	uint64_t msg[4];
+} oracle_gin_post_t;
+typedef struct {
+	int (*post)(void *fabric, const oracle_gin_post_t *post);
+	int (*cq_read)(void *fabric, uint32_t rail, uint32_t *contexts, uint32_t max);
+	void *fabric;
+} oracle_gin_fabric_ops_t;
+typedef struct {
+	uint64_t posts, refused, retries, retried_ok, completions;
+	uint32_t pending, pending_max, requests, requests_max, outstanding_acks, pad;
+} oracle_gin_tx_stats_t;
+typedef struct oracle_gin_tx oracle_gin_tx_t;
+oracle_gin_tx_t *oracle_gin_tx_create(uint32_t num_rails, uint32_t cq_read_count,
+				      uint32_t cq_process_max_iter, uint32_t max_requests,
+				      const oracle_gin_fabric_ops_t *ops);
+void oracle_gin_tx_destroy(oracle_gin_tx_t *tx);
+int oracle_gin_tx_iput_signal(oracle_gin_tx_t *tx, uint32_t peer, const oracle_gin_wire_t *wire,
+			      int32_t *request);
+int oracle_gin_tx_send_ack(oracle_gin_tx_t *tx, uint32_t peer, uint64_t ack_msg);
+int oracle_gin_tx_progress(oracle_gin_tx_t *tx);
+int oracle_gin_tx_test(oracle_gin_tx_t *tx, int32_t request, int *done);
+void oracle_gin_tx_stats(const oracle_gin_tx_t *tx, oracle_gin_tx_stats_t *out);
 
 /* ---- receiver side (oracle_gin_rx.c) ---- */
 

@@ -45,6 +45,26 @@ class GinWire(ctypes.Structure):
                 ("ack_req", c_u32), ("writes", GinWrite * 4), ("meta", c_u64 * 4)]
 
 
+class GinPost(ctypes.Structure):
+    _fields_ = [("kind", c_u32), ("rail", c_u32), ("more", c_u32), ("context", c_u32), ("peer", c_u32),
+                ("imm", c_u32), ("src", c_u64), ("len", c_u64), ("dest", c_u64), ("key", c_u64),
+                ("msg", c_u64 * 4)]
+
+
+FABRIC_POST_FN = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(GinPost))
+FABRIC_CQ_READ_FN = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, c_u32, ctypes.POINTER(c_u32), c_u32)
+
+
+class GinFabricOps(ctypes.Structure):
+    _fields_ = [("post", FABRIC_POST_FN), ("cq_read", FABRIC_CQ_READ_FN), ("fabric", ctypes.c_void_p)]
+
+
+class GinTxStats(ctypes.Structure):
+    _fields_ = [("posts", c_u64), ("refused", c_u64), ("retries", c_u64), ("retried_ok", c_u64),
+                ("completions", c_u64), ("pending", c_u32), ("pending_max", c_u32), ("requests", c_u32),
+                ("requests_max", c_u32), ("outstanding_acks", c_u32), ("pad", c_u32)]
+
+
 class GinMr(ctypes.Structure):
     _fields_ = [("local_base", c_u64), ("remote_address", c_u64),
                 ("remote_address_offset", c_u64), ("key", c_u64 * 4)]
@@ -129,6 +149,14 @@ class Point(ctypes.Structure):
 
 
 _ORACLE_PROTOS = {
+    "oracle_gin_tx_create": (ctypes.c_void_p, [c_u32, c_u32, c_u32, c_u32, ctypes.POINTER(GinFabricOps)]),
+    "oracle_gin_tx_destroy": (None, [ctypes.c_void_p]),
+    "oracle_gin_tx_iput_signal": (c_int, [ctypes.c_void_p, c_u32, ctypes.POINTER(GinWire),
+                                          ctypes.POINTER(c_i32)]),
+    "oracle_gin_tx_send_ack": (c_int, [ctypes.c_void_p, c_u32, c_u64]),
+    "oracle_gin_tx_progress": (c_int, [ctypes.c_void_p]),
+    "oracle_gin_tx_test": (c_int, [ctypes.c_void_p, c_i32, ctypes.POINTER(c_int)]),
+    "oracle_gin_tx_stats": (None, [ctypes.c_void_p, ctypes.POINTER(GinTxStats)]),
     "oracle_sched_init": (None, [ctypes.POINTER(Sched), c_int, c_u64, c_u64]),
     "oracle_sched_num_stripes": (c_int, [ctypes.POINTER(Sched), c_u64]),
     "oracle_sched_get_schedule": (c_int, [ctypes.POINTER(Sched), c_u64, c_u64, ctypes.POINTER(Xfer)]),

@@ -50,12 +50,14 @@ def build_ops(rng, nctx, ops, src_bytes, max_size):
     return table, replay, dst_pos + 64
 
 
-@pytest.mark.parametrize("nctx,ops,waves,reorder,batch,max_size", [
-    (1, 300, 1, 0, 64, 70_000),
-    (4, 1500, 3, 37, 512, 300_000),
-    (3, 6000, 2, 500, 4096, 40_000),      # more than 4096 ops per context in flight at times: ACKs matter
+@pytest.mark.parametrize("nctx,ops,waves,reorder,batch,max_size,sq_depth", [
+    (1, 300, 1, 0, 64, 70_000, 0),
+    (4, 1500, 3, 37, 512, 300_000, 0),
+    (3, 6000, 2, 500, 4096, 40_000, 0),   # more than 4096 ops per context in flight at times: ACKs matter
+    (4, 6000, 2, 64, 1024, 600_000, 8),   # send queues of 8 entries per rail, a progress call every 16 ops
+    (2, 3000, 1, 0, 256, 300_000, 1),     # one entry per rail: most posts between two progress calls are refused
 ])
-def test_puts_and_signals_arrive_bit_exact(lib, gpu, nctx, ops, waves, reorder, batch, max_size):
+def test_puts_and_signals_arrive_bit_exact(lib, gpu, nctx, ops, waves, reorder, batch, max_size, sq_depth):
     rng = np.random.default_rng(nctx * 1000 + ops)
     src_bytes = 32 << 20
     src = rng.integers(0, 256, src_bytes, dtype=np.uint8)
@@ -85,7 +87,8 @@ def test_puts_and_signals_arrive_bit_exact(lib, gpu, nctx, ops, waves, reorder, 
     # the copies and signal updates go on their own stream: the producer kernel occupies the first
     side = torch.cuda.Stream()
     rc = lib.ofi_amd_gin_loopback_run(rings, ops, ctypes.cast(comms, ctypes.c_void_p),
-                                      ctypes.cast(mrs, ctypes.c_void_p), len(mrs), regions, 1, reorder, batch, 20000,
+                                      ctypes.cast(mrs, ctypes.c_void_p), len(mrs), regions, 1, reorder, batch,
+                                      sq_depth, 16 if sq_depth else 1, 20000,
                                       ctypes.c_void_p(side.cuda_stream), ctypes.byref(stats))
     torch.cuda.synchronize()
     assert rc == 0 and lib.ofi_amd_gin_producer_status(rings) == 0
@@ -116,6 +119,15 @@ def test_puts_and_signals_arrive_bit_exact(lib, gpu, nctx, ops, waves, reorder, 
             assert outstanding < ops                  # ACKs did come back
     if ops > 4096 + 64:
         assert stats.acks > 0
+    # every post completed on the initiator: one per RDMA write, metadata message and ACK
+    assert stats.tx_completions == stats.writes + stats.signals + stats.acks
+    if sq_depth:
+        # bounded send queues: posts were refused, queued and posted again by progress calls, and
+        # everything above still holds
+        assert stats.posts_refused > (2000 if sq_depth == 8 else 3000), stats.posts_refused
+        assert stats.post_retries >= stats.posts_refused and stats.pending_max > 1
+    else:
+        assert stats.posts_refused == 0 and stats.post_retries == 0
     assert _gpu.fetch_async_errors(lib) == 0
     lib.ofi_amd_gin_rings_destroy(rings)
 
@@ -154,8 +166,8 @@ def test_bad_arguments(lib, gpu):
     regions = (m.GinSignalRegion * 1)()
     stats = m.GinLoopbackStats()
     args = (ctypes.cast(comms, ctypes.c_void_p), ctypes.cast(mrs, ctypes.c_void_p), 3, regions)
-    assert lib.ofi_amd_gin_loopback_run(None, 1, *args, 1, 0, 64, 10, None, ctypes.byref(stats)) == -22
-    assert lib.ofi_amd_gin_loopback_run(rings, 1, *args, 0, 0, 64, 10, None, ctypes.byref(stats)) == -22
-    assert lib.ofi_amd_gin_loopback_run(rings, 1, *args, 1, 0, 0, 10, None, ctypes.byref(stats)) == -22
-    assert lib.ofi_amd_gin_loopback_run(rings, 1, *args, 1, 5000, 64, 10, None, ctypes.byref(stats)) == -22
+    assert lib.ofi_amd_gin_loopback_run(None, 1, *args, 1, 0, 64, 0, 1, 10, None, ctypes.byref(stats)) == -22
+    assert lib.ofi_amd_gin_loopback_run(rings, 1, *args, 0, 0, 64, 0, 1, 10, None, ctypes.byref(stats)) == -22
+    assert lib.ofi_amd_gin_loopback_run(rings, 1, *args, 1, 0, 0, 0, 1, 10, None, ctypes.byref(stats)) == -22
+    assert lib.ofi_amd_gin_loopback_run(rings, 1, *args, 1, 5000, 64, 0, 1, 10, None, ctypes.byref(stats)) == -22
     lib.ofi_amd_gin_rings_destroy(rings)
