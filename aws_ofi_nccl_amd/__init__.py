@@ -228,6 +228,11 @@ class NcclTunerV2(ctypes.Structure):
                 ("destroy", ctypes.CFUNCTYPE(ctypes.c_int, c_vp))]
 
 
+class TunerCtxStats(ctypes.Structure):
+    """ofi_amd_tuner_ctx_stats_t"""
+    _fields_ = [("hits", c_u64), ("misses", c_u64), ("preloaded", c_u64)]
+
+
 class NcclTunerV3(ctypes.Structure):
     """ncclTuner_v3_t"""
     _fields_ = [("name", ctypes.c_char_p),
@@ -286,7 +291,7 @@ PROTOTYPES = {
     "ofi_amd_sched_batch_noalloc": (ctypes.c_int, [c_vp, c_vp, c_u64, c_u64, c_vp, c_vp, c_vp]),
     "ofi_amd_sched_get_schedule": (ctypes.c_int, [ctypes.POINTER(SchedState), c_u64, c_u64,
                                                   ctypes.POINTER(XferInfo)]),
-    "ofi_amd_bounce_scatter": (ctypes.c_int, [c_vp, c_vp, c_u64, c_vp, c_vp, c_vp, c_u32, c_vp,
+    "ofi_amd_bounce_scatter": (ctypes.c_int, [c_vp, c_u64, c_vp, c_u64, c_vp, c_vp, c_vp, c_u32, c_vp,
                                               c_vp]),
     "ofi_amd_eager_copy_batch": (ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_u32, c_vp, c_vp,
                                                 c_vp]),
@@ -425,6 +430,8 @@ PROTOTYPES = {
     "ofi_amd_tuner_model_grid": (ctypes.c_int, [c_vp, c_vp, c_u32, c_vp, c_vp, c_vp]),
     "ofi_amd_tuner_region_grid": (ctypes.c_int, [c_vp, c_vp, c_u32, c_vp, c_vp]),
     "ofi_amd_tuner_query": (ctypes.c_int, [c_vp, c_u32, c_vp]),
+    "ofi_amd_tuner_query_prepare": (ctypes.c_int, [c_u32]),
+    "ofi_amd_tuner_ctx_stats": (ctypes.c_int, [c_vp, ctypes.POINTER(TunerCtxStats)]),
 }
 
 

@@ -139,7 +139,7 @@ __device__ __forceinline__ void copy_words(const uint8_t *__restrict__ s, uint8_
 }
 
 __global__ __launch_bounds__(kBlock) void bounce_scatter_kernel(
-	const uint8_t *__restrict__ src, uint8_t *__restrict__ arena, uint64_t arena_bytes,
+	const uint8_t *__restrict__ src, uint64_t src_bytes, uint8_t *__restrict__ arena, uint64_t arena_bytes,
 	const uint64_t *__restrict__ src_off, const uint64_t *__restrict__ dst_off,
 	const uint32_t *__restrict__ len, uint32_t n, uint32_t *__restrict__ flush,
 	uint32_t *__restrict__ err)
@@ -162,8 +162,11 @@ __global__ __launch_bounds__(kBlock) void bounce_scatter_kernel(
 	const uint64_t doff = dst_off[buf];
 	const uint32_t bytes = len[buf];
 	const uint64_t soff = src_off[buf];
-	/* precondition check: skip (and report) instead of writing out of range */
-	if ((doff & 63u) != 0 || doff > arena_bytes || bytes > arena_bytes - doff) {
+	/* precondition check: skip (and report) instead of reading or writing out of range; the
+	 * read-back takes four bytes at the destination whatever the length */
+	const uint64_t need = (flush != nullptr && bytes < 4u) ? 4u : bytes;
+	if ((doff & 63u) != 0 || doff > arena_bytes || need > arena_bytes - doff || soff > src_bytes ||
+	    bytes > src_bytes - soff) {
 		if (lane == 0) {
 			atomicOr(err, ofi_amd::ASYNC_ERR_BOUNCE_RANGE);
 		}
@@ -341,7 +344,7 @@ using namespace ofi_amd;
 
 extern "C" {
 
-int ofi_amd_bounce_scatter(const void *d_src, void *d_arena, uint64_t arena_bytes,
+int ofi_amd_bounce_scatter(const void *d_src, uint64_t src_bytes, void *d_arena, uint64_t arena_bytes,
 			   const uint64_t *d_src_off, const uint64_t *d_dst_off,
 			   const uint32_t *d_len, uint32_t n, uint32_t *d_flush, void *stream)
 {
@@ -352,7 +355,7 @@ int ofi_amd_bounce_scatter(const void *d_src, void *d_arena, uint64_t arena_byte
 	if (n == 0) {
 		return 0;
 	}
-	if (!d_src || !d_arena || !d_src_off || !d_dst_off || !d_len) {
+	if (!d_src || !d_arena || !d_src_off || !d_dst_off || !d_len || n > (1u << 30)) {
 		return -EINVAL;
 	}
 	uint32_t *err = async_error_word();
@@ -363,7 +366,7 @@ int ofi_amd_bounce_scatter(const void *d_src, void *d_arena, uint64_t arena_byte
 	const uint32_t round = kXcds * kGroup; /* whole rounds over the XCDs */
 	blocks = (blocks + round - 1) / round * round;
 	hipLaunchKernelGGL(bounce_scatter_kernel, dim3(blocks), dim3(kBlock), kLdsPerBlock, as_stream(stream),
-			   static_cast<const uint8_t *>(d_src), static_cast<uint8_t *>(d_arena),
+			   static_cast<const uint8_t *>(d_src), src_bytes, static_cast<uint8_t *>(d_arena),
 			   arena_bytes, d_src_off, d_dst_off, d_len, n, d_flush, err);
 	OFI_AMD_HIP_TRY(hipGetLastError());
 	return 0;

@@ -310,17 +310,23 @@ double log2_coord(double v)
 	return std::log2(v);
 }
 
-/* Built once per process (about 13 KiB of device memory, never freed). */
+/* Built once per process (about 13 KiB of device memory, never freed).  A failed build is
+ * not remembered: the next caller tries again. */
 int device_region_tables(region_tables_t *out)
 {
-	static std::once_flag once;
+	static std::mutex lock;
 	static region_tables_t tables;
-	static int status = -ENODEV;
-	std::call_once(once, [] { status = build_region_tables(&tables); });
-	if (status == 0) {
-		*out = tables;
+	static bool built = false;
+	std::lock_guard<std::mutex> g(lock);
+	if (!built) {
+		const int status = build_region_tables(&tables);
+		if (status != 0) {
+			return status;
+		}
+		built = true;
 	}
-	return status;
+	*out = tables;
+	return 0;
 }
 
 } // namespace ofi_amd_tuner

@@ -2,10 +2,15 @@
  * NCCL / RCCL tuner plugin symbols on top of the GPU tuner: ncclTunerPlugin_v2, _v3 and
  * _v6 with the behaviour of src/tuner/nccl_ofi_tuner.cpp:29-279 in the reference.
  *
- * NCCL calls getCollInfo once per collective launch and a training job repeats the same
- * few (collective, size) pairs, so every distinct question is evaluated once on the GPU
- * (ofi_amd_tuner_query) and then served from a per-communicator table.  There is no host
- * evaluation path: without a usable GPU init fails.
+ * NCCL calls getCollInfo once per collective launch, at enqueue time -- possibly inside a
+ * stream capture -- and a training job repeats the same few (collective, size) pairs.  So
+ * init does everything that allocates (the query stream, its pinned staging, the region
+ * tables in device memory) and evaluates, in one batched launch, the power-of-two size
+ * ladder of every collective for the communicator's shape; after that a question is served
+ * from the per-communicator table, and only a size off the ladder costs a GPU round trip
+ * (a launch on a private stream and a wait, no allocation), once.  There is no host
+ * evaluation path: without a usable GPU init fails, and a query that fails later hands the
+ * decision back to NCCL's own tuner.
  *
  * Platform selection follows include/tuner/nccl_ofi_tuner_process_config.h:17-116: the
  * EC2 product name (OFI_NCCL_FORCE_PRODUCT_NAME, else the DMI product_name file,
@@ -22,6 +27,7 @@
 #include <new>
 #include <string>
 #include <unordered_map>
+#include <vector>
 
 #include <strings.h>
 
@@ -66,14 +72,82 @@ struct key_hash {
 	}
 };
 
+constexpr uint32_t kCtxMagic = 0x544e5543u;
+
 struct tuner_ctx {
+	uint32_t magic = kCtxMagic;
 	int platform;
 	int model; /* 0: region tuner, 1: model tuner */
 	uint64_t ranks, nodes;
 	int num_channels, net_comp_overhead;
 	std::mutex lock;
 	std::unordered_map<key_t, ofi_amd_tuner_answer_t, key_hash> memo;
+	ofi_amd_tuner_ctx_stats_t stats = {};
 };
+
+constexpr int kMaxPreloadPipeOps = 4; /* numPipeOps values evaluated ahead for the model tuner */
+constexpr uint32_t kPreloadCapacity = 1024;
+
+void fill_query(const tuner_ctx *ctx, const key_t &key, ofi_amd_tuner_query_t *q)
+{
+	std::memset(q, 0, sizeof(*q));
+	q->platform = ctx->platform;
+	q->kind = key.kind;
+	q->coll = key.coll;
+	q->pipe_ops = key.pipe_ops;
+	q->num_channels = ctx->num_channels;
+	q->net_comp_overhead = ctx->net_comp_overhead;
+	q->algo = key.algo;
+	q->proto = key.proto;
+	q->allowed_mask = key.mask;
+	q->nbytes = key.nbytes;
+	q->num_ranks = ctx->ranks;
+	q->num_nodes = ctx->nodes;
+}
+
+/* The questions a job typically asks first: every collective at the powers of two from 1 B to
+ * 64 GiB with nothing ruled out, and the chunk sizes of the two tuned (collective, algorithm,
+ * protocol) combinations, in one launch. */
+int preload(tuner_ctx *ctx)
+{
+	std::vector<key_t> keys;
+	try {
+		for (int coll = 0; coll < NCCL_NUM_FUNCTIONS; coll++) {
+			for (int e = 0; e <= 36; e++) {
+				const uint64_t nbytes = 1ull << e;
+				if (ctx->model) {
+					for (int pipe = 1; pipe <= kMaxPreloadPipeOps; pipe++) {
+						keys.push_back(key_t{ nbytes, kAllAllowed, 1, coll, pipe, 0, 0 });
+					}
+				} else {
+					keys.push_back(key_t{ nbytes, kAllAllowed, 0, coll, 0, 0, 0 });
+				}
+			}
+		}
+		if (!ctx->model) {
+			for (int e = 0; e <= 36; e++) {
+				keys.push_back(key_t{ 1ull << e, kAllAllowed, 2, 4 /* AllReduce */, 0, 0 /* Tree */, 1 /* LL128 */ });
+				keys.push_back(key_t{ 1ull << e, kAllAllowed, 2, 2 /* AllGather */, 0, kAlgoPat, 2 /* Simple */ });
+			}
+		}
+		std::vector<ofi_amd_tuner_query_t> qs(keys.size());
+		std::vector<ofi_amd_tuner_answer_t> as(keys.size());
+		for (size_t i = 0; i < keys.size(); i++) {
+			fill_query(ctx, keys[i], &qs[i]);
+		}
+		const int rc = ofi_amd_tuner_query(qs.data(), (uint32_t)qs.size(), as.data());
+		if (rc != 0) {
+			return rc;
+		}
+		for (size_t i = 0; i < keys.size(); i++) {
+			ctx->memo.emplace(keys[i], as[i]);
+		}
+		ctx->stats.preloaded = keys.size();
+	} catch (...) {
+		return -ENOMEM;
+	}
+	return 0;
+}
 
 /* nccl_net_ofi_get_product_name, src/nccl_ofi_system.cpp:110-160 */
 std::string product_name()
@@ -161,6 +235,12 @@ ncclResult_t tuner_init(size_t nRanks, size_t nNodes, ncclDebugLogger_t logFunct
 		TUNER_WARN("GPU tuner unavailable (ofi_amd_gpu_init: %d)", rc);
 		return ncclSystemError;
 	}
+	/* everything the later queries need is created here, not inside a getCollInfo call */
+	rc = ofi_amd_tuner_query_prepare(kPreloadCapacity);
+	if (rc != 0) {
+		TUNER_WARN("GPU tuner unavailable (ofi_amd_tuner_query_prepare: %d)", rc);
+		return ncclSystemError;
+	}
 	auto *ctx = new (std::nothrow) tuner_ctx();
 	if (!ctx) {
 		TUNER_WARN("Context allocation failed.");
@@ -174,6 +254,14 @@ ncclResult_t tuner_init(size_t nRanks, size_t nNodes, ncclDebugLogger_t logFunct
 	ctx->net_comp_overhead = env_int("OFI_NCCL_TUNER_NET_COMP_OVERHEAD", 3);
 	TUNER_INFO("%s base Tuner is chosen for platform: %s", ctx->model ? "Model" : "Region", name.c_str());
 	TUNER_INFO("Tuner init: comm with %ld ranks and %ld nodes.", (long)nRanks, (long)nNodes);
+	if (nRanks > 0 && nNodes > 0) {
+		rc = preload(ctx);
+		if (rc != 0) {
+			TUNER_WARN("GPU tuner pre-evaluation failed: %d", rc);
+			delete ctx;
+			return ncclSystemError;
+		}
+	}
 	*context = ctx;
 	return ncclSuccess;
 }
@@ -207,22 +295,31 @@ int ask(tuner_ctx *ctx, int kind, int coll, uint64_t nbytes, int pipe_ops, uint3
 	auto it = ctx->memo.find(key);
 	if (it != ctx->memo.end()) {
 		*out = it->second;
+		ctx->stats.hits++;
 		return 0;
 	}
+	if (kind != 2 && mask != kAllAllowed) {
+		/* The answer with nothing ruled out also holds under a narrower mask that still
+		 * allows the chosen cell: the region tuner takes the first region in table order
+		 * that holds the point and is allowed (src/tuner/nccl_ofi_regions.cpp:2106-2128),
+		 * so if the first region that holds the point is allowed it stays the answer, and
+		 * if no region holds the point none does under any mask; the model tuner's minimum
+		 * over all cells stays the minimum when a cell other than it is taken away. */
+		key_t open = key;
+		open.mask = kAllAllowed;
+		it = ctx->memo.find(open);
+		if (it != ctx->memo.end()) {
+			const ofi_amd_tuner_answer_t &a = it->second;
+			if (a.algo < 0 || ((mask >> (a.algo * NCCL_NUM_PROTOCOLS + a.proto)) & 1u)) {
+				*out = a;
+				ctx->stats.hits++;
+				return 0;
+			}
+		}
+	}
+	ctx->stats.misses++;
 	ofi_amd_tuner_query_t q;
-	std::memset(&q, 0, sizeof(q));
-	q.platform = ctx->platform;
-	q.kind = kind;
-	q.coll = coll;
-	q.pipe_ops = pipe_ops;
-	q.num_channels = ctx->num_channels;
-	q.net_comp_overhead = ctx->net_comp_overhead;
-	q.algo = algo;
-	q.proto = proto;
-	q.allowed_mask = mask;
-	q.nbytes = nbytes;
-	q.num_ranks = ctx->ranks;
-	q.num_nodes = ctx->nodes;
+	fill_query(ctx, key, &q);
 	int rc = ofi_amd_tuner_query(&q, 1, out);
 	if (rc == 0) {
 		if (ctx->memo.size() > (1u << 20)) {
@@ -259,8 +356,9 @@ ncclResult_t tuner_get_coll_info(void *context, ncclFunc_t collType, size_t nByt
 	ofi_amd_tuner_answer_t ans;
 	int rc = ask(ctx, ctx->model, (int)collType, nBytes, ctx->model ? numPipeOps : 0, mask, 0, 0, &ans);
 	if (rc != 0) {
-		TUNER_WARN("GPU tuner query failed: %d", rc);
-		return ncclSystemError;
+		/* the cost table is left as NCCL filled it: its own tuner decides this collective */
+		TUNER_WARN("GPU tuner query failed (%d): falling back to NCCL's tuner for this call", rc);
+		return ncclSuccess;
 	}
 	if (ans.algo >= 0 && ans.algo < numAlgo && ans.proto >= 0 && ans.proto < numProto) {
 		table[ans.algo][ans.proto] = 0.0f;
@@ -299,7 +397,8 @@ ncclResult_t tuner_get_coll_info_v2(void *context, ncclFunc_t collType, size_t n
 	ofi_amd_tuner_answer_t ans;
 	int rc = ask(ctx, ctx->model, (int)collType, nBytes, ctx->model ? numPipeOps : 0, mask, 0, 0, &ans);
 	if (rc != 0) {
-		return ncclSystemError;
+		TUNER_WARN("GPU tuner query failed (%d): falling back to NCCL's tuner for this call", rc);
+		return ncclSuccess;
 	}
 	if (ans.algo >= 0 && algorithm && protocol) {
 		*algorithm = ans.algo;
@@ -320,7 +419,8 @@ ncclResult_t tuner_get_chunk_size(void *context, ncclFunc_t collType, size_t nBy
 	ofi_amd_tuner_answer_t ans;
 	int rc = ask(ctx, 2, (int)collType, nBytes, 0, kAllAllowed, algo, proto, &ans);
 	if (rc != 0) {
-		return ncclSystemError;
+		TUNER_WARN("GPU tuner query failed (%d): chunk size left to NCCL", rc);
+		return ncclSuccess;
 	}
 	if (ans.chunk_size != 0) {
 		*chunkSize = (size_t)ans.chunk_size;
@@ -331,6 +431,17 @@ ncclResult_t tuner_get_chunk_size(void *context, ncclFunc_t collType, size_t nBy
 } // namespace
 
 extern "C" {
+
+int ofi_amd_tuner_ctx_stats(const void *context, ofi_amd_tuner_ctx_stats_t *out)
+{
+	auto *ctx = static_cast<const tuner_ctx *>(context);
+	if (!ctx || !out || ctx->magic != kCtxMagic) {
+		return -EINVAL;
+	}
+	std::lock_guard<std::mutex> g(const_cast<tuner_ctx *>(ctx)->lock);
+	*out = ctx->stats;
+	return 0;
+}
 
 __attribute__((visibility("default"))) ncclTuner_v3_t ncclTunerPlugin_v3 = {
 	"nccl_ofi_tuner", tuner_init, tuner_get_coll_info, tuner_destroy

@@ -71,7 +71,46 @@ staging_t g_stage;
 
 } // namespace
 
+/* stream and staging for `want` questions; the caller holds g_stage.lock */
+static int ensure_staging(uint32_t want)
+{
+	if (!g_stage.stream) {
+		OFI_AMD_HIP_TRY(hipStreamCreateWithFlags(&g_stage.stream, hipStreamNonBlocking));
+	}
+	if (want > g_stage.cap) {
+		want = want < 256 ? 256 : want;
+		void *q = nullptr, *a = nullptr;
+		OFI_AMD_HIP_TRY(hipHostMalloc(&q, sizeof(dev_query_t) * want, hipHostMallocMapped));
+		if (hipHostMalloc(&a, sizeof(ofi_amd_tuner_answer_t) * want, hipHostMallocMapped) != hipSuccess) {
+			(void)hipGetLastError();
+			(void)hipHostFree(q);
+			return -ENOMEM;
+		}
+		if (g_stage.q) (void)hipHostFree(g_stage.q);
+		if (g_stage.a) (void)hipHostFree(g_stage.a);
+		g_stage.q = static_cast<dev_query_t *>(q);
+		g_stage.a = static_cast<ofi_amd_tuner_answer_t *>(a);
+		g_stage.cap = want;
+	}
+	return 0;
+}
+
 using namespace ofi_amd;
+
+extern "C" int ofi_amd_tuner_query_prepare(uint32_t capacity)
+{
+	int rc = require_device();
+	if (rc != 0) {
+		return rc;
+	}
+	region_tables_t tables;
+	rc = device_region_tables(&tables);
+	if (rc != 0) {
+		return rc;
+	}
+	std::lock_guard<std::mutex> g(g_stage.lock);
+	return ensure_staging(capacity);
+}
 
 extern "C" int ofi_amd_tuner_query(const ofi_amd_tuner_query_t *queries, uint32_t n,
 				   ofi_amd_tuner_answer_t *answers)
@@ -103,22 +142,9 @@ extern "C" int ofi_amd_tuner_query(const ofi_amd_tuner_query_t *queries, uint32_
 	}
 
 	std::lock_guard<std::mutex> g(g_stage.lock);
-	if (!g_stage.stream) {
-		OFI_AMD_HIP_TRY(hipStreamCreateWithFlags(&g_stage.stream, hipStreamNonBlocking));
-	}
-	if (n > g_stage.cap) {
-		const uint32_t want = n < 256 ? 256 : n;
-		void *q = nullptr, *a = nullptr;
-		OFI_AMD_HIP_TRY(hipHostMalloc(&q, sizeof(dev_query_t) * want, hipHostMallocMapped));
-		if (hipHostMalloc(&a, sizeof(ofi_amd_tuner_answer_t) * want, hipHostMallocMapped) != hipSuccess) {
-			(void)hipHostFree(q);
-			return -ENOMEM;
-		}
-		if (g_stage.q) (void)hipHostFree(g_stage.q);
-		if (g_stage.a) (void)hipHostFree(g_stage.a);
-		g_stage.q = static_cast<dev_query_t *>(q);
-		g_stage.a = static_cast<ofi_amd_tuner_answer_t *>(a);
-		g_stage.cap = want;
+	rc = ensure_staging(n);
+	if (rc != 0) {
+		return rc;
 	}
 	for (uint32_t i = 0; i < n; i++) {
 		dev_query_t &d = g_stage.q[i];

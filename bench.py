@@ -83,7 +83,7 @@ def bench_bounce(lib, oracle, torch, np, args):
     stream = _gpu.stream()
 
     def step():
-        rc = lib.ofi_amd_bounce_scatter(d_src.data_ptr(), d_arena.data_ptr(), w["arena_bytes"],
+        rc = lib.ofi_amd_bounce_scatter(d_src.data_ptr(), d_src.numel(), d_arena.data_ptr(), w["arena_bytes"],
                                         d_so.data_ptr(), d_do.data_ptr(), d_len.data_ptr(), n,
                                         d_flush.data_ptr(), stream)
         if rc != 0:
@@ -362,7 +362,66 @@ def bench_tuner(lib, oracle, torch, np, args):
         out["model_speedup_vs_cpu_core"] = out["model_cells_per_s"] / out["cpu_model_cells_per_s"]
         out["region_speedup_vs_cpu_core"] = out["region_points_per_s"] / out["cpu_region_points_per_s"]
     lib.ofi_amd_tuner_plan_destroy(plan)
+    # 256 grids per launch beside the 64 above: where the model kernel ends up once the launch is long
+    # enough for its fixed costs not to count
+    nv4 = 256
+    variants4 = (m.TunerVariant * nv4)(*[m.TunerVariant(i % 2, 1 + (i // 2) % 32, 8 + i // 64, 3) for i in range(nv4)])
+    d_cost4 = torch.zeros(nv4 * cells, dtype=torch.float64, device="cuda")
+    d_choice4 = torch.zeros(nv4 * points * 2, dtype=torch.int8, device="cuda")
+    plan4 = ctypes.c_void_p()
+    m.check(lib.ofi_amd_tuner_plan_create(colls.ctypes.data, len(colls), sizes.ctypes.data, len(sizes),
+                                          nodes.ctypes.data, len(nodes), ppn.ctypes.data, len(ppn),
+                                          algos.ctypes.data, len(algos), ctypes.byref(plan4)), "plan_create")
+    _, model4_ms = timed_steps(lambda: m.check(lib.ofi_amd_tuner_model_grid(
+        plan4, variants4, nv4, d_cost4.data_ptr(), d_choice4.data_ptr(), stream), "model_grid"),
+        args.steps, args.warmup, torch)
+    out["model_256_grids_ms"] = model4_ms
+    out["model_256_grids_cells_per_s"] = nv4 * cells / model4_ms * 1e3
+    out["model_256_grids_write_gbs"] = nv4 * (cells * 8 + points * 2) / model4_ms / 1e6
+    lib.ofi_amd_tuner_plan_destroy(plan4)
+    del d_cost4, d_choice4
+    out.update(bench_tuner_plugin(lib, np))
     return out
+
+
+def bench_tuner_plugin(lib, np):
+    """getCollInfo through the NCCL plugin struct: a question that init evaluated ahead (a size on the
+    power-of-two ladder), a new question (one GPU round trip), and the same question again."""
+    import aws_ofi_nccl_amd as m
+    saved = {k: os.environ.pop(k, None) for k in ("OFI_NCCL_FORCE_PRODUCT_NAME", "OFI_NCCL_TUNER_TYPE",
+                                                  "OFI_NCCL_FORCE_NUM_RAILS")}
+    os.environ["OFI_NCCL_FORCE_PRODUCT_NAME"] = "p5en.48xlarge"
+    try:
+        v3 = m.NcclTunerV3.in_dll(lib, "ncclTunerPlugin_v3")
+        ctx = ctypes.c_void_p()
+        t0 = time.perf_counter()
+        if v3.init(64, 8, None, ctypes.byref(ctx)) != 0 or not ctx.value:
+            return {"plugin_error": "init failed"}
+        init_ms = (time.perf_counter() - t0) * 1e3
+        table = np.full((7, 3), 1337.0, dtype=np.float32)
+        nch = ctypes.c_int(0)
+
+        def ask(size):
+            table[:] = 1337.0
+            t = time.perf_counter()
+            rc = v3.getCollInfo(ctx, 4, size, 1, table.ctypes.data, 7, 3, ctypes.byref(nch))
+            return rc, (time.perf_counter() - t) * 1e6
+
+        ladder = [ask(1 << e)[1] for e in range(4, 34)]                       # evaluated by init
+        fresh = [ask((1 << e) + 12345 + 7 * e)[1] for e in range(14, 34)]      # GPU round trips
+        again = [ask((1 << e) + 12345 + 7 * e)[1] for e in range(14, 34)]      # now in the table
+        st = m.TunerCtxStats()
+        lib.ofi_amd_tuner_ctx_stats(ctx, ctypes.byref(st))
+        v3.destroy(ctx)
+        return {"plugin_init_ms": init_ms, "plugin_preloaded_questions": st.preloaded,
+                "plugin_hit_us": float(np.median(ladder + again)), "plugin_miss_us": float(np.median(fresh)),
+                "plugin_first_call_of_a_ladder_size_us": ladder[0],
+                "plugin_hits": st.hits, "plugin_misses": st.misses}
+    finally:
+        for k, v in saved.items():
+            os.environ.pop(k, None)
+            if v is not None:
+                os.environ[k] = v
 
 
 def bench_gin(lib, oracle, torch, np, args):

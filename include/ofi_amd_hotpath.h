@@ -150,14 +150,26 @@ int ofi_amd_sched_get_schedule(ofi_amd_sched_state_t *state, uint64_t size, uint
  * ====================================================================== */
 
 /*
- * For i in [0,n): copies d_len[i] bytes from d_src + d_src_off[i] to
- * d_arena + d_dst_off[i] (d_dst_off[i] 64-byte aligned, destination ranges
+ * For i in [0,n): copies d_len[i] bytes from d_src + d_src_off[i] (inside [0, src_bytes))
+ * to d_arena + d_dst_off[i] (d_dst_off[i] 64-byte aligned, destination ranges
  * disjoint, each inside [0, arena_bytes)), then, if d_flush is not NULL, reads
  * back the first 4 bytes at each destination into d_flush[i] (device or pinned
- * host memory) after the copy is visible device-wide.  No byte outside the
- * destination ranges is written.
+ * host memory; those 4 bytes must lie inside the arena also for shorter buffers).
+ * No byte outside the destination ranges is written.  A buffer that breaks a
+ * precondition is skipped and reported through ofi_amd_async_error_fetch (bit 0).
+ * n <= 2^30.
+ *
+ * Visibility: the arena bytes and the flush words are complete, for the host and for
+ * work on any stream, once the launch has completed on `stream` (an event, a stream
+ * wait, ofi_amd_flush_post queued behind it) -- as for any kernel.  d_flush[i] is
+ * written while the kernel runs, each after its own wavefront's stores, with no
+ * device-wide ordering: a value that a poller sees before the launch has completed
+ * says nothing about the arena bytes of buffer i, and must not be used as a
+ * per-buffer completion flag.  The completion that the reference's flush gives its
+ * caller (rdma_flush_req, src/nccl_ofi_rdma.cpp:2664-2713) is the sentinel flush
+ * below, queued on the same stream.
  */
-int ofi_amd_bounce_scatter(const void *d_src, void *d_arena, uint64_t arena_bytes,
+int ofi_amd_bounce_scatter(const void *d_src, uint64_t src_bytes, void *d_arena, uint64_t arena_bytes,
 			   const uint64_t *d_src_off, const uint64_t *d_dst_off,
 			   const uint32_t *d_len, uint32_t n, uint32_t *d_flush, void *stream);
 
@@ -170,7 +182,8 @@ int ofi_amd_bounce_scatter(const void *d_src, void *d_arena, uint64_t arena_byte
  * (src/nccl_ofi_rdma.cpp:2729-2776; truncation :2738-2743; zero length copies nothing,
  * :753-762).  rx_base is any device-accessible memory (pinned host rx buffers or HBM).
  * d_copied[i] (optional) receives the byte count; d_flush[i] (optional) the first
- * min(4, count) destination bytes, little-endian, read back after the copy.
+ * min(4, count) destination bytes, little-endian, read back after the copy (valid, like
+ * the copied bytes, once the launch has completed on `stream`; see above).
  */
 int ofi_amd_eager_copy_batch(const void *rx_base, const uint64_t *d_rx_off, const uint32_t *d_recv_len,
 			     void *dst_base, const uint64_t *d_dst_off, const uint32_t *d_dst_len,
@@ -713,9 +726,23 @@ typedef struct {
 	uint64_t chunk_size; /* kind 2; 0: left alone */
 } ofi_amd_tuner_answer_t; /* 16 bytes */
 
-/* Synchronous: queries and answers are host arrays. */
+/* Synchronous: queries and answers are host arrays.  The first call creates what the launches
+ * need (a private stream, pinned staging for the questions and answers, the region tables in
+ * device memory); ofi_amd_tuner_query_prepare(capacity) does that ahead of time, after which
+ * a call with n <= capacity allocates nothing (a launch and a wait on the private stream). */
+int ofi_amd_tuner_query_prepare(uint32_t capacity);
 int ofi_amd_tuner_query(const ofi_amd_tuner_query_t *queries, uint32_t n,
 			ofi_amd_tuner_answer_t *answers);
+
+/* Counters of the tuner plugin's per-communicator answer table (context = what the plugin's
+ * init returned): questions answered from the table, questions that went to the GPU, entries
+ * evaluated ahead of time by init. */
+typedef struct {
+	uint64_t hits;
+	uint64_t misses;
+	uint64_t preloaded;
+} ofi_amd_tuner_ctx_stats_t;
+int ofi_amd_tuner_ctx_stats(const void *context, ofi_amd_tuner_ctx_stats_t *out);
 
 /*
  * NCCL tuner plugin symbols, same names and struct layouts as the reference exports

@@ -53,7 +53,7 @@ def test_gpu_entry_points_fail_loudly_without_a_gpu(lib):
     assert lib.ofi_amd_gpu_init() == enodev
     p = ctypes.c_void_p()
     assert lib.ofi_amd_gpu_mem_alloc(ctypes.byref(p), 64) == enodev
-    assert lib.ofi_amd_bounce_scatter(1, 1, 64, 1, 1, 1, 1, None, None) == enodev
+    assert lib.ofi_amd_bounce_scatter(1, 64, 1, 64, 1, 1, 1, 1, None, None) == enodev
     assert lib.ofi_amd_flush_read(1, 1, 1, 1, None) == enodev
     assert lib.ofi_amd_sched_batch(1, 1, 1, 128, 1, 1, None) == enodev
     assert lib.ofi_amd_gin_rings_create(4, 256, ctypes.byref(p)) == enodev

@@ -18,7 +18,7 @@ def scatter(lib, src, arena_t, src_off, dst_off, length, flush=True):
     d_src = _gpu.to_dev(src)
     d_so, d_do, d_len = _gpu.to_dev(src_off), _gpu.to_dev(dst_off), _gpu.to_dev(length)
     d_flush = torch.full((max(n, 1),), -1, dtype=torch.int32, device="cuda")
-    rc = lib.ofi_amd_bounce_scatter(d_src.data_ptr(), arena_t.data_ptr(), arena_t.numel(),
+    rc = lib.ofi_amd_bounce_scatter(d_src.data_ptr(), d_src.numel(), arena_t.data_ptr(), arena_t.numel(),
                                     d_so.data_ptr(), d_do.data_ptr(), d_len.data_ptr(), n,
                                     d_flush.data_ptr() if flush else None, _gpu.stream())
     assert rc == 0
@@ -94,7 +94,7 @@ def test_lengths_beyond_one_trip_and_every_row_count(lib, oracle, gpu):
 
 def test_empty_batch_and_all_zero_lengths(lib, oracle, gpu):
     arena = torch.full((4096,), 9, dtype=torch.uint8, device="cuda")
-    assert lib.ofi_amd_bounce_scatter(arena.data_ptr(), arena.data_ptr(), 4096, None, None, None, 0,
+    assert lib.ofi_amd_bounce_scatter(arena.data_ptr(), 4096, arena.data_ptr(), 4096, None, None, None, 0,
                                       None, _gpu.stream()) == 0
     src = np.arange(64, dtype=np.uint8)
     flush = scatter(lib, src, arena, np.zeros(8, np.uint64), np.arange(8, dtype=np.uint64) * 64,
@@ -124,7 +124,7 @@ def test_flush_into_pinned_host_memory(lib, oracle, gpu):
     arena = torch.zeros(w["arena_bytes"], dtype=torch.uint8, device="cuda")
     d_src = _gpu.to_dev(src)
     d = [_gpu.to_dev(w[k]) for k in ("src_off", "dst_off", "len")]
-    assert lib.ofi_amd_bounce_scatter(d_src.data_ptr(), arena.data_ptr(), arena.numel(), d[0].data_ptr(),
+    assert lib.ofi_amd_bounce_scatter(d_src.data_ptr(), d_src.numel(), arena.data_ptr(), arena.numel(), d[0].data_ptr(),
                                       d[1].data_ptr(), d[2].data_ptr(), 300, dev, _gpu.stream()) == 0
     _gpu.sync()
     got = np.ctypeslib.as_array(ctypes.cast(host, ctypes.POINTER(ctypes.c_uint32)), shape=(300,)).copy()
@@ -149,6 +149,26 @@ def test_out_of_range_destination_is_skipped_and_reported(lib, gpu):
     assert np.all(got[:64] == 0xEE) and not got[64:].any()
     assert _gpu.fetch_async_errors(lib) & 1
     assert _gpu.fetch_async_errors(lib) == 0          # fetch clears
+
+
+def test_out_of_range_source_and_read_back_are_skipped_and_reported(lib, gpu):
+    """A source range outside the bounce region, and a read-back whose four bytes would lie past
+    the arena (a short buffer in its last bytes, or an empty one at its very end), are skipped."""
+    src = np.full(256, 0xEE, dtype=np.uint8)
+    for dst, soff, length, with_flush, bad in [
+            (0, 0, 256, True, False), (0, 1, 256, True, True), (0, 257, 0, True, True), (0, 256, 0, True, False),
+            (4096, 0, 0, True, True),            # empty buffer at the very end: nothing to read back from
+            (4096, 0, 0, False, False),          # ... which is fine without a read-back
+            (4096 - 64, 0, 64, True, False)]:
+        arena = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+        scatter(lib, src, arena, np.array([soff], np.uint64), np.array([dst], np.uint64),
+                np.array([length], np.uint32), flush=with_flush)
+        got = arena.cpu().numpy()
+        assert bool(_gpu.fetch_async_errors(lib) & 1) == bad, (dst, soff, length, with_flush)
+        assert int(np.count_nonzero(got)) == (0 if bad else length)
+    big = torch.zeros(8, dtype=torch.uint8, device="cuda")
+    assert lib.ofi_amd_bounce_scatter(big.data_ptr(), 8, big.data_ptr(), 8, big.data_ptr(), big.data_ptr(),
+                                      big.data_ptr(), (1 << 30) + 1, None, _gpu.stream()) == -22
 
 
 def test_full_size_configuration(lib, oracle, gpu):

@@ -86,7 +86,7 @@ def test_graph_of_hot_path_launches_replays_exactly(lib, oracle, gpu):
         assert lib.ofi_amd_copy_table(d_tsrc.data_ptr(), d_tdst.data_ptr(), d_tlen.data_ptr(), n_t, sp) == 0
         assert lib.ofi_amd_sched_batch(d_state.data_ptr(), d_sizes.data_ptr(), n_msg, 128, d_num.data_ptr(),
                                        d_xf.data_ptr(), sp) == 0
-        assert lib.ofi_amd_bounce_scatter(d_src.data_ptr(), d_arena.data_ptr(), w["arena_bytes"],
+        assert lib.ofi_amd_bounce_scatter(d_src.data_ptr(), d_src.numel(), d_arena.data_ptr(), w["arena_bytes"],
                                           d_so.data_ptr(), d_do.data_ptr(), d_len.data_ptr(), 2048,
                                           d_flush.data_ptr(), sp) == 0
         assert lib.ofi_amd_gin_signal_apply(d_work.data_ptr(), n_sig, regions, 1, None, sp) == 0

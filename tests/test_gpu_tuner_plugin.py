@@ -265,3 +265,53 @@ def test_query_heuristic_breakpoints_by_hand(lib, gpu):
     bad = [i for i in range(n) if got[i] != want[i]]
     assert not bad, [(qs[i].nbytes, qs[i].num_nodes, got[i], want[i]) for i in bad[:5]]
     assert n >= 150
+
+
+def test_init_evaluates_the_size_ladder_ahead(lib, oracle, gpu, clean_env):
+    """init prepares everything that allocates and answers the power-of-two ladder of every
+    collective in one launch: a job's first getCollInfo calls are table hits; a narrower cost table
+    that still allows the chosen cell is a hit as well; an off-ladder size goes to the GPU once."""
+    os.environ["OFI_NCCL_FORCE_PRODUCT_NAME"] = PLATFORM_NAMES[2]            # P6: regions for AR, AG, RS
+    v3 = m.NcclTunerV3.in_dll(lib, "ncclTunerPlugin_v3")
+    ctx = ctypes.c_void_p()
+    assert v3.init(64, 8, None, ctypes.byref(ctx)) == 0 and ctx.value
+    st = m.TunerCtxStats()
+    assert lib.ofi_amd_tuner_ctx_stats(ctx, ctypes.byref(st)) == 0
+    assert st.preloaded >= 5 * 37 and (st.hits, st.misses) == (0, 0)
+    a, p, ch = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    nch = ctypes.c_int(-5)
+    asked = 0
+    for coll in (4, 2, 3):
+        for e in range(0, 37):
+            table = np.full((7, 3), 1337.0, dtype=np.float32)
+            assert v3.getCollInfo(ctx, coll, 1 << e, 1, table.ctypes.data, 7, 3, ctypes.byref(nch)) == 0
+            ch.value = -5
+            oracle.oracle_region_decide(2, coll, 1 << e, 64, 8, ctypes.byref(a), ctypes.byref(p), ctypes.byref(ch))
+            zero = [(int(i), int(j)) for i, j in zip(*np.where(table == 0.0))]
+            assert zero == ([(a.value, p.value)] if a.value >= 0 else []), (coll, e)
+            asked += 1
+    assert lib.ofi_amd_tuner_ctx_stats(ctx, ctypes.byref(st)) == 0
+    assert (st.hits, st.misses) == (asked, 0)
+    # NCCL rules out a cell the answer does not use (NVLS): still the same first region -> a hit
+    table = np.full((7, 3), 1337.0, dtype=np.float32)
+    table[4, :] = -1.0
+    oracle.oracle_region_decide(2, 4, 1 << 20, 64, 8, ctypes.byref(a), ctypes.byref(p), ctypes.byref(ch))
+    assert a.value not in (-1, 4)
+    assert v3.getCollInfo(ctx, 4, 1 << 20, 1, table.ctypes.data, 7, 3, ctypes.byref(nch)) == 0
+    assert table[a.value, p.value] == 0.0
+    # ... and one that rules out the chosen cell itself has to be asked
+    table = np.full((7, 3), 1337.0, dtype=np.float32)
+    table[a.value, p.value] = -1.0
+    mask = 0x1FFFFF & ~(1 << (a.value * 3 + p.value))
+    oracle.oracle_region_decide_masked(2, 4, 1 << 20, 64, 8, mask, ctypes.byref(a), ctypes.byref(p), ctypes.byref(ch))
+    assert v3.getCollInfo(ctx, 4, 1 << 20, 1, table.ctypes.data, 7, 3, ctypes.byref(nch)) == 0
+    if a.value >= 0:
+        assert table[a.value, p.value] == 0.0
+    # off the ladder: one round trip, then a hit
+    for _ in range(2):
+        table = np.full((7, 3), 1337.0, dtype=np.float32)
+        assert v3.getCollInfo(ctx, 4, (1 << 20) + 3, 1, table.ctypes.data, 7, 3, ctypes.byref(nch)) == 0
+    assert lib.ofi_amd_tuner_ctx_stats(ctx, ctypes.byref(st)) == 0
+    assert (st.hits, st.misses) == (asked + 2, 2)
+    assert v3.destroy(ctx) == 0
+    assert lib.ofi_amd_tuner_ctx_stats(None, ctypes.byref(st)) == -22
