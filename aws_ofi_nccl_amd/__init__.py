@@ -319,6 +319,7 @@ PROTOTYPES = {
     "ofi_amd_gin_rings_device_view": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(GinDevRing)]),
     "ofi_amd_gin_produce_table": (ctypes.c_int, [c_vp, c_vp, c_u64, c_u32, c_u64, c_vp]),
     "ofi_amd_gin_producer_status": (ctypes.c_int, [c_vp]),
+    "ofi_amd_gin_rings_reset": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(c_u64)]),
     "ofi_amd_gin_ring_push": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(GinDesc)]),
     "ofi_amd_gin_ring_pop": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(GinDesc)]),
     "ofi_amd_gin_comm_init": (ctypes.c_int, [ctypes.POINTER(GinComm), c_u32, c_u32, c_u64, c_u64,

@@ -303,6 +303,44 @@ int ofi_amd_gin_rings_create(uint32_t n_contexts, uint32_t capacity, ofi_amd_gin
 	return 0;
 }
 
+int ofi_amd_gin_rings_reset(ofi_amd_gin_rings_t *r, uint32_t context, uint64_t *dropped)
+{
+	if (!r || (context != OFI_AMD_GIN_ALL_CONTEXTS && context >= r->n_contexts)) {
+		return -EINVAL;
+	}
+	const uint32_t first = context == OFI_AMD_GIN_ALL_CONTEXTS ? 0 : context;
+	const uint32_t last = context == OFI_AMD_GIN_ALL_CONTEXTS ? r->n_contexts : context + 1;
+	const uint32_t cap = r->capacity, mask = cap - 1;
+	uint64_t lost = 0;
+	for (uint32_t c = first; c < last; c++) {
+		/* everything from the consumer's position on is handed back to the producers: slot of
+		 * position p free for p, whatever a producer that gave up left in it */
+		const uint32_t base = r->dequeue_pos[c];
+		uint32_t *seq = r->sequences + (size_t)c * cap;
+		for (uint32_t k = 0; k < cap; k++) {
+			const uint32_t pos = base + k;
+			if (seq[pos & mask] == pos + 1u) {
+				lost++; /* published, never popped */
+			}
+			seq[pos & mask] = pos;
+		}
+		__atomic_store_n(&r->enqueue_pos[c * 16], base, __ATOMIC_RELAXED);
+		/* cursor back to the consumer's position; every slot is free, so the horizon is a
+		 * whole lap ahead and the next producers need not look over the host link */
+		const uint32_t cursor[2] = { base, base + cap };
+		OFI_AMD_HIP_TRY(hipMemcpy(r->d_reserve + (size_t)c * kGinReserveStride, cursor, sizeof(cursor),
+					  hipMemcpyHostToDevice));
+	}
+	if (context == OFI_AMD_GIN_ALL_CONTEXTS) {
+		__atomic_store_n(r->status, 0u, __ATOMIC_RELAXED);
+	}
+	__atomic_thread_fence(__ATOMIC_SEQ_CST);
+	if (dropped) {
+		*dropped = lost;
+	}
+	return 0;
+}
+
 int ofi_amd_gin_rings_view(ofi_amd_gin_rings_t *r, void **records, uint32_t **sequences,
 			   uint32_t *n_contexts, uint32_t *capacity)
 {

@@ -23,7 +23,8 @@
  * Wave-collective: all 64 lanes of the wavefront call it together (no divergence around
  * the call); lanes with active == true each put *desc.  Returns 0, or -1 when the ring
  * stayed full for spin_limit polls -- the timeout bit is then set in the ring's status word
- * and the reserved slots are never published, so the ring must not be used any further.
+ * and the reserved slots are never published, so the ring must not be used any further
+ * until the host has reset it (ofi_amd_gin_rings_reset, once the kernel has ended).
  *
  * The wave's descriptors take consecutive positions in lane order: one atomic add on the
  * device-resident cursor per call (not per descriptor, and nothing atomic over the host

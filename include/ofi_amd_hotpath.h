@@ -264,6 +264,21 @@ typedef struct ofi_amd_gin_rings ofi_amd_gin_rings_t;
  * pinned host memory: record array (64 B each) + sequence array (u32 each). */
 int ofi_amd_gin_rings_create(uint32_t n_contexts, uint32_t capacity, ofi_amd_gin_rings_t **out);
 int ofi_amd_gin_rings_destroy(ofi_amd_gin_rings_t *rings);
+/*
+ * Recovery after a producer gave up on a full ring (ofi_amd_gin_producer_status -ETIMEDOUT;
+ * the reference never gives up: await_tx_window, src/rdma/gin/nccl_ofi_gin.cpp:518-537, blocks
+ * and carries on, which a kernel that must end cannot).  To be called by the consumer's thread
+ * once every producing kernel has ended (the streams are synchronised) and no push or drain is
+ * running: the ring of `context` -- or every ring, OFI_AMD_GIN_ALL_CONTEXTS -- restarts at the
+ * consumer's position: records published but not popped are dropped (*dropped, optional, counts
+ * them), slots reserved by producers that gave up are free again, and the cursors of GPU and
+ * host producers and the GPU producers' horizon are set accordingly.  Which ring a producer
+ * gave up on is not recorded, so after a reported time-out reset all of them; only that form
+ * clears the status ofi_amd_gin_producer_status reports.  The producers re-issue what they
+ * could not put; what the consumer had popped before stays delivered.
+ */
+#define OFI_AMD_GIN_ALL_CONTEXTS 0xffffffffu
+int ofi_amd_gin_rings_reset(ofi_amd_gin_rings_t *rings, uint32_t context, uint64_t *dropped);
 /* Raw views for tests / external consumers (host addresses of pinned memory). */
 int ofi_amd_gin_rings_view(ofi_amd_gin_rings_t *rings, void **records, uint32_t **sequences,
 			   uint32_t *n_contexts, uint32_t *capacity);

@@ -348,6 +348,54 @@ def test_host_push_pop_ring_behaviour(lib, gpu):
     lib.ofi_amd_gin_rings_destroy(rings)
 
 
+def test_rings_recover_from_a_producer_timeout(lib, oracle, gpu):
+    """A time-out forced from the host (no consumer, a tiny spin limit: every wave leaves after its
+    bounded wait), then ofi_amd_gin_rings_reset, then bit-exact streams on the same rings -- from
+    the seeded generator and from several waves per ring through the general device put.  The
+    rings restart at the consumer's position, which is not 0 for the ring that had been drained
+    in part."""
+    nctx, cap = 3, 256
+    rings = make_rings(lib, nctx, cap)
+    assert lib.ofi_amd_gin_produce_seeded(rings, SEED, 1000, 1, 64, 1, 1, 50, _gpu.stream()) == 0
+    _gpu.sync()
+    assert lib.ofi_amd_gin_producer_status(rings) == -errno.ETIMEDOUT
+    # pop 100 records of ring 1 by hand: its consumer position moves, the other rings' do not
+    d = m.GinDesc()
+    for _ in range(100):
+        assert lib.ofi_amd_gin_ring_pop(rings, 1, ctypes.byref(d)) == 1
+    dropped = ctypes.c_uint64()
+    assert lib.ofi_amd_gin_rings_reset(rings, 7, None) == -22
+    assert lib.ofi_amd_gin_rings_reset(rings, 0, ctypes.byref(dropped)) == 0 and dropped.value == 256
+    assert lib.ofi_amd_gin_producer_status(rings) == -errno.ETIMEDOUT      # one ring alone does not clear it
+    assert lib.ofi_amd_gin_rings_reset(rings, 0xFFFFFFFF, ctypes.byref(dropped)) == 0
+    assert dropped.value == 156 + 256                                      # ring 0 was already clean
+    assert lib.ofi_amd_gin_producer_status(rings) == 0
+    assert lib.ofi_amd_gin_ring_pop(rings, 1, ctypes.byref(d)) == 0        # nothing left in the rings
+
+    ops = 5000
+    rc, stats, descs, _ = produce_and_drain(lib, rings, nctx, ops, mode=1)
+    assert rc == 0 and lib.ofi_amd_gin_producer_status(rings) == 0
+    got = np.frombuffer(descs, dtype=np.uint64).reshape(nctx, ops, 8)
+    assert np.array_equal(got, oracle_stream(oracle, nctx, ops, 64, 1, 1))
+    # the general device put on the same rings: one wave per ring keeps the table order
+    rng = np.random.default_rng(4)
+    table = rng.integers(0, 1 << 62, (nctx, 3000, 8), dtype=np.uint64)
+    d_table = _gpu.to_dev(table)
+    assert lib.ofi_amd_gin_produce_table(rings, d_table.data_ptr(), 3000, 1, 0, _gpu.stream()) == 0
+    rc, _stats, got = drain_descs(lib, rings, nctx, 3000)
+    assert rc == 0 and np.array_equal(got, table)
+    # a second time-out and reset on the same rings, then host producers
+    assert lib.ofi_amd_gin_produce_table(rings, d_table.data_ptr(), 3000, 3, 50, _gpu.stream()) == 0
+    _gpu.sync()
+    assert lib.ofi_amd_gin_producer_status(rings) == -errno.ETIMEDOUT
+    assert lib.ofi_amd_gin_rings_reset(rings, 0xFFFFFFFF, None) == 0
+    one = m.GinDesc(1, 2, 3, 4, 5, 6, 0, 0, 2, 0, 1, 0xFFFF, 1)
+    assert lib.ofi_amd_gin_ring_push(rings, 2, ctypes.byref(one)) == 1
+    assert lib.ofi_amd_gin_ring_pop(rings, 2, ctypes.byref(d)) == 1 and bytes(d) == bytes(one)
+    assert lib.ofi_amd_gin_ring_pop(rings, 2, ctypes.byref(d)) == 0
+    lib.ofi_amd_gin_rings_destroy(rings)
+
+
 def test_host_producers_threaded(lib, gpu):
     """Four CPU producer threads on one ring, the proxy loop as consumer (mpsc_ring.cpp:134-189):
     per-producer FIFO, no loss, no duplicate."""
