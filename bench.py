@@ -167,17 +167,26 @@ def bench_bounce(lib, oracle, torch, np, args):
         region = ctypes.c_void_p()
         m.check(lib.ofi_amd_devcopy_register(d_arena.data_ptr(), w["arena_bytes"], ctypes.byref(region)),
                 "devcopy_register")
-        t0 = time.perf_counter()
-        for i in range(sample):
-            rc = lib.ofi_amd_devcopy_to_device(src.ctypes.data + int(w["src_off"][i]), region,
-                                               int(w["dst_off"][i]), int(w["len"][i]))
-            if rc != 0:
-                raise RuntimeError("devcopy_to_device: %d" % rc)
-        per_call_s = time.perf_counter() - t0
+        # plain Python ints ahead of the loop: the loop should time the calls, not numpy scalar conversions
+        calls = list(zip((w["src_off"][:sample].astype(np.int64) + src.ctypes.data).tolist(),
+                         w["dst_off"][:sample].tolist(), w["len"][:sample].tolist()))
+        to_device = lib.ofi_amd_devcopy_to_device
+        # two passes over the same buffers: the first touches each page of the CPU mapping of the arena
+        # for the first time (a page fault each), the second is what a caller that reuses its
+        # registered buffers, as the plugin does, sees
+        passes = []
+        for _ in range(2):
+            t0 = time.perf_counter()
+            for src_addr, dst, length in calls:
+                if to_device(src_addr, region, dst, length) != 0:
+                    raise RuntimeError("devcopy_to_device failed")
+            passes.append(time.perf_counter() - t0)
+        first_pass_s, per_call_s = passes
         lib.ofi_amd_devcopy_deregister(region)
         out["per_buffer_copy_calls"] = {
             "value": float(w["len"][:sample].sum()) / per_call_s / 1e9, "unit": "GB/s payload",
-            "buffers_per_s": sample / per_call_s, "sample": "%d buffers, one host-to-device call each" % sample}
+            "buffers_per_s": sample / per_call_s, "buffers_per_s_first_touch": sample / first_pass_s,
+            "sample": "%d buffers, one host-to-device call each (CPU stores through the BAR mapping)" % sample}
     del d_arena, d_src, d_tmp
     torch.cuda.empty_cache()
     return out, cpu

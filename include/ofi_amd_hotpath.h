@@ -223,8 +223,16 @@ int ofi_amd_flush_buffer_fill(void *d_flush_buf, uint64_t sentinel, void *stream
 int ofi_amd_flush_post(const void *d_flush_buf, void *slots_dev, uint32_t num_rails, void *stream);
 int ofi_amd_flush_test(const void *slots_host, uint32_t num_rails, uint64_t sentinel);
 
-/* nccl_ofi_device_copy, include/nccl_ofi_device_copy.h:14-69: register a device
- * region, then small synchronous host<->device copies at an offset. */
+/* nccl_ofi_device_copy, include/nccl_ofi_device_copy.h:14-69: register a device region, then
+ * small synchronous host<->device copies at an offset, done by the CPU through a mapping of
+ * the device memory as GDRCopy does (src/nccl_ofi_gdrcopy.cpp:108-179).  On a large-BAR
+ * system (hipDeviceAttributeIsLargeBar) device memory is CPU-addressable at its device
+ * address, which is the mapping; register returns -ENOTSUP where it is not -- there is no
+ * second path.  copy_to_device up to 2 MiB is CPU stores plus a store fence (0.2-0.4 us up to
+ * a page, 20 GB/s beyond), copy_from_device up to 256 bytes CPU loads (2.5 us per 64 bytes);
+ * larger copies, where the copy engine wins, go through it.  As with GDRCopy, neither call
+ * waits for GPU work: a store is seen by work submitted after the call returns, a load sees
+ * the results of work that has completed. */
 typedef struct ofi_amd_devcopy_region ofi_amd_devcopy_region_t;
 int ofi_amd_devcopy_register(void *device_ptr, size_t size, ofi_amd_devcopy_region_t **out);
 int ofi_amd_devcopy_to_device(const void *host_ptr, ofi_amd_devcopy_region_t *h, size_t offset,

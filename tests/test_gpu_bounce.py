@@ -216,6 +216,48 @@ def test_device_copy_interface(lib, gpu):
     assert lib.ofi_amd_devcopy_register(host.ctypes.data, 16, ctypes.byref(h)) < 0   # not device memory
 
 
+def test_device_copy_is_ordered_with_gpu_work(lib, gpu):
+    """The copies are CPU stores and loads through the mapping of device memory (no copy engine, no
+    stream): a store is seen by a kernel launched after the call returns, a load sees what a
+    kernel that has completed wrote -- for every size class (CPU path and copy-engine path) and at
+    odd offsets."""
+    size = 8 << 20
+    buf = torch.zeros(size, dtype=torch.uint8, device="cuda")
+    h = ctypes.c_void_p()
+    assert lib.ofi_amd_devcopy_register(buf.data_ptr(), size, ctypes.byref(h)) == 0
+    rng = np.random.default_rng(7)
+    for n, off in [(1, 3), (8, 8), (63, 1), (64, 64), (255, 5), (256, 0), (257, 11), (4096, 4097),
+                   (65537, 99), (2 << 20, 7), ((2 << 20) + 1, 13), (3 << 20, 1 << 20)]:
+        data = rng.integers(0, 256, n, dtype=np.uint8)
+        assert lib.ofi_amd_devcopy_to_device(data.ctypes.data, h, off, n) == 0
+        # a kernel launched now reads the bytes and writes their complement next to them
+        out = (buf[off:off + n] ^ 0xFF).clone()
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), data ^ 0xFF), (n, off)
+        buf[off:off + n] = out                       # a kernel writes the region ...
+        torch.cuda.synchronize()
+        back = np.zeros(n, dtype=np.uint8)
+        assert lib.ofi_amd_devcopy_from_device(h, off, back.ctypes.data, n) == 0   # ... and the load sees it
+        assert np.array_equal(back, data ^ 0xFF), (n, off)
+        # nothing around the range was touched
+        assert int(buf[:off].sum()) + int(buf[off + n:].sum()) == 0
+        buf.zero_()
+        torch.cuda.synchronize()
+    # a signal counter updated from the host the way the reference's GDRCopy worker does
+    # (read-modify-write of 8 bytes, src/rdma/gin/nccl_ofi_gin.cpp:1193-1256)
+    cnt = torch.zeros(8, dtype=torch.int64, device="cuda")
+    assert lib.ofi_amd_devcopy_deregister(h) == 0
+    assert lib.ofi_amd_devcopy_register(cnt.data_ptr(), 64, ctypes.byref(h)) == 0
+    word = np.zeros(1, dtype=np.uint64)
+    for k in range(100):
+        assert lib.ofi_amd_devcopy_from_device(h, 24, word.ctypes.data, 8) == 0
+        word[0] += 3
+        assert lib.ofi_amd_devcopy_to_device(word.ctypes.data, h, 24, 8) == 0
+    torch.cuda.synchronize()
+    assert cnt.cpu().tolist() == [0, 0, 0, 300, 0, 0, 0, 0]
+    assert lib.ofi_amd_devcopy_deregister(h) == 0
+
+
 def test_gpu_glue(lib, gpu):
     p = ctypes.c_void_p()
     assert lib.ofi_amd_gpu_mem_alloc(ctypes.byref(p), 1 << 20) == 0
