@@ -92,6 +92,8 @@ __global__ __launch_bounds__(256) void model_grid_kernel(grid_dims_t g,
 	}
 }
 
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
 constexpr int kMaxSetPolys = 8;  /* polygons of one (platform, shape, collective) set */
 constexpr int kMaxSetVerts = 64; /* their vertices together */
 constexpr uint32_t kRegionBlock = 64; /* threads per workgroup of the region kernel: one wavefront */
@@ -99,12 +101,16 @@ static_assert(kRegionBlock >= (uint32_t)kMaxSetVerts && kRegionBlock >= (uint32_
 	      "one thread per staged vertex and per staged polygon word");
 
 /*
- * One thread per point; blockIdx.y is the platform entry.  A workgroup works on one (collective,
- * ranks per node) pair -- `blocks_per_run` workgroups share the pair's n_sizes x n_nodes points,
- * node count fastest -- because the polygon set depends on that pair alone: the set (at most 8
- * polygons, 64 vertices, with their bounds) is copied into LDS once and every lane then walks
- * the same polygons out of LDS instead of chasing them through global memory, and workgroups of
- * pairs without regions leave after one table lookup.
+ * One thread per (collective, size, node count); blockIdx.y is the platform entry.  A workgroup
+ * works on one collective -- `blocks_per_run` workgroups share its n_sizes x n_nodes points, node
+ * count fastest -- and takes the ranks-per-node values in turn, because the polygon set depends
+ * on the (collective, ranks per node) pair alone: for each pair the set (at most 8 polygons, 64
+ * vertices, with their bounds) is copied into LDS once and every lane then walks the same
+ * polygons out of LDS instead of chasing them through global memory; pairs without regions cost
+ * one table lookup.  A thread ends up with the decisions of all ranks-per-node values of its
+ * point, which are neighbours in the output: it writes them as one 16-byte store per four (the
+ * wavefront then writes 1 KiB contiguous), where a thread per output record had written 4 bytes
+ * at a 16-byte stride -- four times the write traffic for the same records.
  */
 __global__ __launch_bounds__(kRegionBlock) void region_choice_kernel(grid_dims_t g, region_tables_t t,
 							    const int32_t *__restrict__ platforms,
@@ -115,58 +121,70 @@ __global__ __launch_bounds__(kRegionBlock) void region_choice_kernel(grid_dims_t
 	__shared__ double s_bounds[kMaxSetPolys * 4];
 	__shared__ pt_t s_verts[kMaxSetVerts];
 
-	/* Workgroups go to the eight XCDs in turn, and the pairs that have regions sit at a fixed
-	 * period in the run index: taken in launch order, all the long-running workgroups would land
-	 * on the same few XCDs.  `spread` is coprime to the grid width, so this is a permutation
-	 * that scatters every period over all XCDs. */
+	/* Workgroups go to the eight XCDs in turn, and collectives with many regions sit at a fixed
+	 * period in the run index: taken in launch order, the long-running workgroups would land on
+	 * the same few XCDs.  `spread` is coprime to the grid width, so this is a permutation that
+	 * scatters every period over all XCDs. */
 	const uint32_t block = (uint32_t)(((uint64_t)blockIdx.x * spread) % gridDim.x);
-	const uint32_t run = block / blocks_per_run;
-	const uint32_t in_run = (block - run * blocks_per_run) * kRegionBlock + threadIdx.x;
-	const uint32_t pi = run % g.n_ppn;
-	const uint32_t ci = run / g.n_ppn;
+	const uint32_t ci = block / blocks_per_run;
+	const uint32_t in_run = (block - ci * blocks_per_run) * kRegionBlock + threadIdx.x;
 	const int platform = platforms[blockIdx.y];
 	const int coll = g.colls[ci];
-	const uint32_t ppn = g.ppn[pi];
-
-	/* ranks = nodes * ppn with nodes >= 1: the shape is a function of ppn */
-	int first, count;
-	region_set(t, platform, coll, ppn, 1, first, count);
-	if (count > 0) {
-		const int v0 = t.poly[first * 4 + 2];
-		const int v_end = t.poly[(first + count - 1) * 4 + 2] + t.poly[(first + count - 1) * 4 + 3];
-		if ((int)threadIdx.x < count * 4) {
-			const int32_t w = t.poly[first * 4 + threadIdx.x];
-			s_poly[threadIdx.x] = (threadIdx.x & 3u) == 2u ? w - v0 : w; /* vertex index within the set */
-			s_bounds[threadIdx.x] = t.bbox[first * 4 + threadIdx.x];
-		}
-		if ((int)threadIdx.x < v_end - v0) {
-			s_verts[threadIdx.x] = t.verts[v0 + threadIdx.x];
-		}
-		__syncthreads();
-	}
-	if (in_run >= g.n_sizes * g.n_nodes) {
-		return;
-	}
-	const uint32_t ni = in_run % g.n_nodes;
-	const uint32_t si = in_run / g.n_nodes;
-	const uint32_t p = ((ci * g.n_sizes + si) * g.n_nodes + ni) * g.n_ppn + pi; /* output order */
-
+	const bool live = in_run < g.n_sizes * g.n_nodes;
+	const uint32_t ni = live ? in_run % g.n_nodes : 0;
+	const uint32_t si = live ? in_run / g.n_nodes : 0;
 	const uint64_t nodes = g.nodes[ni];
-	int algorithm = -1, protocol = -1, nchannels = -1;
-	if (count > 0 && nodes > 2) {
-		int a, pr;
-		const pt_t at = { g.log2_sizes[si], g.log2_ranks[ni * g.n_ppn + pi] };
-		if (region_pick(s_poly, s_bounds, s_verts, count, at, kAllAllowed, t.far_point, a, pr) >= 0) {
-			algorithm = a;
-			protocol = pr;
-			nchannels = region_channels(platform, g.sizes[si], nodes * ppn, nodes, a, pr);
+	const uint64_t first_record = (uint64_t)blockIdx.y * points_per_platform +
+				      (uint64_t)((ci * g.n_sizes + si) * g.n_nodes + ni) * g.n_ppn;
+	uint32_t *out = reinterpret_cast<uint32_t *>(choice) + first_record;
+	const bool wide = (reinterpret_cast<uintptr_t>(choice) & 15u) == 0 && (first_record & 3u) == 0;
+
+	uint32_t group[4];
+	for (uint32_t pi = 0; pi < g.n_ppn; pi++) {
+		const uint32_t ppn = g.ppn[pi];
+		/* ranks = nodes * ppn with nodes >= 1: the shape is a function of ppn */
+		int first, count;
+		region_set(t, platform, coll, ppn, 1, first, count);
+		if (count > 0) {
+			__syncthreads(); /* the previous pair's set is no longer being read */
+			const int v0 = t.poly[first * 4 + 2];
+			const int v_end = t.poly[(first + count - 1) * 4 + 2] + t.poly[(first + count - 1) * 4 + 3];
+			if ((int)threadIdx.x < count * 4) {
+				const int32_t w = t.poly[first * 4 + threadIdx.x];
+				s_poly[threadIdx.x] = (threadIdx.x & 3u) == 2u ? w - v0 : w; /* vertex index within the set */
+				s_bounds[threadIdx.x] = t.bbox[first * 4 + threadIdx.x];
+			}
+			if ((int)threadIdx.x < v_end - v0) {
+				s_verts[threadIdx.x] = t.verts[v0 + threadIdx.x];
+			}
+			__syncthreads();
+		}
+		int algorithm = -1, protocol = -1, nchannels = -1;
+		if (live && count > 0 && nodes > 2) {
+			int a, pr;
+			const pt_t at = { g.log2_sizes[si], g.log2_ranks[ni * g.n_ppn + pi] };
+			if (region_pick(s_poly, s_bounds, s_verts, count, at, kAllAllowed, t.far_point, a, pr) >= 0) {
+				algorithm = a;
+				protocol = pr;
+				nchannels = region_channels(platform, g.sizes[si], nodes * ppn, nodes, a, pr);
+			}
+		}
+		/* {int8 algorithm, int8 protocol, int16 nchannels} */
+		group[pi & 3u] = ((uint32_t)(uint8_t)(int8_t)algorithm) | ((uint32_t)(uint8_t)(int8_t)protocol << 8) |
+				 ((uint32_t)(uint16_t)(int16_t)nchannels << 16);
+		const bool group_full = (pi & 3u) == 3u;
+		if (live && (group_full || pi == g.n_ppn - 1)) {
+			const uint32_t g0 = pi & ~3u;
+			if (group_full && wide) {
+				u32x4_t v = { group[0], group[1], group[2], group[3] };
+				*reinterpret_cast<u32x4_t *>(out + g0) = v;
+			} else {
+				for (uint32_t k = g0; k <= pi; k++) {
+					out[k] = group[k & 3u];
+				}
+			}
 		}
 	}
-	const uint64_t idx = (uint64_t)blockIdx.y * points_per_platform + p;
-	/* {int8 algorithm, int8 protocol, int16 nchannels} as one 4-byte store */
-	reinterpret_cast<uint32_t *>(choice)[idx] = ((uint32_t)(uint8_t)(int8_t)algorithm) |
-						     ((uint32_t)(uint8_t)(int8_t)protocol << 8) |
-						     ((uint32_t)(uint16_t)(int16_t)nchannels << 16);
 }
 
 /* ---- host side: building the log2-space polygon tables ---- */
@@ -572,7 +590,7 @@ int ofi_amd_tuner_region_grid(ofi_amd_tuner_plan_t *plan, const int32_t *platfor
 	const uint32_t points = (uint32_t)plan->points;
 	const uint64_t run_len = (uint64_t)plan->g.n_sizes * plan->g.n_nodes;
 	const uint64_t blocks_per_run = (run_len + kRegionBlock - 1) / kRegionBlock;
-	const uint64_t blocks = blocks_per_run * plan->g.n_colls * plan->g.n_ppn;
+	const uint64_t blocks = blocks_per_run * plan->g.n_colls;
 	if (blocks == 0 || blocks > 0x7fffffffull) {
 		return -EINVAL;
 	}
