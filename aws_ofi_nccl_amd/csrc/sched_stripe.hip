@@ -46,9 +46,16 @@ constexpr uint32_t kThreads = 256;
 constexpr uint32_t kPassesSmall = 2, kPassesLarge = 8;
 constexpr uint64_t kSmallBatch = 1ull << 21;
 constexpr uint32_t kScanThreads = 1024;
+constexpr uint32_t kScanPer = 8; /* tiles per thread and round of the scan kernel */
 constexpr uint64_t kMaxBatch = 1ull << 28;
 /* residues are < 4, so packed 16-bit sums over this many tiles cannot overflow */
-constexpr uint32_t kInlineTiles = 4096;
+#ifndef OFI_STRIPE_INLINE_TILES
+#define OFI_STRIPE_INLINE_TILES 4096
+#endif
+constexpr uint32_t kInlineTiles = OFI_STRIPE_INLINE_TILES;
+#ifndef OFI_STRIPE_NT_STORES
+#define OFI_STRIPE_NT_STORES 1
+#endif
 
 struct params_t {
 	uint64_t max_small;
@@ -57,6 +64,8 @@ struct params_t {
 	int32_t min_stripe_shift; /* log2 when a power of two, else -1 */
 	int32_t align_shift;
 	uint32_t num_rails;
+	uint32_t stripe_counts; /* get_num_stripes for this rail count, 4 bits per requested count 1..4 */
+	uint32_t mod_magic;     /* 65536 / num_rails + 1, see mod_rails */
 };
 
 __device__ __forceinline__ uint64_t div_by(uint64_t x, uint64_t d, int32_t shift)
@@ -70,18 +79,23 @@ __device__ __forceinline__ uint64_t div_ceil_by(uint64_t x, uint64_t d, int32_t 
 	return x == 0 ? 0 : 1 + div_by(x - 1, d, shift);
 }
 
-/* get_num_stripes, src/nccl_ofi_scheduler.cpp:47-64 */
+/* get_num_stripes, src/nccl_ofi_scheduler.cpp:47-64: the request, capped to the rail count,
+ * goes down to the largest count >= 2 that divides the rail count and stays as it is when there
+ * is none (3 rails: 2 stays 2).  At most 4 rails, so the loop is a 16-entry table. */
+constexpr uint64_t kStripeCounts = 0x4221332122211111ull; /* 16 bits per rail count, 4 per request */
+
 __device__ __forceinline__ uint32_t num_stripes(uint64_t size, const params_t &p)
 {
 	uint64_t want = div_ceil_by(size, p.min_stripe, p.min_stripe_shift);
 	uint32_t n = (uint32_t)(want < p.num_rails ? want : p.num_rails);
 	n = n > 1 ? n : 1;
-	for (uint32_t i = n; i > 1; i--) {
-		if ((p.num_rails % i) == 0) {
-			return i;
-		}
-	}
-	return n;
+	return (p.stripe_counts >> (4u * (n - 1u))) & 7u;
+}
+
+/* x mod num_rails for x < 16384, by multiply and shift (checked exhaustively for 1..4 rails) */
+__device__ __forceinline__ uint32_t mod_rails(uint32_t x, const params_t &p)
+{
+	return x - p.num_rails * ((x * p.mod_magic) >> 16);
 }
 
 /* Thresholds come from the device-resident state; a power-of-two divisor becomes a
@@ -100,18 +114,9 @@ __device__ __forceinline__ bool load_params(const ofi_amd_sched_state_t *st, uin
 	p.min_stripe_shift = log2_if_pow2_dev(p.min_stripe);
 	p.align_shift = log2_if_pow2_dev(align);
 	p.num_rails = (uint32_t)st->num_rails;
+	p.stripe_counts = (uint32_t)(kStripeCounts >> (16u * ((p.num_rails - 1u) & 3u))) & 0xffffu;
+	p.mod_magic = 65536u / (p.num_rails ? p.num_rails : 1u) + 1u;
 	return st->num_rails >= 1 && st->num_rails <= OFI_AMD_MAX_NUM_RAILS && p.min_stripe != 0;
-}
-
-/* x / k for k in 1..4 without a general 64-bit division */
-__device__ __forceinline__ uint64_t div_small(uint64_t x, uint32_t k)
-{
-	switch (k) {
-	case 1: return x;
-	case 2: return x >> 1;
-	case 3: return x / 3;
-	default: return x >> 2;
-	}
 }
 
 /* packed (small count << 16 | stripe count) contribution of one message */
@@ -125,15 +130,17 @@ __device__ __forceinline__ uint32_t contribution(uint64_t size, const params_t &
 	return n_out;
 }
 
-__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, uint32_t lane)
+/* Inclusive sum over the 64 lanes with lane-to-lane moves inside the vector unit: shifts by 1,
+ * 2, 4 and 8 lanes within each row of 16 (a lane shifted in from outside the row reads 0), then
+ * lane 15 of rows 0 and 2 added to rows 1 and 3, then lane 31 added to rows 2 and 3. */
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, uint32_t)
 {
-#pragma unroll
-	for (uint32_t d = 1; d < 64; d <<= 1) {
-		uint32_t up = __shfl_up(v, d, 64);
-		if (lane >= d) {
-			v += up;
-		}
-	}
+	v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, false); /* row_shr:1 */
+	v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, false); /* row_shr:2 */
+	v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, false); /* row_shr:4 */
+	v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, false); /* row_shr:8 */
+	v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false); /* row_bcast:15 */
+	v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false); /* row_bcast:31 */
 	return v;
 }
 
@@ -144,6 +151,15 @@ __global__ __launch_bounds__(kThreads) void stripe_count_kernel(
 	uint32_t *__restrict__ err)
 {
 	__shared__ uint32_t wave_sum[kThreads / 64];
+	/* the tile's sizes are requested before anything waits for the state, so a workgroup pays
+	 * one memory latency, not two */
+	const uint32_t base = blockIdx.x * (kThreads * PASSES);
+	uint64_t size_of[PASSES];
+#pragma unroll
+	for (uint32_t pass = 0; pass < PASSES; pass++) {
+		const uint32_t i = base + pass * kThreads + threadIdx.x;
+		size_of[pass] = i < n ? sizes[i] : 0;
+	}
 	params_t p;
 	if (!load_params(state, align, p)) {
 		if (blockIdx.x == 0 && threadIdx.x == 0) {
@@ -154,15 +170,12 @@ __global__ __launch_bounds__(kThreads) void stripe_count_kernel(
 	if (blockIdx.x == 0 && threadIdx.x == 0) {
 		*seed0 = ((state->rr_small_counter % p.num_rails) << 16) | (state->rr_counter % p.num_rails);
 	}
-	const uint32_t base = blockIdx.x * (kThreads * PASSES);
 	uint32_t acc = 0;
 #pragma unroll
 	for (uint32_t pass = 0; pass < PASSES; pass++) {
-		uint32_t i = base + pass * kThreads + threadIdx.x;
-		if (i < n) {
-			uint32_t k;
-			acc += contribution(sizes[i], p, k);
-		}
+		uint32_t k;
+		const uint32_t c = contribution(size_of[pass], p, k);
+		acc += base + pass * kThreads + threadIdx.x < n ? c : 0u;
 	}
 #pragma unroll
 	for (uint32_t d = 32; d > 0; d >>= 1) {
@@ -200,10 +213,29 @@ __global__ __launch_bounds__(kScanThreads) void stripe_scan_kernel(
 	uint32_t carry_small = state->rr_small_counter % num_rails;
 	uint32_t carry_big = state->rr_counter % num_rails;
 
-	for (uint32_t start = 0; start < num_tiles; start += kScanThreads) {
-		uint32_t t = start + threadIdx.x;
-		uint32_t packed = t < num_tiles ? tile_totals[t] : 0;
-		uint32_t s = packed >> 16, b = packed & 0xffffu;
+	/* eight consecutive tiles per thread and round: 16 M messages are one round, so the kernel
+	 * waits for memory once */
+	for (uint32_t start = 0; start < num_tiles; start += kScanThreads * kScanPer) {
+		const uint32_t t0 = start + threadIdx.x * kScanPer;
+		const bool whole = t0 + kScanPer <= num_tiles;
+		uint32_t v[kScanPer];
+		if (whole) {
+			const u32x4 lo = *reinterpret_cast<const u32x4 *>(tile_totals + t0);
+			const u32x4 hi = *reinterpret_cast<const u32x4 *>(tile_totals + t0 + 4);
+			v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w;
+			v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+		} else {
+#pragma unroll
+			for (uint32_t j = 0; j < kScanPer; j++) {
+				v[j] = t0 + j < num_tiles ? tile_totals[t0 + j] : 0;
+			}
+		}
+		uint32_t s = 0, b = 0;
+#pragma unroll
+		for (uint32_t j = 0; j < kScanPer; j++) {
+			s += v[j] >> 16;
+			b += v[j] & 0xffffu;
+		}
 		uint32_t inc_s = wave_inclusive_scan(s, lane);
 		uint32_t inc_b = wave_inclusive_scan(b, lane);
 		if (lane == 63) {
@@ -221,10 +253,25 @@ __global__ __launch_bounds__(kScanThreads) void stripe_scan_kernel(
 			tot_s += ws;
 			tot_b += wb;
 		}
-		if (t < num_tiles) {
-			uint32_t ex_s = (carry_small + off_s + inc_s - s) % num_rails;
-			uint32_t ex_b = (carry_big + off_b + inc_b - b) % num_rails;
-			tile_prefix[t] = (ex_s << 16) | ex_b;
+		uint32_t run_s = carry_small + off_s + inc_s - s;
+		uint32_t run_b = carry_big + off_b + inc_b - b;
+		uint32_t out[kScanPer];
+#pragma unroll
+		for (uint32_t j = 0; j < kScanPer; j++) {
+			out[j] = ((run_s % num_rails) << 16) | (run_b % num_rails);
+			run_s += v[j] >> 16;
+			run_b += v[j] & 0xffffu;
+		}
+		if (whole) {
+			*reinterpret_cast<u32x4 *>(tile_prefix + t0) = u32x4{ out[0], out[1], out[2], out[3] };
+			*reinterpret_cast<u32x4 *>(tile_prefix + t0 + 4) = u32x4{ out[4], out[5], out[6], out[7] };
+		} else {
+#pragma unroll
+			for (uint32_t j = 0; j < kScanPer; j++) {
+				if (t0 + j < num_tiles) {
+					tile_prefix[t0 + j] = out[j];
+				}
+			}
 		}
 		carry_small = (carry_small + tot_s) % num_rails;
 		carry_big = (carry_big + tot_b) % num_rails;
@@ -244,15 +291,23 @@ __global__ __launch_bounds__(kThreads) void stripe_emit_kernel(
 	uint64_t align, const uint32_t *__restrict__ tile_prefix, const uint32_t *__restrict__ seed0,
 	uint32_t *__restrict__ num_xfers, u32x4 *__restrict__ xfers)
 {
-	params_t p;
-	if (!load_params(state, align, p)) {
-		return;
-	}
 	/* 256 rows of 96 bytes = 6 x 16 B each */
 	__shared__ u32x4 rows[kThreads * 6];
 	__shared__ uint32_t wave_sum[kThreads / 64];
 	const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
 	const uint32_t base = blockIdx.x * (kThreads * PASSES);
+	/* every pass's size is requested up front: the passes below then run out of registers
+	 * instead of each waiting for its own load */
+	uint64_t size_of[PASSES];
+#pragma unroll
+	for (uint32_t pass = 0; pass < PASSES; pass++) {
+		const uint32_t i = base + pass * kThreads + threadIdx.x;
+		size_of[pass] = i < n ? __builtin_nontemporal_load(&sizes[i]) : 0;
+	}
+	params_t p;
+	if (!load_params(state, align, p)) {
+		return;
+	}
 	const uint32_t R = p.num_rails;
 
 	uint32_t seed;
@@ -278,6 +333,7 @@ __global__ __launch_bounds__(kThreads) void stripe_emit_kernel(
 	}
 	uint32_t carry_small = seed >> 16, carry_big = seed & 0xffffu; /* both < R */
 
+#pragma unroll
 	for (uint32_t pass = 0; pass < PASSES; pass++) {
 		const uint32_t first = base + pass * kThreads;
 		if (first >= n) {
@@ -285,7 +341,7 @@ __global__ __launch_bounds__(kThreads) void stripe_emit_kernel(
 		}
 		const uint32_t i = first + threadIdx.x;
 		const bool live = i < n;
-		const uint64_t size = live ? sizes[i] : 0;
+		const uint64_t size = size_of[pass];
 		uint32_t k = 0;
 		const uint32_t c = live ? contribution(size, p, k) : 0;
 
@@ -305,31 +361,32 @@ __global__ __launch_bounds__(kThreads) void stripe_emit_kernel(
 
 		/* set_schedule_by_threshold, src/nccl_ofi_scheduler.cpp:77-133 */
 		const bool small = (c >> 16) != 0;
-		uint32_t rail = small ? (carry_small + (excl >> 16)) % R
-				      : (carry_big + (excl & 0xffffu)) % R;
+		uint32_t rail = mod_rails(small ? carry_small + (excl >> 16) : carry_big + (excl & 0xffffu), p);
 		uint64_t max_stripe = size;
 		if (!small) {
-			uint64_t per = size == 0 ? 0 : 1 + div_small(size - 1, k);
+			/* (size - 1) / k: k is 1, 2 or 4 unless there are three rails */
+			uint64_t whole = size == 0 ? 0 : (size - 1) >> (k >> 1);
+			if (R == 3) {
+				whole = k == 3 ? (size == 0 ? 0 : (size - 1) / 3) : whole;
+			}
+			const uint64_t per = size == 0 ? 0 : 1 + whole;
 			max_stripe = div_ceil_by(per, p.align, p.align_shift) * p.align;
 		}
+		/* k stripes of max_stripe cover the message, so `left` is 0 from stripe k on and the
+		 * length of an unused entry comes out as 0 by itself; lanes past the end have k = 0 */
 		uint64_t left = size, offset = 0;
 		u32x4 *row = &rows[threadIdx.x * 6];
 		uint64_t f[12]; /* 4 x {rail word, offset, msg_size} */
 #pragma unroll
 		for (uint32_t s = 0; s < 4; s++) {
-			if (live && s < k) {
-				uint64_t stripe = left < max_stripe ? left : max_stripe;
-				f[3 * s + 0] = rail; /* rail_id in the low 16 bits, padding zero */
-				f[3 * s + 1] = offset;
-				f[3 * s + 2] = stripe;
-				offset += stripe;
-				left -= stripe;
-				rail = (rail + 1) % R;
-			} else {
-				f[3 * s + 0] = 0;
-				f[3 * s + 1] = 0;
-				f[3 * s + 2] = 0;
-			}
+			const bool used = s < k;
+			const uint64_t stripe = left < max_stripe ? left : max_stripe;
+			f[3 * s + 0] = used ? rail : 0; /* rail_id in the low 16 bits, padding zero */
+			f[3 * s + 1] = used ? offset : 0;
+			f[3 * s + 2] = stripe;
+			offset += stripe;
+			left -= stripe;
+			rail = rail + 1 == R ? 0 : rail + 1;
 		}
 #pragma unroll
 		for (uint32_t q = 0; q < 6; q++) {
@@ -349,11 +406,15 @@ __global__ __launch_bounds__(kThreads) void stripe_emit_kernel(
 		const uint32_t valid = (n - first) < kThreads ? (n - first) : kThreads;
 		u32x4 *out = xfers + (uint64_t)first * 6;
 		for (uint32_t v = threadIdx.x; v < valid * 6; v += kThreads) {
+#if OFI_STRIPE_NT_STORES
 			__builtin_nontemporal_store(rows[v], &out[v]);
+#else
+			out[v] = rows[v];
+#endif
 		}
 
-		carry_small = (carry_small + (tot >> 16)) % R;
-		carry_big = (carry_big + (tot & 0xffffu)) % R;
+		carry_small = mod_rails(carry_small + (tot >> 16), p);
+		carry_big = mod_rails(carry_big + (tot & 0xffffu), p);
 		__syncthreads();
 	}
 	if (INLINE && blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {

@@ -68,6 +68,28 @@ def test_parity_random(lib, oracle, gpu, n, rails, min_stripe, max_small, seeds)
     assert (st.max_small_msg_size, st.min_stripe_size, st.num_rails) == (max_small, min_stripe, rails)
 
 
+@pytest.mark.parametrize("n", [1, 2, 511, 513, 70001, 3_000_001])
+def test_sizes_array_at_an_odd_eight_byte_offset(lib, oracle, gpu, n):
+    """The sizes array only has to be 8-byte aligned."""
+    sizes = synthetic.stripe_sizes(n + 5, n)
+    sizes[::7] = sizes[::7] % np.uint64(100)
+    want_num, want_xf, ost = _oracle.sched_batch(oracle, sizes, 4, 131072, 64, (3, 1))
+    for shift in (0, 1):
+        d_state = dev_state(4, 131072, 64, (3, 1))
+        d_all = _gpu.to_dev(np.concatenate([np.zeros(shift, dtype=np.uint64), sizes]))
+        d_sizes = d_all[shift:]
+        assert d_sizes.data_ptr() % 16 == 8 * shift
+        d_num = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+        d_xf = torch.full((n * 12,), -1, dtype=torch.int64, device="cuda")
+        assert lib.ofi_amd_sched_batch(d_state.data_ptr(), d_sizes.data_ptr(), n, 128, d_num.data_ptr(),
+                                       d_xf.data_ptr(), _gpu.stream()) == 0
+        _gpu.sync()
+        assert np.array_equal(_gpu.to_host(d_num, np.uint32), want_num)
+        assert np.array_equal(_gpu.to_host(d_xf, np.uint64).reshape(n, 4, 3), want_xf)
+        st = read_state(d_state)
+        assert (st.rr_small_counter, st.rr_counter) == (ost.rr_small_counter, ost.rr_counter)
+
+
 def test_chained_batches_carry_state(lib, oracle, gpu):
     sizes = synthetic.stripe_sizes(77, 30000)
     want_num, want_xf, ost = _oracle.sched_batch(oracle, sizes, 4, 131072, 64, (1, 2))
