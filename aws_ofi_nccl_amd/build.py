@@ -16,7 +16,6 @@ ROOT = os.path.dirname(PKG)
 CSRC = os.path.join(PKG, "csrc")
 LIBDIR = os.path.join(PKG, "lib")
 LIB = os.path.join(LIBDIR, "libofi_amd_hotpath.so")
-TUNER_LIB = os.path.join(LIBDIR, "libofi_amd_tuner.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops off: hipcc must not form packed fp32 instructions.

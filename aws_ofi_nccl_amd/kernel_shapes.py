@@ -6,8 +6,9 @@ nothing else of interest, which keeps counter runs short.  The shapes:
 
   bounce    configured   65,536 buffers, lengths uniform 0..8,192 B, packed source (any byte
                          alignment), 64-byte-aligned destinations scattered over 2 GiB
-            aligned8k    65,536 buffers of exactly 8,192 B, sources 8 KiB apart, the same kind of
-                         scattered destinations (what the length and alignment mix costs)
+            aligned8k    --buffers (default 65,536) buffers of exactly 8,192 B, sources 8 KiB
+                         apart, the same kind of scattered destinations (what the length and
+                         alignment mix costs); 32,768 buffers move the configured batch's bytes
             dense8k      the same with destination i right behind destination i-1 (what the
                          scatter costs)
   copy      payload      a plain device-to-device copy of the configured payload (268,444,074 B):
@@ -34,6 +35,7 @@ def main():
     ap.add_argument("--kernel", required=True, choices=["bounce", "copy", "fill", "striping", "model", "region", "eager"])
     ap.add_argument("--shape", default=None)
     ap.add_argument("--launches", type=int, default=30)
+    ap.add_argument("--buffers", type=int, default=65536, help="bounce aligned8k / dense8k: buffer count")
     ap.add_argument("--no-flush", action="store_true", help="bounce / eager: no read-back")
     ap.add_argument("--graph", action="store_true",
                     help="record one call into a HIP graph and replay it --launches times")
@@ -63,6 +65,9 @@ def main():
         w = synthetic.bounce_workload(SEED)
         n = len(w["len"])
         if shape in ("aligned8k", "dense8k"):
+            n = args.buffers
+            if not 0 < n <= (2 << 30) // 8192:
+                ap.error("--buffers out of range")
             length = np.full(n, 8192, dtype=np.uint32)
             src_off = np.arange(n, dtype=np.uint64) * np.uint64(8192)
             if shape == "dense8k":
