@@ -413,7 +413,7 @@ __device__ __forceinline__ int log2i_nodes(uint64_t nodes)
 
 /* Which polygon set answers for (platform, collective, ranks per node): shape selection as in
  * the per-platform init functions (:302,:485,:675,:768,:878,...).  count 0: no regions. */
-__device__ __forceinline__ void region_set(const region_tables_t &t, int platform, int coll, uint64_t ranks,
+__host__ __device__ __forceinline__ void region_set(const region_tables_t &t, int platform, int coll, uint64_t ranks,
 					    uint64_t nodes, int &first, int &count)
 {
 	first = 0;

@@ -8,6 +8,7 @@
  * Nothing here is matrix-shaped: one thread per decision point, which also evaluates the
  * point's cost cells (staged in LDS, written out as contiguous runs).
  */
+#include <algorithm>
 #include <cstring>
 #include <mutex>
 #include <new>
@@ -97,94 +98,103 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 constexpr int kMaxSetPolys = 8;  /* polygons of one (platform, shape, collective) set */
 constexpr int kMaxSetVerts = 64; /* their vertices together */
 constexpr uint32_t kRegionBlock = 64; /* threads per workgroup of the region kernel: one wavefront */
+constexpr uint32_t kXcds = 8;         /* workgroup w of a launch runs on XCD w mod 8, each with its own L2 */
 static_assert(kRegionBlock >= (uint32_t)kMaxSetVerts && kRegionBlock >= (uint32_t)kMaxSetPolys * 4,
 	      "one thread per staged vertex and per staged polygon word");
 
 /*
- * One thread per (collective, size, node count); blockIdx.y is the platform entry.  A workgroup
- * works on one collective -- `blocks_per_run` workgroups share its n_sizes x n_nodes points, node
- * count fastest -- and takes the ranks-per-node values in turn, because the polygon set depends
- * on the (collective, ranks per node) pair alone: for each pair the set (at most 8 polygons, 64
- * vertices, with their bounds) is copied into LDS once and every lane then walks the same
- * polygons out of LDS instead of chasing them through global memory; pairs without regions cost
- * one table lookup.  A thread ends up with the decisions of all ranks-per-node values of its
- * point, which are neighbours in the output: it writes them as one 16-byte store per four (the
- * wavefront then writes 1 KiB contiguous), where a thread per output record had written 4 bytes
- * at a 16-byte stride -- four times the write traffic for the same records.
+ * One thread per point.  A workgroup (one wavefront) works on
+ * 64 points of one (collective, ranks per node) pair -- `blocks_per_run` chunks make up the
+ * pair's n_sizes x n_nodes points, node count fastest -- because the polygon set depends on that
+ * pair alone: the set (at most 8 polygons, 64 vertices, with their bounds) is copied into LDS
+ * once and every lane then walks the same polygons out of LDS instead of chasing them through
+ * global memory, and workgroups of pairs without regions leave after one table lookup.
+ *
+ * In the output the ranks-per-node index runs fastest, so a wavefront's 64 records lie 4 x
+ * n_ppn bytes apart and the records between them belong to the same chunk's other
+ * ranks-per-node values, i.e. to other workgroups.  Those workgroups are given numbers that
+ * are equal mod 8: they run on the same XCD, their partial writes to a cache line meet in that
+ * XCD's L2 and leave it as one line (measured: 4.7 MB written for 4.7 MB of records; with the
+ * workgroups of a chunk on different XCDs every L2 wrote its quarter of each line, 18.9 MB).
+ * Giving a thread all ranks-per-node values of its point, or a workgroup four wavefronts that
+ * share an LDS staging buffer, writes the same 4.7 MB but makes the units of work four times
+ * coarser, and the launch, which lasts as long as its most loaded SIMD, 15-18 % longer.
  */
 __global__ __launch_bounds__(kRegionBlock) void region_choice_kernel(grid_dims_t g, region_tables_t t,
 							    const int32_t *__restrict__ platforms,
 							    uint32_t points_per_platform, uint32_t blocks_per_run,
-							    uint32_t spread, int8_t *__restrict__ choice)
+							    const uint2 *__restrict__ order, int8_t *__restrict__ choice)
 {
 	__shared__ int32_t s_poly[kMaxSetPolys * 4];
 	__shared__ double s_bounds[kMaxSetPolys * 4];
 	__shared__ pt_t s_verts[kMaxSetVerts];
 
-	/* Workgroups go to the eight XCDs in turn, and collectives with many regions sit at a fixed
-	 * period in the run index: taken in launch order, the long-running workgroups would land on
-	 * the same few XCDs.  `spread` is coprime to the grid width, so this is a permutation that
-	 * scatters every period over all XCDs. */
-	const uint32_t block = (uint32_t)(((uint64_t)blockIdx.x * spread) % gridDim.x);
-	const uint32_t ci = block / blocks_per_run;
-	const uint32_t in_run = (block - ci * blocks_per_run) * kRegionBlock + threadIdx.x;
-	const int platform = platforms[blockIdx.y];
+	/* blockIdx.x = k * 8 + x (a one-dimensional grid, so x is the XCD).  order[k] names a
+	 * (platform entry, group, pi): chunk 8 * group + x' of the collectives' chunks,
+	 * ranks-per-node index pi -- whatever the order, the workgroups of one chunk and platform
+	 * entry share x.  The host lists the triples by falling cost (polygons of the pair's set):
+	 * the long workgroups start first and the short ones fill the end of the launch, and
+	 * workgroups of equal cost are neighbours in launch order, which the dispatcher deals to
+	 * the CUs of an XCD in turn.  (In (entry, group, pi) order, or scattered by a fixed stride,
+	 * the pairs with many regions recur at periods that keep meeting the same CUs: 74-78 us
+	 * against 54 us.) */
+	const uint32_t x = blockIdx.x % kXcds;
+	const uint2 item = order[blockIdx.x / kXcds];
+	const uint32_t entry = item.x;
+	const uint32_t pi = item.y % g.n_ppn;
+	const uint32_t group = item.y / g.n_ppn;
+	/* which of a group's eight chunks an XCD takes rotates with the platform entry: the chunks
+	 * differ in cost (collective, size range), and an XCD that kept the same ones for every
+	 * entry would keep the same share of the long ones */
+	const uint32_t chunk = group * kXcds + (x + entry) % kXcds;
+	if (chunk >= blocks_per_run * g.n_colls) {
+		return; /* padding of the last group */
+	}
+	const uint32_t ci = chunk / blocks_per_run;
+	const uint32_t in_run = (chunk - ci * blocks_per_run) * kRegionBlock + threadIdx.x;
+	const int platform = platforms[entry];
 	const int coll = g.colls[ci];
-	const bool live = in_run < g.n_sizes * g.n_nodes;
-	const uint32_t ni = live ? in_run % g.n_nodes : 0;
-	const uint32_t si = live ? in_run / g.n_nodes : 0;
-	const uint64_t nodes = g.nodes[ni];
-	const uint64_t first_record = (uint64_t)blockIdx.y * points_per_platform +
-				      (uint64_t)((ci * g.n_sizes + si) * g.n_nodes + ni) * g.n_ppn;
-	uint32_t *out = reinterpret_cast<uint32_t *>(choice) + first_record;
-	const bool wide = (reinterpret_cast<uintptr_t>(choice) & 15u) == 0 && (first_record & 3u) == 0;
+	const uint32_t ppn = g.ppn[pi];
 
-	uint32_t group[4];
-	for (uint32_t pi = 0; pi < g.n_ppn; pi++) {
-		const uint32_t ppn = g.ppn[pi];
-		/* ranks = nodes * ppn with nodes >= 1: the shape is a function of ppn */
-		int first, count;
-		region_set(t, platform, coll, ppn, 1, first, count);
-		if (count > 0) {
-			__syncthreads(); /* the previous pair's set is no longer being read */
-			const int v0 = t.poly[first * 4 + 2];
-			const int v_end = t.poly[(first + count - 1) * 4 + 2] + t.poly[(first + count - 1) * 4 + 3];
-			if ((int)threadIdx.x < count * 4) {
-				const int32_t w = t.poly[first * 4 + threadIdx.x];
-				s_poly[threadIdx.x] = (threadIdx.x & 3u) == 2u ? w - v0 : w; /* vertex index within the set */
-				s_bounds[threadIdx.x] = t.bbox[first * 4 + threadIdx.x];
-			}
-			if ((int)threadIdx.x < v_end - v0) {
-				s_verts[threadIdx.x] = t.verts[v0 + threadIdx.x];
-			}
-			__syncthreads();
+	/* ranks = nodes * ppn with nodes >= 1: the shape is a function of ppn */
+	int first, count;
+	region_set(t, platform, coll, ppn, 1, first, count);
+	if (count > 0) {
+		const int v0 = t.poly[first * 4 + 2];
+		const int v_end = t.poly[(first + count - 1) * 4 + 2] + t.poly[(first + count - 1) * 4 + 3];
+		if ((int)threadIdx.x < count * 4) {
+			const int32_t w = t.poly[first * 4 + threadIdx.x];
+			s_poly[threadIdx.x] = (threadIdx.x & 3u) == 2u ? w - v0 : w; /* vertex index within the set */
+			s_bounds[threadIdx.x] = t.bbox[first * 4 + threadIdx.x];
 		}
-		int algorithm = -1, protocol = -1, nchannels = -1;
-		if (live && count > 0 && nodes > 2) {
-			int a, pr;
-			const pt_t at = { g.log2_sizes[si], g.log2_ranks[ni * g.n_ppn + pi] };
-			if (region_pick(s_poly, s_bounds, s_verts, count, at, kAllAllowed, t.far_point, a, pr) >= 0) {
-				algorithm = a;
-				protocol = pr;
-				nchannels = region_channels(platform, g.sizes[si], nodes * ppn, nodes, a, pr);
-			}
+		if ((int)threadIdx.x < v_end - v0) {
+			s_verts[threadIdx.x] = t.verts[v0 + threadIdx.x];
 		}
-		/* {int8 algorithm, int8 protocol, int16 nchannels} */
-		group[pi & 3u] = ((uint32_t)(uint8_t)(int8_t)algorithm) | ((uint32_t)(uint8_t)(int8_t)protocol << 8) |
-				 ((uint32_t)(uint16_t)(int16_t)nchannels << 16);
-		const bool group_full = (pi & 3u) == 3u;
-		if (live && (group_full || pi == g.n_ppn - 1)) {
-			const uint32_t g0 = pi & ~3u;
-			if (group_full && wide) {
-				u32x4_t v = { group[0], group[1], group[2], group[3] };
-				*reinterpret_cast<u32x4_t *>(out + g0) = v;
-			} else {
-				for (uint32_t k = g0; k <= pi; k++) {
-					out[k] = group[k & 3u];
-				}
-			}
+		__syncthreads();
+	}
+	if (in_run >= g.n_sizes * g.n_nodes) {
+		return;
+	}
+	const uint32_t ni = in_run % g.n_nodes;
+	const uint32_t si = in_run / g.n_nodes;
+	const uint32_t p = ((ci * g.n_sizes + si) * g.n_nodes + ni) * g.n_ppn + pi; /* output order */
+
+	const uint64_t nodes = g.nodes[ni];
+	int algorithm = -1, protocol = -1, nchannels = -1;
+	if (count > 0 && nodes > 2) {
+		int a, pr;
+		const pt_t at = { g.log2_sizes[si], g.log2_ranks[ni * g.n_ppn + pi] };
+		if (region_pick(s_poly, s_bounds, s_verts, count, at, kAllAllowed, t.far_point, a, pr) >= 0) {
+			algorithm = a;
+			protocol = pr;
+			nchannels = region_channels(platform, g.sizes[si], nodes * ppn, nodes, a, pr);
 		}
 	}
+	const uint64_t idx = (uint64_t)entry * points_per_platform + p;
+	/* {int8 algorithm, int8 protocol, int16 nchannels} as one 4-byte store */
+	reinterpret_cast<uint32_t *>(choice)[idx] = ((uint32_t)(uint8_t)(int8_t)algorithm) |
+						     ((uint32_t)(uint8_t)(int8_t)protocol << 8) |
+						     ((uint32_t)(uint16_t)(int16_t)nchannels << 16);
 }
 
 /* ---- host side: building the log2-space polygon tables ---- */
@@ -366,6 +376,11 @@ struct ofi_amd_tuner_plan {
 	/* what d_variants currently holds, so that an unchanged list is not uploaded again */
 	std::vector<ofi_amd_tuner_variant_t> h_variants;
 	std::vector<int32_t> h_platforms;
+	/* region launch order for the current platform list (see region_choice_kernel) */
+	std::vector<int32_t> h_colls;
+	std::vector<uint32_t> h_ppn;
+	uint2 *d_order;
+	uint64_t order_cap;
 };
 
 using namespace ofi_amd;
@@ -387,6 +402,7 @@ int ofi_amd_tuner_plan_destroy(ofi_amd_tuner_plan_t *plan)
 	(void)hipFree(plan->d_log2_ranks);
 	(void)hipFree(plan->d_variants);
 	(void)hipFree(plan->d_platforms);
+	(void)hipFree(plan->d_order);
 	delete plan;
 	return 0;
 }
@@ -426,6 +442,7 @@ int ofi_amd_tuner_plan_create(const int32_t *colls, uint32_t n_colls, const uint
 	}
 
 	auto *plan = new (std::nothrow) ofi_amd_tuner_plan();
+	/* value-initialised: every pointer and capacity starts at zero */
 	if (!plan) {
 		return -ENOMEM;
 	}
@@ -460,6 +477,13 @@ int ofi_amd_tuner_plan_create(const int32_t *colls, uint32_t n_colls, const uint
 		return rc;
 	}
 
+	try {
+		plan->h_colls.assign(colls, colls + n_colls);
+		plan->h_ppn.assign(ppn, ppn + n_ppn);
+	} catch (...) {
+		ofi_amd_tuner_plan_destroy(plan);
+		return -ENOMEM;
+	}
 	grid_dims_t &g = plan->g;
 	g.n_colls = n_colls;
 	g.n_sizes = n_sizes;
@@ -563,55 +587,81 @@ int ofi_amd_tuner_region_grid(ofi_amd_tuner_plan_t *plan, const int32_t *platfor
 			return -EINVAL;
 		}
 	}
-	hipStream_t s = as_stream(stream);
-	if (n_platforms > plan->platforms_cap) {
-		OFI_AMD_HIP_TRY(hipStreamSynchronize(s));
-		(void)hipFree(plan->d_platforms);
-		plan->d_platforms = nullptr;
-		plan->platforms_cap = 0;
-		plan->h_platforms.clear();
-		OFI_AMD_HIP_TRY(hipMalloc((void **)&plan->d_platforms, sizeof(int32_t) * n_platforms));
-		plan->platforms_cap = n_platforms;
-	}
-	try {
-		if (plan->h_platforms.size() != n_platforms ||
-		    std::memcmp(plan->h_platforms.data(), platforms, sizeof(int32_t) * n_platforms) != 0) {
-			plan->h_platforms.assign(platforms, platforms + n_platforms);
-			OFI_AMD_HIP_TRY(hipMemcpyAsync(plan->d_platforms, plan->h_platforms.data(),
-						       sizeof(int32_t) * n_platforms, hipMemcpyHostToDevice, s));
-			OFI_AMD_HIP_TRY(hipStreamSynchronize(s));
-		}
-	} catch (...) {
-		return -ENOMEM;
-	}
 	if (plan->points > (1ull << 31) || n_platforms > 65535) {
 		return -EINVAL;
 	}
 	const uint32_t points = (uint32_t)plan->points;
 	const uint64_t run_len = (uint64_t)plan->g.n_sizes * plan->g.n_nodes;
 	const uint64_t blocks_per_run = (run_len + kRegionBlock - 1) / kRegionBlock;
-	const uint64_t blocks = blocks_per_run * plan->g.n_colls;
+	const uint64_t n_chunks = blocks_per_run * plan->g.n_colls;
+	const uint64_t n_groups = (n_chunks + kXcds - 1) / kXcds;
+	const uint64_t per_entry = n_groups * plan->g.n_ppn;
+	const uint64_t per_xcd = per_entry * n_platforms;
+	const uint64_t blocks = per_xcd * kXcds;
 	if (blocks == 0 || blocks > 0x7fffffffull) {
 		return -EINVAL;
 	}
-	/* a multiplier near blocks / golden ratio, coprime to blocks */
-	uint64_t spread = (uint64_t)((double)blocks * 0.6180339887498949);
-	spread = spread < 1 ? 1 : spread;
-	for (;;) {
-		uint64_t a = spread, b = blocks;
-		while (b != 0) {
-			const uint64_t r = a % b;
-			a = b;
-			b = r;
-		}
-		if (a == 1) {
-			break;
-		}
-		spread++;
+
+	hipStream_t s = as_stream(stream);
+	if (n_platforms > plan->platforms_cap || per_xcd > plan->order_cap) {
+		OFI_AMD_HIP_TRY(hipStreamSynchronize(s));
+		(void)hipFree(plan->d_platforms);
+		(void)hipFree(plan->d_order);
+		plan->d_platforms = nullptr;
+		plan->d_order = nullptr;
+		plan->platforms_cap = 0;
+		plan->order_cap = 0;
+		plan->h_platforms.clear();
+		OFI_AMD_HIP_TRY(hipMalloc((void **)&plan->d_platforms, sizeof(int32_t) * n_platforms));
+		plan->platforms_cap = n_platforms;
+		OFI_AMD_HIP_TRY(hipMalloc((void **)&plan->d_order, sizeof(uint2) * per_xcd));
+		plan->order_cap = per_xcd;
 	}
-	hipLaunchKernelGGL(region_choice_kernel, dim3((uint32_t)blocks, n_platforms), dim3(kRegionBlock), 0, s,
-			   plan->g, plan->t, plan->d_platforms, points, (uint32_t)blocks_per_run, (uint32_t)(spread % blocks),
-			   d_choice);
+	try {
+		if (plan->h_platforms.size() != n_platforms ||
+		    std::memcmp(plan->h_platforms.data(), platforms, sizeof(int32_t) * n_platforms) != 0) {
+			plan->h_platforms.clear(); /* stays empty if an upload fails: the next call uploads again */
+			/* launch order: (entry, group, pi) by falling number of polygons in the pair's set; a
+			 * group that straddles two collectives counts as the costlier one */
+			struct item_t {
+				int32_t cost;
+				uint2 v;
+			};
+			std::vector<item_t> items;
+			items.reserve(per_xcd);
+			for (uint32_t pi = 0; pi < plan->g.n_ppn; pi++) {
+				for (uint64_t group = 0; group < n_groups; group++) {
+					const uint64_t last = std::min<uint64_t>(group * kXcds + kXcds - 1, n_chunks - 1);
+					const int32_t c0 = plan->h_colls[group * kXcds / blocks_per_run];
+					const int32_t c1 = plan->h_colls[last / blocks_per_run];
+					for (uint32_t e = 0; e < n_platforms; e++) {
+						int first, count0, count1;
+						region_set(plan->t, platforms[e], c0, plan->h_ppn[pi], 1, first, count0);
+						region_set(plan->t, platforms[e], c1, plan->h_ppn[pi], 1, first, count1);
+						items.push_back({ std::max(count0, count1),
+								  make_uint2(e, (uint32_t)(group * plan->g.n_ppn + pi)) });
+					}
+				}
+			}
+			std::stable_sort(items.begin(), items.end(),
+					 [](const item_t &a, const item_t &b) { return a.cost > b.cost; });
+			std::vector<uint2> order(items.size());
+			for (size_t i = 0; i < items.size(); i++) {
+				order[i] = items[i].v;
+			}
+			OFI_AMD_HIP_TRY(hipMemcpyAsync(plan->d_platforms, platforms, sizeof(int32_t) * n_platforms,
+						       hipMemcpyHostToDevice, s));
+			OFI_AMD_HIP_TRY(hipMemcpyAsync(plan->d_order, order.data(), sizeof(uint2) * order.size(),
+						       hipMemcpyHostToDevice, s));
+			OFI_AMD_HIP_TRY(hipStreamSynchronize(s));
+			plan->h_platforms.assign(platforms, platforms + n_platforms);
+		}
+	} catch (...) {
+		plan->h_platforms.clear();
+		return -ENOMEM;
+	}
+	hipLaunchKernelGGL(region_choice_kernel, dim3((uint32_t)blocks), dim3(kRegionBlock), 0, s, plan->g, plan->t,
+			   plan->d_platforms, points, (uint32_t)blocks_per_run, plan->d_order, d_choice);
 	OFI_AMD_HIP_TRY(hipGetLastError());
 	return 0;
 }
