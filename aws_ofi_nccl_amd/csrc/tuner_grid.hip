@@ -118,7 +118,8 @@ static_assert(kRegionBlock >= (uint32_t)kMaxSetVerts && kRegionBlock >= (uint32_
  * workgroups of a chunk on different XCDs every L2 wrote its quarter of each line, 18.9 MB).
  * Giving a thread all ranks-per-node values of its point, or a workgroup four wavefronts that
  * share an LDS staging buffer, writes the same 4.7 MB but makes the units of work four times
- * coarser, and the launch, which lasts as long as its most loaded SIMD, 15-18 % longer.
+ * coarser, and the launch, which lasts as long as its most loaded SIMD, 15-18 % longer than
+ * with single-wavefront units.
  */
 __global__ __launch_bounds__(kRegionBlock) void region_choice_kernel(grid_dims_t g, region_tables_t t,
 							    const int32_t *__restrict__ platforms,
