@@ -268,7 +268,9 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 				event_t ev;
 				std::memset(&ev, 0, sizeof(ev));
 				ev.peer = p.peer;
-				if (p.kind == OFI_AMD_GIN_POST_WRITE) {
+				if (p.kind == OFI_AMD_GIN_POST_WRITE || p.kind == OFI_AMD_GIN_POST_READ) {
+					/* a read is the same copy the other way, and the target hears nothing of it */
+					const bool read = p.kind == OFI_AMD_GIN_POST_READ;
 					const uint64_t pieces = (p.len + kPiece - 1) / kPiece;
 					if (pieces > cap_copy) {
 						return -EMSGSIZE; /* a write larger than the table: raise batch_writes */
@@ -282,15 +284,19 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 					batch_t &b = batches[cur];
 					for (uint64_t off = 0; off < p.len; off += kPiece) {
 						const uint64_t len = p.len - off < kPiece ? p.len - off : kPiece;
-						b.src[b.n_copy] = p.src + off;
-						b.dst[b.n_copy] = p.dest + off;
+						b.src[b.n_copy] = (read ? p.dest : p.src) + off;
+						b.dst[b.n_copy] = (read ? p.src : p.dest) + off;
 						b.len[b.n_copy] = (uint32_t)len;
 						b.n_copy++;
 					}
 					st.bytes += p.len;
-					st.writes++;
-					ev.imm = p.imm;
-					in_flight.push_back(ev);
+					if (read) {
+						st.reads++;
+					} else {
+						st.writes++;
+						ev.imm = p.imm;
+						in_flight.push_back(ev);
+					}
 				} else if (p.kind == OFI_AMD_GIN_POST_META) {
 					ev.is_meta = 1;
 					std::memcpy(ev.meta, p.msg, sizeof(ev.meta));
@@ -332,7 +338,7 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 					break;
 				}
 				ofi_amd_gin_wire_t wire;
-				rc = ofi_amd_gin_iput_signal(&comms[c], mrs, n_mrs, &d, &wire);
+				rc = ofi_amd_gin_derive(&comms[c], mrs, n_mrs, &d, &wire);
 				const auto w0 = clock::now();
 				while (rc == -EAGAIN) {
 					/* window closed (await_tx_window, :518-537, progresses until it opens): let
@@ -340,7 +346,7 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 					rc = pump();
 					if (rc == 0) rc = deliver_some(0);
 					if (rc == 0) rc = pump();
-					if (rc == 0) rc = ofi_amd_gin_iput_signal(&comms[c], mrs, n_mrs, &d, &wire);
+					if (rc == 0) rc = ofi_amd_gin_derive(&comms[c], mrs, n_mrs, &d, &wire);
 					if (rc == -EAGAIN &&
 					    std::chrono::duration_cast<std::chrono::milliseconds>(clock::now() - w0).count() >
 						    (long long)timeout_ms) {
@@ -360,7 +366,8 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 					break;
 				}
 				int32_t req = -1;
-				rc = ofi_amd_gin_tx_iput_signal(tx, c, &wire, &req);
+				rc = d.kind == OFI_AMD_GIN_KIND_GET ? ofi_amd_gin_tx_iget(tx, c, &wire, &req)
+								   : ofi_amd_gin_tx_iput_signal(tx, c, &wire, &req);
 				if (rc != 0) {
 					break;
 				}

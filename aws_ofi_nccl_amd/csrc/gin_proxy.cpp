@@ -141,7 +141,9 @@ static int drain_contexts(ofi_amd_gin_rings_t *r, uint32_t c_begin, uint32_t c_e
 					ofi_amd_gin_wire_t local;
 					ofi_amd_gin_wire_t *wire =
 						out_wire ? &out_wire[(size_t)c * ops_per_context + i] : &local;
-					int e = ofi_amd_gin_iput_signal(&comms[c], mrs, n_mrs, d, wire);
+					int e = d->kind == OFI_AMD_GIN_KIND_GET
+							? ofi_amd_gin_iget(&comms[c], mrs, n_mrs, d, wire)
+							: ofi_amd_gin_iput_signal(&comms[c], mrs, n_mrs, d, wire);
 					if (e != 0) {
 						rc = e;
 						break;

@@ -195,12 +195,11 @@ int ofi_amd_gin_tx_destroy(ofi_amd_gin_tx_t *tx)
 	return 0;
 }
 
-int ofi_amd_gin_tx_iput_signal(ofi_amd_gin_tx_t *tx, uint32_t peer, const ofi_amd_gin_wire_t *wire,
-			       int32_t *request)
+/* The posts of one operation: its writes (or, for a get, its reads) in stripe order, then its
+ * metadata message. */
+static int post_operation(ofi_amd_gin_tx_t *tx, uint32_t peer, const ofi_amd_gin_wire_t *wire,
+			  uint32_t transfer_kind, int32_t *request)
 {
-	if (!tx || !wire || !request || wire->num_writes > OFI_AMD_MAX_NUM_RAILS) {
-		return -EINVAL;
-	}
 	*request = -1;
 	const uint32_t need = 1 + wire->num_writes + (wire->has_meta ? 1u : 0u);
 	if (tx->free_list.size() < need) {
@@ -222,7 +221,10 @@ int ofi_amd_gin_tx_iput_signal(ofi_amd_gin_tx_t *tx, uint32_t peer, const ofi_am
 	uint32_t n_subs = 0;
 
 	/* a post failed for good: the umbrella goes back to the pool and the posts already made
-	 * lose their way back to it (clear_write_reqs_pending_back_pointers, :746-758) */
+	 * lose their way back to it (clear_write_reqs_pending_back_pointers, :746-758;
+	 * clear_read_reqs_pending_back_pointers, :869-877).  The failed request goes back too; the
+	 * reference's iget leaves its failed read request out of the pool (:925-931), which is not
+	 * repeated here. */
 	auto give_up = [&](uint32_t failed) {
 		for (uint32_t k = 0; k < n_subs; k++) {
 			if (subs[k] != failed) {
@@ -233,7 +235,7 @@ int ofi_amd_gin_tx_iput_signal(ofi_amd_gin_tx_t *tx, uint32_t peer, const ofi_am
 		tx->release(op);
 	};
 
-	for (uint32_t k = 0; k < wire->num_writes; k++) { /* :737-784 */
+	for (uint32_t k = 0; k < wire->num_writes; k++) { /* :737-784, :901-932 */
 		const ofi_amd_gin_write_t &w = wire->writes[k];
 		uint32_t idx = 0;
 		(void)tx->alloc(&idx);
@@ -241,7 +243,7 @@ int ofi_amd_gin_tx_iput_signal(ofi_amd_gin_tx_t *tx, uint32_t peer, const ofi_am
 		r.use = kSub;
 		r.slot = (uint8_t)k;
 		r.parent = (int32_t)op;
-		r.post = ofi_amd_gin_post_t{OFI_AMD_GIN_POST_WRITE, w.rail, w.more, idx, peer, wire->imm,
+		r.post = ofi_amd_gin_post_t{transfer_kind, w.rail, w.more, idx, peer, wire->imm,
 					    w.src, w.len, w.dest, w.key, {0, 0, 0, 0}};
 		tx->pool[op].pending_mask |= 1u << k;
 		subs[n_subs++] = idx;
@@ -280,6 +282,26 @@ int ofi_amd_gin_tx_iput_signal(ofi_amd_gin_tx_t *tx, uint32_t peer, const ofi_am
 	}
 	*request = (int32_t)op;
 	return 0;
+}
+
+int ofi_amd_gin_tx_iput_signal(ofi_amd_gin_tx_t *tx, uint32_t peer, const ofi_amd_gin_wire_t *wire,
+			       int32_t *request)
+{
+	if (!tx || !wire || !request || wire->num_writes > OFI_AMD_MAX_NUM_RAILS) {
+		return -EINVAL;
+	}
+	return post_operation(tx, peer, wire, OFI_AMD_GIN_POST_WRITE, request);
+}
+
+int ofi_amd_gin_tx_iget(ofi_amd_gin_tx_t *tx, uint32_t peer, const ofi_amd_gin_wire_t *wire,
+			int32_t *request)
+{
+	/* a get's record: reads only, nothing for the target (ofi_amd_gin_iget) */
+	if (!tx || !wire || !request || wire->num_writes < 1 || wire->num_writes > OFI_AMD_MAX_NUM_RAILS ||
+	    wire->has_meta || wire->nseg != 0 || wire->imm != 0) {
+		return -EINVAL;
+	}
+	return post_operation(tx, peer, wire, OFI_AMD_GIN_POST_READ, request);
 }
 
 int ofi_amd_gin_tx_send_ack(ofi_amd_gin_tx_t *tx, uint32_t peer, uint64_t ack_msg)

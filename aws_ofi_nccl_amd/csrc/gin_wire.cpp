@@ -280,4 +280,49 @@ int ofi_amd_gin_iput_signal(ofi_amd_gin_comm_t *c, const ofi_amd_gin_mr_t *mrs, 
 	return fast ? derive<true>(c, mrs, n_mrs, d, out) : derive_general(c, mrs, n_mrs, d, out);
 }
 
+/* nccl_ofi_rdma_gin_put_comm::iget, src/rdma/gin/nccl_ofi_gin.cpp:879-939: the schedule of the
+ * size from the endpoint's scheduler (:899), and per stripe a read into
+ * local input_address + localOff + offset from remote address_offset + remoteOff + offset with
+ * the remote registration's key for the stripe's rail (:903-916).  No sequence number, no
+ * window, no pin: gets are rare next to puts, so this is the plain loop. */
+int ofi_amd_gin_iget(ofi_amd_gin_comm_t *c, const ofi_amd_gin_mr_t *mrs, uint32_t n_mrs,
+		     const ofi_amd_gin_desc_t *d, ofi_amd_gin_wire_t *out)
+{
+	if (!c || !mrs || !d || !out) {
+		return -EINVAL;
+	}
+	std::memset(out, 0, sizeof(*out));
+	if (d->kind != OFI_AMD_GIN_KIND_GET || d->src_mr >= n_mrs || d->dst_mr >= n_mrs) {
+		return -EINVAL;
+	}
+	ofi_amd_xfer_info_t xfers[OFI_AMD_MAX_NUM_RAILS];
+	const int n = ofi_amd_sched_get_schedule(&c->sched, d->size, kStripeAlign, xfers);
+	if (n < 1 || n > OFI_AMD_MAX_NUM_RAILS) {
+		return n < 0 ? n : -ENOMEM;
+	}
+	const ofi_amd_gin_mr_t &remote = mrs[d->src_mr];
+	const uint64_t local = mrs[d->dst_mr].local_base + d->dst_off;
+	const uint64_t from = remote.remote_address_offset + d->src_off;
+	for (int k = 0; k < n; k++) {
+		ofi_amd_gin_write_t &r = out->writes[k];
+		r.rail = xfers[k].rail_id;
+		r.src = local + xfers[k].offset;
+		r.len = xfers[k].msg_size;
+		r.dest = from + xfers[k].offset;
+		r.key = remote.key[r.rail];
+		r.more = 0; /* "iget uses fi_read -- not part of the FI_MORE write-doorbell path" (:884) */
+	}
+	out->num_writes = (uint32_t)n;
+	return 0;
+}
+
+int ofi_amd_gin_derive(ofi_amd_gin_comm_t *c, const ofi_amd_gin_mr_t *mrs, uint32_t n_mrs,
+		       const ofi_amd_gin_desc_t *d, ofi_amd_gin_wire_t *out)
+{
+	if (d && d->kind == OFI_AMD_GIN_KIND_GET) {
+		return ofi_amd_gin_iget(c, mrs, n_mrs, d, out);
+	}
+	return ofi_amd_gin_iput_signal(c, mrs, n_mrs, d, out);
+}
+
 } /* extern "C" */

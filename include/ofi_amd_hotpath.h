@@ -263,8 +263,15 @@ typedef struct {
 	uint16_t src_mr;
 	uint16_t dst_mr;
 	uint16_t sig_mr;     /* 0xffff: no signal handle */
-	uint16_t kind;       /* 1 put, 2 put-signal */
+	uint16_t kind;       /* 1 put, 2 put-signal, 3 get */
 } ofi_amd_gin_desc_t;    /* 64 bytes */
+
+/* A get (iget, include/nccl_ofi_gin_base.h; src/rdma/gin/nccl_ofi_gin.cpp:879-939) moves data
+ * the other way: src_off / src_mr are remoteOff / remoteMhandle (where the bytes are read),
+ * dst_off / dst_mr are localOff / localMhandle (where they land); the signal fields are 0. */
+#define OFI_AMD_GIN_KIND_PUT 1
+#define OFI_AMD_GIN_KIND_PUT_SIGNAL 2
+#define OFI_AMD_GIN_KIND_GET 3
 
 typedef struct ofi_amd_gin_rings ofi_amd_gin_rings_t;
 
@@ -355,7 +362,9 @@ typedef struct {
 	uint64_t key[OFI_AMD_MAX_NUM_RAILS];
 } ofi_amd_gin_mr_t;
 
-/* One RDMA write the proxy would post (fi_writemsg arguments minus libfabric handles). */
+/* One RDMA write the proxy would post (fi_writemsg arguments minus libfabric handles), or one
+ * RDMA read of a get (fi_read arguments): src is the local buffer -- read from by a write,
+ * filled by a read -- and dest the offset in the peer's registration. */
 typedef struct {
 	uint64_t src;
 	uint64_t len;
@@ -405,6 +414,18 @@ int ofi_amd_gin_comm_init(ofi_amd_gin_comm_t *c, uint32_t comm_id, uint32_t num_
  * full; the reference blocks in await_tx_window).  *out is all-zero on failure. */
 int ofi_amd_gin_iput_signal(ofi_amd_gin_comm_t *c, const ofi_amd_gin_mr_t *mrs, uint32_t n_mrs,
 			    const ofi_amd_gin_desc_t *d, ofi_amd_gin_wire_t *out);
+/* iget's derivation (src/rdma/gin/nccl_ofi_gin.cpp:879-939): the schedule of d->size from the
+ * same scheduler as the puts, one read per stripe in out->writes[0..num_writes), never FI_MORE.
+ * A get has no sequence number, takes no room in the TX window and tells the target nothing:
+ * seq, nseg, imm, ack_req and the metadata fields of *out are 0 (nseg == 0 marks a get's
+ * record), and of *c only the scheduler's counters change.  A size of 0 is one read of length
+ * 0, as the reference posts it.  0; -EINVAL (a NULL argument, a descriptor of another kind, a
+ * handle >= n_mrs; *out all-zero). */
+int ofi_amd_gin_iget(ofi_amd_gin_comm_t *c, const ofi_amd_gin_mr_t *mrs, uint32_t n_mrs,
+		     const ofi_amd_gin_desc_t *d, ofi_amd_gin_wire_t *out);
+/* Either of the two by the descriptor's kind: what a proxy runs per popped descriptor. */
+int ofi_amd_gin_derive(ofi_amd_gin_comm_t *c, const ofi_amd_gin_mr_t *mrs, uint32_t n_mrs,
+		       const ofi_amd_gin_desc_t *d, ofi_amd_gin_wire_t *out);
 /* apply_rx_consumed, include/rdma/gin/nccl_ofi_gin.h:535-543 */
 void ofi_amd_gin_apply_ack(ofi_amd_gin_comm_t *c, uint32_t wire_rx_consumed);
 /* Wire encoders, include/rdma/gin/nccl_ofi_gin_types.h:39-181 */
@@ -427,7 +448,8 @@ typedef struct {
  * progress (-ETIMEDOUT).
  *   mode 0: pop + fold every descriptor into the checksum;
  *   mode 1: also store the descriptors: out_desc[c * ops_per_context + i];
- *   mode 2: also run the iputSignal derivation per context (comms[c], mrs[0..n_mrs));
+ *   mode 2: also run the derivation per context (comms[c], mrs[0..n_mrs); ofi_amd_gin_derive:
+ *           iputSignal's for puts, iget's for gets);
  *           out_wire (may be NULL) receives the wire records at
  *           [c * ops_per_context + i].  The checksum is that of mode 0: what a proxy
  *           does with a record (the posts) is not this library's, and checking is
@@ -468,6 +490,7 @@ int ofi_amd_gin_proxy_drain_mt(ofi_amd_gin_rings_t *rings, uint64_t ops_per_cont
 #define OFI_AMD_GIN_POST_WRITE 1 /* fi_writemsg with FI_REMOTE_CQ_DATA */
 #define OFI_AMD_GIN_POST_META 2  /* fi_sendmsg of the 32-byte metadata message */
 #define OFI_AMD_GIN_POST_ACK 3   /* fi_send of the 8-byte ACK */
+#define OFI_AMD_GIN_POST_READ 4  /* fi_read of one stripe of a get */
 
 typedef struct {
 	uint32_t kind;
@@ -476,7 +499,7 @@ typedef struct {
 	uint32_t context; /* completion context: the fabric returns it through cq_read */
 	uint32_t peer;
 	uint32_t imm;     /* write: immediate data */
-	uint64_t src;     /* write */
+	uint64_t src;     /* write: local source; read: local buffer the bytes land in */
 	uint64_t len;
 	uint64_t dest;
 	uint64_t key;
@@ -520,6 +543,11 @@ int ofi_amd_gin_tx_destroy(ofi_amd_gin_tx_t *tx);
  * post (the operation is given up as the reference does: what was posted completes unobserved). */
 int ofi_amd_gin_tx_iput_signal(ofi_amd_gin_tx_t *tx, uint32_t peer, const ofi_amd_gin_wire_t *wire,
 			       int32_t *request);
+/* iget below its derivation (:879-939): one read per stripe of *wire (a record of
+ * ofi_amd_gin_iget), each a request of the pool, refused posts queued like any other; *request
+ * is done once every read has completed.  Return values as ofi_amd_gin_tx_iput_signal. */
+int ofi_amd_gin_tx_iget(ofi_amd_gin_tx_t *tx, uint32_t peer, const ofi_amd_gin_wire_t *wire,
+			int32_t *request);
 /* send_ack: one ACK send on rail 0. */
 int ofi_amd_gin_tx_send_ack(ofi_amd_gin_tx_t *tx, uint32_t peer, uint64_t ack_msg);
 /* nccl_ofi_gin_resources::progress. */
@@ -611,7 +639,7 @@ int ofi_amd_gin_signal_apply(const ofi_amd_gin_signal_work_t *d_work, uint32_t n
 /*
  * In-process loop-back of the whole GIN path on one GPU: initiator and target are the same
  * device, the "network" is this call.  For every descriptor drained from the rings it
- *   1. derives the wire record (ofi_amd_gin_iput_signal on comms[context], ack_model 0),
+ *   1. derives the wire record (ofi_amd_gin_derive on comms[context], ack_model 0),
  *   2. posts it through the progress engine (ofi_amd_gin_tx_*) into the in-process fabric
  *      (ofi_amd_loopfab_*, sq_depth entries per rail; 0 = 4096): refused posts are queued and
  *      retried by the engine's progress calls -- one every progress_interval operations (0
@@ -622,7 +650,9 @@ int ofi_amd_gin_signal_apply(const ofi_amd_gin_signal_work_t *d_work, uint32_t n
  *      the destination MR's remote_address_offset the device address of the target buffer) --
  *      long writes cut into 64 KiB pieces; the write completions and the metadata message go
  *      to a receiver (ofi_amd_gin_rx_*, one peer per context), up to reorder_window events
- *      out of order,
+ *      out of order; each RDMA read of a get as the copy the other way -- from the read's
+ *      `dest` (the remote MR's remote_address_offset + offset) into the local buffer -- of
+ *      which the receiver hears nothing,
  *   4. sends the receiver's ACKs back through the same engine and fabric; an ACK that arrives
  *      moves the sender's window (ofi_amd_gin_apply_ack),
  * and every batch_writes queued copies (and at the end) launches, in this order on `stream`,
@@ -648,6 +678,7 @@ typedef struct {
 	uint64_t tx_completions;  /* initiator completions read from the CQs */
 	uint32_t pending_max;     /* longest the pending list got */
 	uint32_t requests_max;    /* most request-pool entries in use */
+	uint64_t reads;           /* RDMA reads of gets */
 } ofi_amd_gin_loopback_stats_t;
 
 int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *rings, uint64_t ops_per_context,

@@ -21,6 +21,10 @@
  *                    outstanding; 15 + 1 doorbell batches; pin redirect cases).  The
  *                    reference has no wire-level test and its source does not build
  *                    here, so nothing beyond those cases and the encoders pins it
+ *   gin iget         reads of four gets worked out by hand (stripe counts, rails, lengths,
+ *                    local and remote addresses, keys), the scheduler shared with the
+ *                    puts, window / sequence / pin untouched, a full window that holds
+ *                    puts back but not gets.  The reference has no wire-level test of it
  *   gin receiver     end values of tests/functional/rma.cpp (64 put-signals -> 64)
  *                    and rma_multiseg_signal.cpp (two slots, each its count)
  *                    under arbitrary arrival orders; hand-derived fold runs;
@@ -31,7 +35,8 @@
  *                    runs, the 14-bit cursor wrap and per-peer comm ids
  *   gin tx engine    post / retry / completion orders worked out by hand against scripted
  *                    fabrics (full send queues, FI_MORE dropped on retry, head-of-line stop of
- *                    the retry, 16 completions per rail per progress call)
+ *                    the retry, 16 completions per rail per progress call); a get's reads
+ *                    the same way (refused read queued, failed read gives the get up)
  *   gin signal apply per-slot sums against a plain scatter-add (mod 2^64)
  *   region geometry  ~70 points + 4 extend_region cases of
  *                    tests/unit/region_based_tuner.cpp
@@ -233,12 +238,15 @@ void oracle_gin_comm_init(oracle_gin_comm_t *c, uint32_t comm_id, uint32_t num_r
  * -11 (window full and no ACK can arrive). */
 int oracle_gin_iput_signal(oracle_gin_comm_t *c, const oracle_gin_mr_t *mrs,
 			   const oracle_gin_desc_t *d, oracle_gin_wire_t *out);
+int oracle_gin_iget(oracle_gin_comm_t *c, const oracle_gin_mr_t *mrs, const oracle_gin_desc_t *d,
+		    oracle_gin_wire_t *out);
 void oracle_gin_apply_ack(oracle_gin_comm_t *c, uint32_t wire_rx_consumed);
 
 /* ---- initiator below the derivation (oracle_gin_tx.c): posts, pending retry, CQ drain ---- */
 #define ORACLE_GIN_POST_WRITE 1
 #define ORACLE_GIN_POST_META 2
 #define ORACLE_GIN_POST_ACK 3
+#define ORACLE_GIN_POST_READ 4
 typedef struct {
 	uint32_t kind, rail, more, context, peer, imm;
 	uint64_t src, len, dest, key;
@@ -260,6 +268,8 @@ oracle_gin_tx_t *oracle_gin_tx_create(uint32_t num_rails, uint32_t cq_read_count
 void oracle_gin_tx_destroy(oracle_gin_tx_t *tx);
 int oracle_gin_tx_iput_signal(oracle_gin_tx_t *tx, uint32_t peer, const oracle_gin_wire_t *wire,
 			      int32_t *request);
+int oracle_gin_tx_iget(oracle_gin_tx_t *tx, uint32_t peer, const oracle_gin_wire_t *wire,
+		       int32_t *request);
 int oracle_gin_tx_send_ack(oracle_gin_tx_t *tx, uint32_t peer, uint64_t ack_msg);
 int oracle_gin_tx_progress(oracle_gin_tx_t *tx);
 int oracle_gin_tx_test(oracle_gin_tx_t *tx, int32_t request, int *done);

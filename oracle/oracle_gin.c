@@ -258,6 +258,31 @@ int oracle_gin_iput_signal(oracle_gin_comm_t *c, const oracle_gin_mr_t *mrs,
 	return 0;
 }
 
+/* nccl_ofi_rdma_gin_put_comm::iget, src/rdma/gin/nccl_ofi_gin.cpp:879-939, down to the
+ * arguments of its reads.  Descriptor fields: src_off / src_mr = remoteOff / remoteMhandle,
+ * dst_off / dst_mr = localOff / localMhandle. */
+int oracle_gin_iget(oracle_gin_comm_t *c, const oracle_gin_mr_t *mrs, const oracle_gin_desc_t *d,
+		    oracle_gin_wire_t *out)
+{
+	memset(out, 0, sizeof(*out));
+	const oracle_gin_mr_t *remote_mr = &mrs[d->src_mr];
+	const oracle_gin_mr_t *local_mr = &mrs[d->dst_mr];
+	oracle_xfer_t xfers[ORACLE_MAX_RAILS];
+	/* :899, the endpoint's scheduler: the one the puts use */
+	uint32_t num_xfers = (uint32_t)oracle_sched_get_schedule(&c->sched, d->size, 128, xfers);
+	for (uint32_t i = 0; i < num_xfers; i++) { /* :903-932 */
+		oracle_gin_write_t *r = &out->writes[i];
+		r->rail = xfers[i].rail_id;
+		r->src = local_mr->local_base + d->dst_off + xfers[i].offset;               /* :905-906 */
+		r->len = xfers[i].msg_size;
+		r->dest = remote_mr->remote_address_offset + d->src_off + xfers[i].offset;  /* :908 */
+		r->key = remote_mr->key[r->rail];                                            /* :915 */
+		r->more = 0;
+	}
+	out->num_writes = num_xfers;
+	return 0;
+}
+
 /* handle_ack_completion, src/rdma/gin/nccl_ofi_gin.cpp:1843-1869, with apply_rx_consumed,
  * include/rdma/gin/nccl_ofi_gin.h:535-543: a wire cursor moves the tail forward only, and
  * by at most half the cursor space; a pending ACK request is satisfied by any cursor at or

@@ -203,6 +203,58 @@ int oracle_gin_tx_iput_signal(oracle_gin_tx_t *tx, uint32_t peer, const oracle_g
 	return 0;
 }
 
+/* nccl_ofi_rdma_gin_put_comm::iget below its schedule, src/rdma/gin/nccl_ofi_gin.cpp:895-938:
+ * an umbrella request, one read request per stripe with a back pointer to the umbrella's
+ * flag (:918-920), -FI_EAGAIN -> add_pending_req (:923-924), any other failure gives the
+ * operation up (:925-931).  The reference leaves the failed read request out of the pool on
+ * that path; it is returned here, as the product does. */
+int oracle_gin_tx_iget(oracle_gin_tx_t *tx, uint32_t peer, const oracle_gin_wire_t *wire,
+		       int32_t *request)
+{
+	*request = -1;
+	if (tx->n_free < 1 + wire->num_writes) {
+		return -12;
+	}
+	int op = req_alloc(tx);
+	tx->reqs[op].use = REQ_OP;
+	int posted[ORACLE_MAX_RAILS];
+	int n_posted = 0;
+	for (uint32_t i = 0; i < wire->num_writes; i++) {
+		const oracle_gin_write_t *w = &wire->writes[i];
+		int rd = req_alloc(tx);
+		oreq_t *r = &tx->reqs[rd];
+		r->use = REQ_POST;
+		r->parent = op;
+		r->flag = (int)i;
+		r->post.kind = ORACLE_GIN_POST_READ;
+		r->post.rail = w->rail;
+		r->post.more = 0;
+		r->post.context = (uint32_t)rd;
+		r->post.peer = peer;
+		r->post.src = w->src;   /* local_buf */
+		r->post.len = w->len;
+		r->post.dest = w->dest; /* remote_offset */
+		r->post.key = w->key;
+		tx->reqs[op].reqs_pending[i] = 1;
+		posted[n_posted++] = rd;
+		int ret = req_post(tx, rd);
+		if (ret == -11) {
+			add_pending_req(tx, rd);
+		} else if (ret != 0) {
+			for (int k = 0; k < n_posted - 1; k++) {
+				tx->reqs[posted[k]].parent = -1;
+			}
+			req_free(tx, rd);
+			req_free(tx, op);
+			return ret;
+		} else {
+			tx->st.posts++;
+		}
+	}
+	*request = op;
+	return 0;
+}
+
 int oracle_gin_tx_send_ack(oracle_gin_tx_t *tx, uint32_t peer, uint64_t ack_msg)
 {
 	int ar = req_alloc(tx);

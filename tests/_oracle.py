@@ -153,6 +153,7 @@ _ORACLE_PROTOS = {
     "oracle_gin_tx_destroy": (None, [ctypes.c_void_p]),
     "oracle_gin_tx_iput_signal": (c_int, [ctypes.c_void_p, c_u32, ctypes.POINTER(GinWire),
                                           ctypes.POINTER(c_i32)]),
+    "oracle_gin_tx_iget": (c_int, [ctypes.c_void_p, c_u32, ctypes.POINTER(GinWire), ctypes.POINTER(c_i32)]),
     "oracle_gin_tx_send_ack": (c_int, [ctypes.c_void_p, c_u32, c_u64]),
     "oracle_gin_tx_progress": (c_int, [ctypes.c_void_p]),
     "oracle_gin_tx_test": (c_int, [ctypes.c_void_p, c_i32, ctypes.POINTER(c_int)]),
@@ -181,6 +182,8 @@ _ORACLE_PROTOS = {
     "oracle_gin_comm_init": (None, [ctypes.POINTER(GinComm), c_u32, c_u32, c_u64, c_u64, c_u32]),
     "oracle_gin_iput_signal": (c_int, [ctypes.POINTER(GinComm), ctypes.POINTER(GinMr),
                                        ctypes.POINTER(GinDesc), ctypes.POINTER(GinWire)]),
+    "oracle_gin_iget": (c_int, [ctypes.POINTER(GinComm), ctypes.POINTER(GinMr), ctypes.POINTER(GinDesc),
+                                ctypes.POINTER(GinWire)]),
     "oracle_gin_apply_ack": (None, [ctypes.POINTER(GinComm), c_u32]),
     "oracle_gin_rx_create": (c_vp, [c_u32, ctypes.POINTER(c_u32)]),
     "oracle_gin_rx_destroy": (None, [c_vp]),

@@ -144,6 +144,51 @@ def test_proxy_mode_two_derives_without_folding_the_wire_records(lib, oracle, gp
                                                           _oracle.default_mrs())
 
 
+def test_proxy_derives_gets_among_puts_like_the_oracle(lib, oracle, gpu):
+    """A table in which every third descriptor is a get goes through the device-side put, the ring
+    and the proxy's derivation (mode 2); every wire record and the final comm state equal what
+    the oracle derives from the same descriptors one by one."""
+    ops, cap = 3000, 512
+    rng = np.random.default_rng(99)
+    table = np.zeros((1, ops, 8), dtype=np.uint64)
+    for i in range(ops):
+        size = int(2 ** rng.uniform(0, 21))
+        if i % 3 == 2:      # get: remote handle 2, local handle 0
+            table[0, i] = [int(rng.integers(0, 1 << 30)), int(rng.integers(0, 1 << 30)), size, 0, 0, 1, 0,
+                           2 | (0 << 16) | (0xFFFF << 32) | (3 << 48)]
+        else:
+            sop = 1 if i % 7 == 0 else 0
+            table[0, i] = [int(rng.integers(0, 1 << 30)), int(rng.integers(0, 1 << 30)), size, 8 * (i % 16) if sop else 0,
+                           0, 1 | (sop << 32), int(rng.integers(0, 2)),
+                           0 | (1 << 16) | ((2 if sop else 0xFFFF) << 32) | ((2 if sop else 1) << 48)]
+    d_table = _gpu.to_dev(table)
+    rings = make_rings(lib, 1, cap)
+    comms = (m.GinComm * 1)()
+    assert lib.ofi_amd_gin_comm_init(ctypes.byref(comms[0]), 9, 4, 131072, 64, 1) == 0
+    pmrs, omrs = _oracle.default_mrs(m.GinMr), _oracle.default_mrs()
+    wires = (m.GinWire * ops)()
+    assert lib.ofi_amd_gin_produce_table(rings, d_table.data_ptr(), ops, 1, 0, _gpu.stream()) == 0
+    stats = m.GinProxyStats()
+    rc = lib.ofi_amd_gin_proxy_drain(rings, ops, 2, None, ctypes.cast(comms, ctypes.c_void_p),
+                                     ctypes.cast(pmrs, ctypes.c_void_p), 3, ctypes.cast(wires, ctypes.c_void_p),
+                                     5000, ctypes.byref(stats))
+    _gpu.sync()
+    assert rc == 0 and stats.descriptors == ops
+    oc = _oracle.GinComm()
+    oracle.oracle_gin_comm_init(ctypes.byref(oc), 9, 4, 131072, 64, 1)
+    n_reads = 0
+    for i in range(ops):
+        d = _oracle.GinDesc.from_buffer_copy(table[0, i].tobytes())
+        w = _oracle.GinWire()
+        fn = oracle.oracle_gin_iget if d.kind == 3 else oracle.oracle_gin_iput_signal
+        assert fn(ctypes.byref(oc), omrs, ctypes.byref(d), ctypes.byref(w)) == 0
+        assert bytes(w) == bytes(wires[i]), i
+        n_reads += w.num_writes if d.kind == 3 else 0
+    assert bytes(oc) == bytes(comms[0]) and comms[0].tx_head == ops - ops // 3
+    assert n_reads > ops // 3
+    lib.ofi_amd_gin_rings_destroy(rings)
+
+
 def test_proxy_stops_at_a_descriptor_with_a_handle_outside_the_table(lib, gpu):
     """The handle indices of a record are written by device code; the proxy checks them against the
     registration table it was given and ends the drain with -EINVAL instead of reading past it."""

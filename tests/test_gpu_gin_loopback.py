@@ -132,6 +132,90 @@ def test_puts_and_signals_arrive_bit_exact(lib, gpu, nctx, ops, waves, reorder, 
     lib.ofi_amd_gin_rings_destroy(rings)
 
 
+def test_gets_land_bit_exact_beside_puts(lib, gpu):
+    """Every fourth operation is a get (iget, src/rdma/gin/nccl_ofi_gin.cpp:879-939): its reads come
+    back as copies from the peer's registration into a local landing buffer.  Gets use the same
+    scheduler as the puts, but no sequence number: the window counts the puts only, the receiver
+    hears of the puts only, and every read completes on the initiator."""
+    rng = np.random.default_rng(4242)
+    nctx, ops = 3, 2000
+    src_bytes = 16 << 20
+    src = rng.integers(0, 256, src_bytes, dtype=np.uint8)
+    remote = rng.integers(0, 256, src_bytes, dtype=np.uint8)      # what the gets read
+    table, replay, dst_bytes = build_ops(rng, nctx, ops, src_bytes, 300_000)
+    land_pos, gets, want_reads = 0, [], 0
+    for c in range(nctx):
+        for i in range(3, ops, 4):
+            size = int(2 ** rng.uniform(0, 19.5)) if rng.random() < 0.9 else 0
+            remote_off = int(rng.integers(0, src_bytes - size))
+            local_off = land_pos + int(rng.integers(0, 24))
+            land_pos = local_off + size + int(rng.integers(0, 8))
+            # remote handle 3, local handle 4, kind 3
+            table[c, i] = [remote_off, local_off, size, 0, 0, 1, (c << 32), 3 | (4 << 16) | (0xFFFF << 32) | (3 << 48)]
+            replay[c * ops + i] = None
+            gets.append((remote_off, local_off, size))
+            want_reads += 1 if size <= 131072 else (2 if size <= 393216 else 4)
+    d_src, d_remote = _gpu.to_dev(src), _gpu.to_dev(remote)
+    d_dst = torch.full((dst_bytes,), 0xEE, dtype=torch.uint8, device="cuda")
+    d_land = torch.full((land_pos + 64,), 0xDD, dtype=torch.uint8, device="cuda")
+    start = rng.integers(0, 1 << 63, N_SLOTS, dtype=np.uint64)
+    d_cnt = _gpu.to_dev(start)
+    d_table = _gpu.to_dev(table)
+
+    mrs = (m.GinMr * 5)()
+    mrs[0].local_base = d_src.data_ptr()
+    mrs[1].remote_address_offset = d_dst.data_ptr()
+    mrs[2].remote_address = SIG_BASE
+    mrs[3].remote_address_offset = d_remote.data_ptr()            # the peer's memory the gets read
+    mrs[4].local_base = d_land.data_ptr()                          # where they land
+    for i in range(5):
+        for r in range(4):
+            mrs[i].key[r] = 0x100 * (i + 1) + r
+    comms = (m.GinComm * nctx)()
+    for c in range(nctx):
+        assert lib.ofi_amd_gin_comm_init(ctypes.byref(comms[c]), 100 + c, 4, 131072, 64, 0) == 0
+    regions = (m.GinSignalRegion * 1)(m.GinSignalRegion(SIG_BASE, 8 * N_SLOTS, d_cnt.data_ptr()))
+    rings = ctypes.c_void_p()
+    assert lib.ofi_amd_gin_rings_create(nctx, 1024, ctypes.byref(rings)) == 0
+    assert lib.ofi_amd_gin_produce_table(rings, d_table.data_ptr(), ops, 2, 0, _gpu.stream()) == 0
+    stats = m.GinLoopbackStats()
+    side = torch.cuda.Stream()
+    rc = lib.ofi_amd_gin_loopback_run(rings, ops, ctypes.cast(comms, ctypes.c_void_p),
+                                      ctypes.cast(mrs, ctypes.c_void_p), len(mrs), regions, 1, 50, 512, 8, 16,
+                                      20000, ctypes.c_void_p(side.cuda_stream), ctypes.byref(stats))
+    torch.cuda.synchronize()
+    assert rc == 0 and lib.ofi_amd_gin_producer_status(rings) == 0
+
+    want = np.full(dst_bytes, 0xEE, dtype=np.uint8)
+    counters = [int(x) for x in start]
+    n_signals = n_puts = 0
+    for r in replay:
+        if r is None:
+            continue
+        src_off, dst_off, size, sop, sval, slot = r
+        n_puts += 1
+        want[dst_off:dst_off + size] = src[src_off:src_off + size]
+        if sop:
+            counters[slot] = (counters[slot] + (1 if sop == 1 else sval)) % (1 << 64)
+            n_signals += 1
+    want_land = np.full(land_pos + 64, 0xDD, dtype=np.uint8)
+    for remote_off, local_off, size in gets:
+        want_land[local_off:local_off + size] = remote[remote_off:remote_off + size]
+    assert np.array_equal(d_dst.cpu().numpy(), want)
+    assert np.array_equal(d_land.cpu().numpy(), want_land)
+    assert [int(x) for x in _gpu.to_host(d_cnt, np.uint64)] == counters
+
+    assert stats.descriptors == nctx * ops and stats.signals == n_signals
+    assert stats.reads == want_reads
+    assert stats.bytes == sum(r[2] for r in replay if r) + sum(g[2] for g in gets)
+    for c in range(nctx):
+        assert comms[c].tx_head == n_puts // nctx                 # the puts only
+    assert stats.tx_completions == stats.writes + stats.signals + stats.acks + stats.reads
+    assert stats.posts_refused > 0
+    assert _gpu.fetch_async_errors(lib) == 0
+    lib.ofi_amd_gin_rings_destroy(rings)
+
+
 def test_copy_table_matches_a_host_replay(lib, gpu):
     """The loop-back's data mover by itself: address triples at any alignment and length."""
     rng = np.random.default_rng(5)
