@@ -102,6 +102,37 @@ def test_model_variants_and_odd_axes(lib, oracle, gpu):
     lib.ofi_amd_tuner_plan_destroy(plan)
 
 
+@pytest.mark.parametrize("n_nodes,n_ppn", [(51, 5), (64, 4), (257, 1), (40, 8), (1, 1)])
+def test_model_grid_on_wide_and_narrow_axes(lib, oracle, gpu, n_nodes, n_ppn):
+    """Many (node count, ranks per node) pairs per size, or a single one; an algorithm list without
+    a PAT column but with NVLS tree; three variants, one on a platform without a model.  The
+    oracle's bits, also when only one of the two outputs is asked for."""
+    rng = np.random.default_rng(n_nodes * 10 + n_ppn)
+    colls = np.array([4, 3], dtype=np.int32)
+    sizes = np.unique((2 ** rng.uniform(0, 36, 7)).astype(np.uint64))
+    nodes = np.arange(1, n_nodes + 1, dtype=np.uint64) * np.uint64(3)
+    ppn = np.array([1, 2, 4, 8, 3, 5, 6, 7][:n_ppn], dtype=np.uint32)
+    algos = np.array([1, 0, 5], dtype=np.int32)                      # Ring, Tree, NVLS tree: no PAT column
+    plan = make_plan(lib, colls, sizes, nodes, ppn, algos)
+    variants = [m.TunerVariant(0, 2, 8, 3), m.TunerVariant(1, 1, 4, 1), m.TunerVariant(3, 1, 8, 3)]
+    shape = (3, 2, len(sizes), n_nodes, n_ppn, 3)
+    want_cost, want_choice = oracle_model_grid(oracle, variants, colls, sizes, nodes, ppn, algos)
+    cost, choice = run_model(lib, plan, variants, shape)
+    assert np.array_equal(cost.astype(np.float32).view(np.uint32), want_cost.view(np.uint32))
+    assert np.array_equal(choice, want_choice)
+    # one output at a time
+    nv, cells, points = 3, lib.ofi_amd_tuner_plan_cells(plan), lib.ofi_amd_tuner_plan_points(plan)
+    arr = (m.TunerVariant * nv)(*variants)
+    d_cost = torch.full((nv * cells,), 7.0, dtype=torch.float64, device="cuda")
+    d_choice = torch.full((nv * points * 2,), 99, dtype=torch.int8, device="cuda")
+    assert lib.ofi_amd_tuner_model_grid(plan, arr, nv, d_cost.data_ptr(), None, _gpu.stream()) == 0
+    assert lib.ofi_amd_tuner_model_grid(plan, arr, nv, None, d_choice.data_ptr(), _gpu.stream()) == 0
+    _gpu.sync()
+    assert np.array_equal(d_cost.cpu().numpy().reshape(shape + (3,)), cost)
+    assert np.array_equal(d_choice.cpu().numpy().reshape(shape[:-1] + (2,)), choice)
+    lib.ofi_amd_tuner_plan_destroy(plan)
+
+
 def oracle_region_grid(oracle, platforms, colls, sizes, nodes, ppn):
     out = np.zeros((len(platforms), len(colls), len(sizes), len(nodes), len(ppn), 3), np.int32)
     a, p, ch = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
