@@ -1,6 +1,7 @@
 /*
- * Device side of the GIN descriptor rings: what a HIP kernel calls to initiate a put or
- * put-signal.  Compile with hipcc for gfx950; host code only needs ofi_amd_hotpath.h.
+ * Device side of the GIN descriptor rings: what a HIP kernel calls to initiate a put, a
+ * put-signal or a get (a descriptor of kind OFI_AMD_GIN_KIND_GET travels the same way).
+ * Compile with hipcc for gfx950; host code only needs ofi_amd_hotpath.h.
  *
  * The reference has no such call on AMD or in proxy mode -- NCCL's own GPU-to-CPU queue
  * feeds its proxy thread, which calls iputSignal (src/rdma/gin/nccl_ofi_gin_api.cpp:370-419);
