@@ -47,6 +47,32 @@ def test_noalloc_matches_allocating_entry_point(lib, oracle, gpu):
         assert _gpu.fetch_async_errors(lib) == 0
 
 
+def test_noalloc_at_its_largest_batch(lib, gpu):
+    """2^26 messages use every tile word of the fixed scratch (32,768 tiles of 2,048).  Compared on
+    the device with the allocating entry point's output for the same batch (6.4 GB of rows each),
+    and through what does not depend on the size: every message's stripes add up to its size."""
+    assert lib.ofi_amd_gpu_init() == 0
+    n = 1 << 26
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    octave = torch.randint(0, 28, (n,), generator=gen, device="cuda", dtype=torch.int64)
+    d_sizes = (torch.randint(0, 1 << 28, (n,), generator=gen, device="cuda", dtype=torch.int64) >> (28 - octave))
+    outs = []
+    for fn in (lib.ofi_amd_sched_batch_noalloc, lib.ofi_amd_sched_batch):
+        d_state = dev_state(4, 131072, 64, (2, 3))
+        d_num = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+        d_xf = torch.full((n * 12,), -1, dtype=torch.int64, device="cuda")
+        assert fn(d_state.data_ptr(), d_sizes.data_ptr(), n, 128, d_num.data_ptr(), d_xf.data_ptr(),
+                  _gpu.stream()) == 0
+        _gpu.sync()
+        outs.append((d_num, d_xf, d_state))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    assert torch.equal(outs[0][2], outs[1][2])
+    rows = outs[0][1].view(n, 4, 3)
+    assert torch.equal(rows[:, :, 2].sum(dim=1), d_sizes)
+    assert int(outs[0][0].min()) == 1 and int(outs[0][0].max()) == 4
+    assert _gpu.fetch_async_errors(lib) == 0
+
+
 def test_noalloc_rejects_oversized_batch(lib, gpu):
     assert lib.ofi_amd_gpu_init() == 0
     d = torch.zeros(16, dtype=torch.int64, device="cuda")
