@@ -168,6 +168,58 @@ def test_full_size_configuration(lib, oracle, gpu):
     assert set(np.unique(num)) <= {1, 2, 4}
 
 
+def test_largest_batch_against_a_prefix_sum_in_torch(lib, gpu):
+    """2^28 messages, the most one call takes (131,072 tiles, 29 GB of output): too large for the
+    scalar oracle's output to be held and compared, so the batch formulation is restated with
+    torch on the device -- stripe counts from the thresholds, start rails from exclusive prefix
+    sums of the two counters mod the rail count -- and every row is compared with it; lengths,
+    offsets and padding through what holds at any size."""
+    n, rails, seeds = 1 << 28, 4, (3, 2)
+    gen = torch.Generator(device="cuda").manual_seed(17)
+    octave = torch.randint(0, 28, (n,), generator=gen, device="cuda", dtype=torch.int64)
+    d_sizes = torch.randint(0, 1 << 28, (n,), generator=gen, device="cuda", dtype=torch.int64) >> (28 - octave)
+    del octave
+    d_state = dev_state(rails, 131072, 64, seeds)
+    d_num = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+    d_xf = torch.full((n * 12,), -1, dtype=torch.int64, device="cuda")
+    assert lib.ofi_amd_sched_batch(d_state.data_ptr(), d_sizes.data_ptr(), n, 128, d_num.data_ptr(),
+                                   d_xf.data_ptr(), _gpu.stream()) == 0
+    _gpu.sync()
+    assert _gpu.fetch_async_errors(lib) == 0
+    small = d_sizes < 64
+    want = torch.clamp((d_sizes + 131071) >> 17, 1, 4)            # ceil(size / 128 KiB), 1..4
+    want = torch.where(want == 3, torch.full_like(want, 2), want)  # 3 does not divide 4 rails
+    want = torch.where(small, torch.ones_like(want), want)
+    assert torch.equal(d_num.to(torch.int64), want)
+    big_steps = torch.where(small, torch.zeros_like(want), want)
+    first_rail = torch.where(small,
+                             (seeds[0] + torch.cumsum(small.to(torch.int64), 0) - small.to(torch.int64)) % rails,
+                             (seeds[1] + torch.cumsum(big_steps, 0) - big_steps) % rails)
+    rows = d_xf.view(n, 4, 3)
+    for k in range(4):
+        used = want > k
+        assert torch.equal(rows[:, k, 0], torch.where(used, (first_rail + k) % rails, torch.zeros_like(want)))
+        if k == 0:
+            assert int(rows[:, 0, 1].abs().max()) == 0          # the first stripe starts at 0
+        else:
+            # a used stripe starts where the one before it ends; unused entries are all zero
+            assert torch.equal(rows[:, k, 1], torch.where(used, rows[:, k - 1, 1] + rows[:, k - 1, 2],
+                                                           torch.zeros_like(want)))
+            assert int(rows[:, k, 2][~used].abs().max()) == 0
+        del used
+    assert torch.equal(rows[:, :, 2].sum(dim=1), d_sizes)
+    # every stripe but a message's last is a multiple of the alignment
+    for k in range(3):
+        not_last = want > k + 1
+        assert int((rows[:, k, 2][not_last] % 128).max()) == 0
+    st = read_state(d_state)
+    assert st.rr_small_counter == (seeds[0] + int(small.sum())) % rails
+    assert st.rr_counter == (seeds[1] + int(big_steps.sum())) % rails
+    # one more than the most: refused, nothing launched
+    assert lib.ofi_amd_sched_batch(d_state.data_ptr(), d_sizes.data_ptr(), n + 1, 128, d_num.data_ptr(),
+                                   d_xf.data_ptr(), _gpu.stream()) == -22
+
+
 def test_batches_on_two_streams_do_not_share_scratch(lib, oracle, gpu):
     """Two scheduler instances driven from two streams at once (two endpoints in one process):
     each stream has its own tile scratch, so overlapping launches cannot mix their seeds."""
