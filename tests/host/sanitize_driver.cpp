@@ -503,8 +503,18 @@ void run_gin_tx(uint64_t seed, uint32_t n_ops, uint32_t ack_model)
 		ofi_amd_gin_wire_t wb;
 		std::memset(&wa, 0, sizeof(wa));
 		std::memset(&wb, 0, sizeof(wb));
-		const int ra = oracle_gin_iput_signal(&ca, mrs, &d, &wa);
-		SAME("iput rc", ra, ofi_amd_gin_iput_signal(&cb, mrs_b, 3, &db, &wb));
+		int ra;
+		if (rng.chance(15)) { /* a get: remote handle 1, local handle 0 */
+			d.kind = db.kind = 3;
+			d.src_mr = db.src_mr = 1;
+			d.dst_mr = db.dst_mr = 0;
+			d.signal_op = db.signal_op = 0;
+			ra = oracle_gin_iget(&ca, mrs, &d, &wa);
+			SAME("iget rc", ra, ofi_amd_gin_derive(&cb, mrs_b, 3, &db, &wb));
+		} else {
+			ra = oracle_gin_iput_signal(&ca, mrs, &d, &wa);
+			SAME("iput rc", ra, ofi_amd_gin_iput_signal(&cb, mrs_b, 3, &db, &wb));
+		}
 		if (ra == 0) {
 			SAME("wire record", std::memcmp(&wa, &wb, sizeof(wa)), 0);
 		} else if (ra == -11) { /* window full: the receiver has consumed up to some point */
@@ -514,6 +524,149 @@ void run_gin_tx(uint64_t seed, uint32_t n_ops, uint32_t ack_model)
 		}
 		SAME("comm state", std::memcmp(&ca, &cb, sizeof(ca)), 0);
 	}
+}
+
+/* ------------------------------------------------- GIN transmit engine (posts, retry, CQ) */
+
+/* A fabric with a bounded send queue per rail; everything done to it is logged. */
+struct sim_fabric_t {
+	uint32_t depth;
+	std::deque<uint32_t> sq[4], cq[4];
+	std::vector<uint64_t> log;
+	uint64_t attempts = 0, fail_every = 0;
+	template <typename P>
+	int post(const P *p)
+	{
+		attempts++;
+		log.push_back(((uint64_t)p->kind << 56) | ((uint64_t)p->rail << 48) | ((uint64_t)p->more << 40) |
+			      ((uint64_t)p->context << 8));
+		log.push_back(p->src ^ (p->len << 1) ^ (p->dest << 2) ^ (p->key << 3) ^ p->msg[0] ^ p->imm ^ p->peer);
+		if (fail_every && attempts % fail_every == 0) {
+			log.push_back(5);
+			return -5;
+		}
+		if (sq[p->rail].size() >= depth) {
+			log.push_back(11);
+			return -11;
+		}
+		sq[p->rail].push_back(p->context);
+		return 0;
+	}
+	int cq_read(uint32_t rail, uint32_t *contexts, uint32_t max)
+	{
+		uint32_t n = 0;
+		while (n < max && !cq[rail].empty()) {
+			contexts[n++] = cq[rail].front();
+			cq[rail].pop_front();
+		}
+		log.push_back(0xC000000000000000ull | ((uint64_t)rail << 32) | n);
+		return (int)n;
+	}
+	void complete_some(rng_t &rng)
+	{
+		for (int r = 0; r < 4; r++) {
+			while (!sq[r].empty() && rng.chance(60)) {
+				cq[r].push_back(sq[r].front());
+				sq[r].pop_front();
+			}
+		}
+	}
+};
+
+int oracle_post_cb(void *f, const oracle_gin_post_t *p) { return static_cast<sim_fabric_t *>(f)->post(p); }
+int oracle_cq_cb(void *f, uint32_t rail, uint32_t *c, uint32_t max) { return static_cast<sim_fabric_t *>(f)->cq_read(rail, c, max); }
+int product_post_cb(void *f, const ofi_amd_gin_post_t *p) { return static_cast<sim_fabric_t *>(f)->post(p); }
+int product_cq_cb(void *f, uint32_t rail, uint32_t *c, uint32_t max) { return static_cast<sim_fabric_t *>(f)->cq_read(rail, c, max); }
+
+void run_gin_engine(uint64_t seed, uint32_t n_ops)
+{
+	rng_t rng{ seed };
+	static_assert(sizeof(oracle_gin_post_t) == sizeof(ofi_amd_gin_post_t), "post layouts");
+	static_assert(sizeof(oracle_gin_tx_stats_t) == sizeof(ofi_amd_gin_tx_stats_t), "stats layouts");
+	sim_fabric_t fa, fb;
+	fa.depth = fb.depth = 1 + rng.below(6);
+	fa.fail_every = fb.fail_every = rng.chance(50) ? 0 : 200 + rng.below(300);
+	const uint32_t pool = 24 + rng.below(64);
+	const uint32_t cq_count = 1 + rng.below(5), cq_iter = 1 + rng.below(4);
+	oracle_gin_fabric_ops_t oa = { oracle_post_cb, oracle_cq_cb, &fa };
+	ofi_amd_gin_fabric_ops_t ob = { product_post_cb, product_cq_cb, &fb };
+	oracle_gin_tx_t *a = oracle_gin_tx_create(4, cq_count, cq_iter, pool, &oa);
+	ofi_amd_gin_tx_t *b = nullptr;
+	SAME("tx create", a != nullptr, ofi_amd_gin_tx_create(4, cq_count, cq_iter, pool, &ob, &b) == 0);
+	std::vector<int32_t> open;
+	for (uint32_t i = 0; i < n_ops; i++) {
+		const uint32_t what = rng.below(100);
+		if (what < 55) { /* an operation: a put (writes, perhaps a metadata send) or a get (reads) */
+			const bool get = rng.chance(25);
+			oracle_gin_wire_t wa;
+			std::memset(&wa, 0, sizeof(wa));
+			wa.num_writes = get ? 1 + rng.below(4) : rng.below(5);
+			for (uint32_t k = 0; k < wa.num_writes; k++) {
+				wa.writes[k].rail = rng.below(4);
+				wa.writes[k].more = get ? 0 : rng.below(2);
+				wa.writes[k].src = rng.next();
+				wa.writes[k].len = rng.below(1u << 20);
+				wa.writes[k].dest = rng.next();
+				wa.writes[k].key = rng.next();
+			}
+			if (!get) {
+				wa.imm = (uint32_t)rng.next();
+				wa.nseg = wa.num_writes;
+				if (wa.num_writes == 0 || rng.chance(30)) {
+					wa.has_meta = 1;
+					wa.nseg++;
+					wa.meta_rail = rng.below(4);
+					wa.meta_more = rng.below(2);
+					for (int k = 0; k < 4; k++) {
+						wa.meta[k] = rng.next();
+					}
+				}
+			}
+			ofi_amd_gin_wire_t wb;
+			std::memcpy(&wb, &wa, sizeof(wb));
+			int32_t qa = -2, qb = -2;
+			const uint32_t peer = rng.below(8);
+			const int ra = get ? oracle_gin_tx_iget(a, peer, &wa, &qa) : oracle_gin_tx_iput_signal(a, peer, &wa, &qa);
+			const int rb = get ? ofi_amd_gin_tx_iget(b, peer, &wb, &qb) : ofi_amd_gin_tx_iput_signal(b, peer, &wb, &qb);
+			SAME("engine op rc", ra, rb);
+			SAME("engine request", qa, qb);
+			if (ra == 0) {
+				open.push_back(qa);
+			}
+		} else if (what < 65) {
+			const uint64_t msg = rng.next();
+			const uint32_t peer = rng.below(8);
+			SAME("send_ack rc", oracle_gin_tx_send_ack(a, peer, msg), ofi_amd_gin_tx_send_ack(b, peer, msg));
+		} else if (what < 85) {
+			rng_t ra{ rng.s }, rb{ rng.s };
+			fa.complete_some(ra);
+			fb.complete_some(rb);
+			rng.s = ra.s;
+			SAME("progress rc", oracle_gin_tx_progress(a), ofi_amd_gin_tx_progress(b));
+		} else if (!open.empty()) {
+			const size_t k = rng.below((uint32_t)open.size());
+			int da = -1, db = -1;
+			SAME("test rc", oracle_gin_tx_test(a, open[k], &da), ofi_amd_gin_tx_test(b, open[k], &db));
+			SAME("test done", da, db);
+			if (da == 1) {
+				open[k] = open.back();
+				open.pop_back();
+			}
+		}
+		SAME("fabric log length", fa.log.size(), fb.log.size());
+		if (fa.log != fb.log) {
+			fail("fabric logs differ", i);
+		}
+		fa.log.clear();
+		fb.log.clear();
+		oracle_gin_tx_stats_t sa;
+		ofi_amd_gin_tx_stats_t sb;
+		oracle_gin_tx_stats(a, &sa);
+		ofi_amd_gin_tx_stats(b, &sb);
+		SAME("engine stats", std::memcmp(&sa, &sb, sizeof(sa)), 0);
+	}
+	oracle_gin_tx_destroy(a);
+	ofi_amd_gin_tx_destroy(b);
 }
 
 } // namespace
@@ -532,6 +685,8 @@ int main(int argc, char **argv)
 		run_gin_rx(s, 20000);
 		run_gin_tx(s, 30000, 0);
 		run_gin_tx(s + 50, 30000, 1);
+		run_gin_engine(s, 20000);
+		run_gin_engine(s + 90, 20000);
 	}
 	std::printf("host state machines: oracle and product agree over %llu seeds\n", (unsigned long long)seeds);
 	return 0;
