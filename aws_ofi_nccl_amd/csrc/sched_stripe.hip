@@ -24,7 +24,7 @@
  *                           totals of the tiles before it by itself (at most 16 KiB
  *                           from L2) instead of waiting for a scan launch, and the
  *                           last workgroup writes the new counters back.
- * A tile is 512 messages for batches up to 2^21 messages and 2048 beyond.
+ * A tile is 512 messages for batches up to 2^21 messages and 1024 beyond.
  *
  * HBM traffic per message: 8 B read twice + 4 B + 96 B written.
  */
@@ -40,10 +40,16 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr uint32_t kThreads = 256;
 /* Messages per workgroup = kThreads * PASSES.  Small batches want many small tiles (the
- * launch is short, so ramp-up and tail dominate: 1,000,000 messages take 26.7 us with two
- * passes per workgroup against 29.4 with four); large ones want fewer, longer workgroups
- * (16,000,000: 348 us with eight passes against 360 with four). */
-constexpr uint32_t kPassesSmall = 2, kPassesLarge = 8;
+ * launch is short, so ramp-up and tail dominate: 1,000,000 messages take 22.2 us with two
+ * passes per workgroup against 24.4 with four); large ones want somewhat longer workgroups
+ * (16,000,000: 322-325 us with three or four passes, 332-334 with two, six or eight). */
+#ifndef OFI_STRIPE_PASSES_SMALL
+#define OFI_STRIPE_PASSES_SMALL 2
+#endif
+#ifndef OFI_STRIPE_PASSES_LARGE
+#define OFI_STRIPE_PASSES_LARGE 4
+#endif
+constexpr uint32_t kPassesSmall = OFI_STRIPE_PASSES_SMALL, kPassesLarge = OFI_STRIPE_PASSES_LARGE;
 constexpr uint64_t kSmallBatch = 1ull << 21;
 constexpr uint32_t kScanThreads = 1024;
 constexpr uint32_t kScanPer = 8; /* tiles per thread and round of the scan kernel */
@@ -439,7 +445,7 @@ std::unordered_map<void *, workspace_t> g_ws_by_stream;
  * The same scratch for callers that may not allocate: one array per GPU, part of the loaded
  * code object, held until the process ends.  Layout in 32-bit words:
  * [0, kNoAllocTiles) tile totals, [kNoAllocTiles, 2 * kNoAllocTiles) tile prefixes, then the
- * seed word.  kNoAllocMaxBatch messages need kNoAllocTiles tiles of 2048.  In host code the
+ * seed word.  kNoAllocMaxBatch messages need kNoAllocTiles tiles of 1024.  In host code the
  * array's name is only a handle for hipGetSymbolAddress; kernels get the address it returns.
  */
 constexpr uint64_t kNoAllocMaxBatch = 1ull << 26;

@@ -126,7 +126,7 @@ int ofi_amd_sched_batch(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes,
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
  * reference.  Same arguments, same results and the same kernels; the tile totals and prefixes
  * that ofi_amd_sched_batch keeps in a per-stream allocation live here in a fixed array inside
- * the library's device code (about 256 KiB per GPU, held until the process ends), so the call
+ * the library's device code (about 512 KiB per GPU, held until the process ends), so the call
  * allocates and frees nothing.  n <= 2^26 messages per call, -E2BIG beyond.  Call
  * ofi_amd_gpu_init() once beforehand (it allocates the asynchronous error word and looks up
  * the array's address on every GPU); -ENXIO otherwise.  All calls on one GPU share that GPU's

@@ -136,10 +136,10 @@ def test_bad_arguments(lib, gpu):
 
 @pytest.mark.parametrize("rails,seeds", [(4, (3, 2)), (3, (1, 2))])
 def test_batches_beyond_the_inline_prefix_limit(lib, oracle, gpu, rails, seeds):
-    """Batches up to 2^21 messages use 512-message tiles, larger ones 2048-message tiles; beyond 4096
+    """Batches up to 2^21 messages use 512-message tiles, larger ones 1024-message tiles; beyond 4096
     tiles the tile seeds come from the separate scan launch.  One message below and one above each
     boundary must chain exactly like the small form."""
-    for n in ((1 << 21), (1 << 21) + 1, 4096 * 2048, 4096 * 2048 + 1, 9_000_011):
+    for n in ((1 << 21), (1 << 21) + 1, 4096 * 1024, 4096 * 1024 + 1, 4096 * 2048 + 1, 9_000_011):
         sizes = synthetic.stripe_sizes(n + rails, n)
         want_num, want_xf, ost = _oracle.sched_batch(oracle, sizes, rails, 131072, 64, seeds)
         d_state = dev_state(rails, 131072, 64, seeds)

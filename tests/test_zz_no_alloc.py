@@ -31,7 +31,7 @@ def run(fn, d_state, d_sizes, n):
 def test_noalloc_matches_allocating_entry_point(lib, oracle, gpu):
     assert lib.ofi_amd_gpu_init() == 0
     # second call smaller than the first (stale totals of the first stay in the scratch),
-    # third call beyond 4096 tiles of 2048 messages: the scan launch and the prefix half
+    # third call beyond 4096 tiles of 1024 messages: the scan launch and the prefix half
     for seed, n in ((11, 300007), (12, 1234), (13, (1 << 23) + 4099)):
         sizes = synthetic.stripe_sizes(seed, n)
         sizes[::7] = sizes[::7] % np.uint64(150)
@@ -48,7 +48,7 @@ def test_noalloc_matches_allocating_entry_point(lib, oracle, gpu):
 
 
 def test_noalloc_at_its_largest_batch(lib, gpu):
-    """2^26 messages use every tile word of the fixed scratch (32,768 tiles of 2,048).  Compared on
+    """2^26 messages use every tile word of the fixed scratch (65,536 tiles of 1,024).  Compared on
     the device with the allocating entry point's output for the same batch (6.4 GB of rows each),
     and through what does not depend on the size: every message's stripes add up to its size."""
     assert lib.ofi_amd_gpu_init() == 0
