@@ -93,8 +93,6 @@ __global__ __launch_bounds__(256) void model_grid_kernel(grid_dims_t g,
 	}
 }
 
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-
 constexpr int kMaxSetPolys = 8;  /* polygons of one (platform, shape, collective) set */
 constexpr int kMaxSetVerts = 64; /* their vertices together */
 constexpr uint32_t kRegionBlock = 64; /* threads per workgroup of the region kernel: one wavefront */
@@ -103,10 +101,9 @@ static_assert(kRegionBlock >= (uint32_t)kMaxSetVerts && kRegionBlock >= (uint32_
 	      "one thread per staged vertex and per staged polygon word");
 
 /*
- * One thread per point.  A workgroup (one wavefront) works on
- * 64 points of one (collective, ranks per node) pair -- `blocks_per_run` chunks make up the
- * pair's n_sizes x n_nodes points, node count fastest -- because the polygon set depends on that
- * pair alone: the set (at most 8 polygons, 64 vertices, with their bounds) is copied into LDS
+ * One thread per point.  A workgroup (one wavefront) works on 64 points of one (collective,
+ * ranks per node) pair -- `blocks_per_run` chunks make up the pair's n_sizes x n_nodes points,
+ * node count fastest -- because the polygon set depends on that pair alone: the set (at most 8 polygons, 64 vertices, with their bounds) is copied into LDS
  * once and every lane then walks the same polygons out of LDS instead of chasing them through
  * global memory, and workgroups of pairs without regions leave after one table lookup.
  *
