@@ -108,7 +108,8 @@ class GinLoopbackStats(ctypes.Structure):
     _fields_ = [("descriptors", c_u64), ("writes", c_u64), ("copy_entries", c_u64), ("bytes", c_u64),
                 ("signals", c_u64), ("work_items", c_u64), ("acks", c_u64), ("launches", c_u64),
                 ("seconds", ctypes.c_double), ("posts_refused", c_u64), ("post_retries", c_u64),
-                ("tx_completions", c_u64), ("pending_max", c_u32), ("requests_max", c_u32), ("reads", c_u64)]
+                ("tx_completions", c_u64), ("pending_max", c_u32), ("requests_max", c_u32), ("reads", c_u64),
+                ("flush_reads", c_u64)]
 
 
 class GinSignalWork(ctypes.Structure):
@@ -344,6 +345,7 @@ PROTOTYPES = {
     "ofi_amd_gin_tx_iput_signal": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(GinWire),
                                                   ctypes.POINTER(c_i32)]),
     "ofi_amd_gin_tx_iget": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(GinWire), ctypes.POINTER(c_i32)]),
+    "ofi_amd_gin_tx_iflush": (ctypes.c_int, [c_vp, c_vp, c_u64, c_u64, ctypes.POINTER(c_i32)]),
     "ofi_amd_gin_tx_send_ack": (ctypes.c_int, [c_vp, c_u32, c_u64]),
     "ofi_amd_gin_tx_progress": (ctypes.c_int, [c_vp]),
     "ofi_amd_gin_tx_test": (ctypes.c_int, [c_vp, c_i32, ctypes.POINTER(ctypes.c_int)]),

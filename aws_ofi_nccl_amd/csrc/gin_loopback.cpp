@@ -130,7 +130,9 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 	/* completion of a batch is observed the reference's way: a sentinel flush read back into a
 	 * host slot behind the batch's launches (iflush, src/rdma/gin/nccl_ofi_gin.cpp:941-1003) */
 	void *d_flush_buf = nullptr;
+	void *fence_slots = nullptr, *d_fence_slots = nullptr; /* iflush: one 64-byte host slot per rail */
 	rc = ofi_amd_gin_rx_create(nctx, comm_ids.data(), &rx);
+	if (rc == 0) rc = alloc_pinned(&fence_slots, &d_fence_slots, 64 * OFI_AMD_MAX_NUM_RAILS);
 	for (int b = 0; b < 2 && rc == 0; b++) {
 		rc = alloc_batch(batches[b], cap_copy, cap_work);
 	}
@@ -148,6 +150,7 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 		free_batch(batches[0]);
 		free_batch(batches[1]);
 		if (d_flush_buf) (void)ofi_amd_gpu_mem_free(d_flush_buf);
+		if (fence_slots) (void)ofi_amd_gpu_host_free(fence_slots);
 		if (rx) (void)ofi_amd_gin_rx_destroy(rx);
 		if (tx) (void)ofi_amd_gin_tx_destroy(tx);
 		if (fab) (void)ofi_amd_loopfab_destroy(fab);
@@ -282,17 +285,26 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 						}
 					}
 					batch_t &b = batches[cur];
+					/* a flush read lands in host memory: the copy kernel reaches the pinned slots
+					 * through their device address */
+					const uint64_t landing = (read && p.peer == OFI_AMD_GIN_PEER_SELF)
+									 ? p.src - reinterpret_cast<uintptr_t>(fence_slots) +
+										   reinterpret_cast<uintptr_t>(d_fence_slots)
+									 : p.src;
 					for (uint64_t off = 0; off < p.len; off += kPiece) {
 						const uint64_t len = p.len - off < kPiece ? p.len - off : kPiece;
 						b.src[b.n_copy] = (read ? p.dest : p.src) + off;
-						b.dst[b.n_copy] = (read ? p.src : p.dest) + off;
+						b.dst[b.n_copy] = (read ? landing : p.dest) + off;
 						b.len[b.n_copy] = (uint32_t)len;
 						b.n_copy++;
 					}
-					st.bytes += p.len;
-					if (read) {
+					if (read && p.peer == OFI_AMD_GIN_PEER_SELF) {
+						st.flush_reads++;
+					} else if (read) {
+						st.bytes += p.len;
 						st.reads++;
 					} else {
+						st.bytes += p.len;
 						st.writes++;
 						ev.imm = p.imm;
 						in_flight.push_back(ev);
@@ -424,6 +436,37 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 		if (std::chrono::duration_cast<std::chrono::milliseconds>(clock::now() - d0).count() >
 		    (long long)timeout_ms) {
 			rc = -ETIMEDOUT;
+		}
+	}
+	if (rc == 0 && st.reads > 0) {
+		/* the gets are fenced the reference's way (iflush, src/rdma/gin/nccl_ofi_gin.cpp:941-1003):
+		 * a 64-byte read per rail from the device flush buffer into host slots, queued behind
+		 * everything the reads of the gets became, and polled for the sentinel */
+		int32_t fence = -1;
+		rc = ofi_amd_gin_tx_iflush(tx, fence_slots, reinterpret_cast<uintptr_t>(d_flush_buf), kSentinel, &fence);
+		const auto f0 = clock::now();
+		while (rc == 0) {
+			rc = pump();
+			if (rc == 0 && batches[cur].n_copy > 0) {
+				rc = flush(); /* what the fabric has transmitted so far, the fence's reads among it */
+			}
+			int fenced = 0;
+			if (rc == 0) rc = ofi_amd_gin_tx_test(tx, fence, &fenced);
+			if (rc != 0 || fenced) {
+				break;
+			}
+			if (std::chrono::duration_cast<std::chrono::milliseconds>(clock::now() - f0).count() >
+			    (long long)timeout_ms) {
+				rc = -ETIMEDOUT;
+			}
+		}
+		/* the reads' own completions return their requests to the pool */
+		while (rc == 0) {
+			(void)ofi_amd_gin_tx_stats(tx, &ts);
+			if (ts.requests == 0) {
+				break;
+			}
+			rc = pump();
 		}
 	}
 	if (rc == 0) {

@@ -22,7 +22,7 @@ namespace {
 constexpr int32_t kNoParent = -1;
 constexpr uint32_t kMetaSlot = OFI_AMD_MAX_NUM_RAILS; /* reqs_pending[MAX_NUM_RAILS]: the metadata send */
 
-enum : uint8_t { kFree = 0, kOperation = 1, kSub = 2 };
+enum : uint8_t { kFree = 0, kOperation = 1, kSub = 2, kFlush = 3 };
 
 /* One pool entry: the umbrella request of an operation (nccl_ofi_rdma_gin_iputsignal_req) or
  * one post (write / metadata send / ACK send request). */
@@ -31,6 +31,8 @@ struct request_t {
 	uint8_t slot = 0;            /* sub: which reqs_pending flag of the parent it clears */
 	int32_t parent = kNoParent;  /* sub: the operation, or kNoParent (ACKs, given-up operations) */
 	uint32_t pending_mask = 0;   /* operation: bit per outstanding post */
+	const volatile uint64_t *flush_slots = nullptr; /* flush: one 64-byte slot per rail in host memory */
+	uint64_t sentinel = 0;       /* flush: what a slot holds once its read has landed */
 	ofi_amd_gin_post_t post;     /* sub */
 };
 
@@ -304,6 +306,54 @@ int ofi_amd_gin_tx_iget(ofi_amd_gin_tx_t *tx, uint32_t peer, const ofi_amd_gin_w
 	return post_operation(tx, peer, wire, OFI_AMD_GIN_POST_READ, request);
 }
 
+/* nccl_ofi_rdma_gin_put_comm::iflush, src/rdma/gin/nccl_ofi_gin.cpp:941-1003: clear the host
+ * slots, take the umbrella request, post one 64-byte read per rail from the device flush buffer
+ * into the rail's slot.  The reads carry no way back to the umbrella ("No pending_flag --
+ * completion detected via sentinel polling"); their own completions only return them to the pool. */
+int ofi_amd_gin_tx_iflush(ofi_amd_gin_tx_t *tx, void *host_slots, uint64_t device_flush_buffer,
+			  uint64_t sentinel, int32_t *request)
+{
+	if (!tx || !host_slots || !request || (reinterpret_cast<uintptr_t>(host_slots) & 7u) != 0) {
+		return -EINVAL;
+	}
+	*request = -1;
+	if (tx->free_list.size() < 1 + tx->num_rails) {
+		return -ENOMEM;
+	}
+	volatile uint64_t *slots = static_cast<volatile uint64_t *>(host_slots);
+	for (uint32_t rail = 0; rail < tx->num_rails; rail++) {
+		slots[rail * 8] = 0; /* :957-962 */
+	}
+	uint32_t op = 0;
+	(void)tx->alloc(&op);
+	tx->pool[op].use = kFlush;
+	tx->pool[op].flush_slots = slots;
+	tx->pool[op].sentinel = sentinel;
+	for (uint32_t rail = 0; rail < tx->num_rails; rail++) { /* :967-996 */
+		uint32_t idx = 0;
+		(void)tx->alloc(&idx);
+		request_t &r = tx->pool[idx];
+		r.use = kSub;
+		r.parent = kNoParent;
+		r.post = ofi_amd_gin_post_t{OFI_AMD_GIN_POST_READ, rail, 0, idx, OFI_AMD_GIN_PEER_SELF, 0,
+					    reinterpret_cast<uintptr_t>(host_slots) + 64u * rail, 64, device_flush_buffer,
+					    0, {0, 0, 0, 0}};
+		const int rc = tx->post_once(idx);
+		if (rc == -EAGAIN) {
+			tx->queue_pending(idx);
+		} else if (rc != 0) {
+			/* the umbrella goes back (:990-993); the reads already posted complete on their own */
+			tx->release(idx);
+			tx->release(op);
+			return rc;
+		} else {
+			tx->st.posts++;
+		}
+	}
+	*request = (int32_t)op;
+	return 0;
+}
+
 int ofi_amd_gin_tx_send_ack(ofi_amd_gin_tx_t *tx, uint32_t peer, uint64_t ack_msg)
 {
 	if (!tx) {
@@ -348,10 +398,24 @@ int ofi_amd_gin_tx_progress(ofi_amd_gin_tx_t *tx)
 int ofi_amd_gin_tx_test(ofi_amd_gin_tx_t *tx, int32_t request, int *done)
 {
 	if (!tx || !done || request < 0 || (size_t)request >= tx->pool.size() ||
-	    tx->pool[(uint32_t)request].use != kOperation) {
+	    (tx->pool[(uint32_t)request].use != kOperation && tx->pool[(uint32_t)request].use != kFlush)) {
 		return -EINVAL;
 	}
 	*done = 0;
+	if (tx->pool[(uint32_t)request].use == kFlush) {
+		/* nccl_ofi_gin_iflush_req::test, src/rdma/gin/nccl_ofi_gin_reqs.cpp:373-394: the sentinel in
+		 * every rail's slot, not the completion queue, says that the reads have landed */
+		const request_t &f = tx->pool[(uint32_t)request];
+		for (uint32_t rail = 0; rail < tx->num_rails; rail++) {
+			if (__atomic_load_n(const_cast<const uint64_t *>(&f.flush_slots[rail * 8]), __ATOMIC_ACQUIRE) !=
+			    f.sentinel) {
+				return 0;
+			}
+		}
+		*done = 1;
+		tx->release((uint32_t)request);
+		return 0;
+	}
 	if (tx->pool[(uint32_t)request].pending_mask == 0) {
 		*done = 1;
 		tx->release((uint32_t)request);

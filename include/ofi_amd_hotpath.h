@@ -548,12 +548,24 @@ int ofi_amd_gin_tx_iput_signal(ofi_amd_gin_tx_t *tx, uint32_t peer, const ofi_am
  * is done once every read has completed.  Return values as ofi_amd_gin_tx_iput_signal. */
 int ofi_amd_gin_tx_iget(ofi_amd_gin_tx_t *tx, uint32_t peer, const ofi_amd_gin_wire_t *wire,
 			int32_t *request);
+/* iflush (src/rdma/gin/nccl_ofi_gin.cpp:941-1003): fences the reads of earlier gets on every
+ * rail.  host_slots: num_rails slots of 64 bytes in host memory the fabric can write (the
+ * engine clears the first 8 bytes of each); device_flush_buffer: the device buffer that holds
+ * `sentinel` (ofi_amd_flush_buffer_fill).  One read of 64 bytes per rail, peer
+ * OFI_AMD_GIN_PEER_SELF, src = the rail's slot, dest = device_flush_buffer.
+ * ofi_amd_gin_tx_test on the returned request reports done once every slot holds the sentinel
+ * (the reads' own completions only return their requests to the pool).  One flush at a time per
+ * host_slots, as in the reference. */
+#define OFI_AMD_GIN_PEER_SELF 0xffffffffu
+int ofi_amd_gin_tx_iflush(ofi_amd_gin_tx_t *tx, void *host_slots, uint64_t device_flush_buffer,
+			  uint64_t sentinel, int32_t *request);
 /* send_ack: one ACK send on rail 0. */
 int ofi_amd_gin_tx_send_ack(ofi_amd_gin_tx_t *tx, uint32_t peer, uint64_t ack_msg);
 /* nccl_ofi_gin_resources::progress. */
 int ofi_amd_gin_tx_progress(ofi_amd_gin_tx_t *tx);
-/* nccl_ofi_rdma_gin_iputsignal_req::test: *done = 1 (and the request is freed) once every post
- * of the operation has completed.  It does not progress. */
+/* nccl_ofi_rdma_gin_iputsignal_req::test / nccl_ofi_gin_iget_req::test: *done = 1 (and the
+ * request is freed) once every post of the operation has completed; for a flush request, once
+ * every slot holds the sentinel.  It does not progress. */
 int ofi_amd_gin_tx_test(ofi_amd_gin_tx_t *tx, int32_t request, int *done);
 int ofi_amd_gin_tx_stats(const ofi_amd_gin_tx_t *tx, ofi_amd_gin_tx_stats_t *out);
 
@@ -652,7 +664,8 @@ int ofi_amd_gin_signal_apply(const ofi_amd_gin_signal_work_t *d_work, uint32_t n
  *      to a receiver (ofi_amd_gin_rx_*, one peer per context), up to reorder_window events
  *      out of order; each RDMA read of a get as the copy the other way -- from the read's
  *      `dest` (the remote MR's remote_address_offset + offset) into the local buffer -- of
- *      which the receiver hears nothing,
+ *      which the receiver hears nothing; a stream with gets ends with a flush
+ *      (ofi_amd_gin_tx_iflush) whose reads are copies of the sentinel into host slots,
  *   4. sends the receiver's ACKs back through the same engine and fabric; an ACK that arrives
  *      moves the sender's window (ofi_amd_gin_apply_ack),
  * and every batch_writes queued copies (and at the end) launches, in this order on `stream`,
@@ -679,6 +692,7 @@ typedef struct {
 	uint32_t pending_max;     /* longest the pending list got */
 	uint32_t requests_max;    /* most request-pool entries in use */
 	uint64_t reads;           /* RDMA reads of gets */
+	uint64_t flush_reads;     /* reads of the flush that fences them (one per rail), 0 without gets */
 } ofi_amd_gin_loopback_stats_t;
 
 int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *rings, uint64_t ops_per_context,

@@ -36,7 +36,8 @@
  *   gin tx engine    post / retry / completion orders worked out by hand against scripted
  *                    fabrics (full send queues, FI_MORE dropped on retry, head-of-line stop of
  *                    the retry, 16 completions per rail per progress call); a get's reads
- *                    the same way (refused read queued, failed read gives the get up)
+ *                    the same way (refused read queued, failed read gives the get up), and
+ *                    the flush (one read per rail to the own rank, done by the sentinel)
  *   gin signal apply per-slot sums against a plain scatter-add (mod 2^64)
  *   region geometry  ~70 points + 4 extend_region cases of
  *                    tests/unit/region_based_tuner.cpp
@@ -270,6 +271,8 @@ int oracle_gin_tx_iput_signal(oracle_gin_tx_t *tx, uint32_t peer, const oracle_g
 			      int32_t *request);
 int oracle_gin_tx_iget(oracle_gin_tx_t *tx, uint32_t peer, const oracle_gin_wire_t *wire,
 		       int32_t *request);
+int oracle_gin_tx_iflush(oracle_gin_tx_t *tx, void *host_slots, uint64_t device_flush_buffer,
+			 uint64_t sentinel, int32_t *request);
 int oracle_gin_tx_send_ack(oracle_gin_tx_t *tx, uint32_t peer, uint64_t ack_msg);
 int oracle_gin_tx_progress(oracle_gin_tx_t *tx);
 int oracle_gin_tx_test(oracle_gin_tx_t *tx, int32_t request, int *done);

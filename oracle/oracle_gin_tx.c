@@ -22,13 +22,15 @@
 
 #include "oracle.h"
 
-enum { REQ_FREE = 0, REQ_OP = 1, REQ_POST = 2 };
+enum { REQ_FREE = 0, REQ_OP = 1, REQ_POST = 2, REQ_FLUSH = 3 };
 
 typedef struct {
 	int use;
 	int parent;          /* REQ_POST: index of its REQ_OP, or -1 */
 	int flag;            /* REQ_POST: which reqs_pending[] flag of the parent it owns */
 	int reqs_pending[ORACLE_MAX_RAILS + 1]; /* REQ_OP: nccl_ofi_rdma_gin_iputsignal_req */
+	const volatile uint64_t *host_buff;     /* REQ_FLUSH: nccl_ofi_gin_iflush_req */
+	uint64_t sentinel;
 	oracle_gin_post_t post;
 } oreq_t;
 
@@ -255,6 +257,49 @@ int oracle_gin_tx_iget(oracle_gin_tx_t *tx, uint32_t peer, const oracle_gin_wire
 	return 0;
 }
 
+/* nccl_ofi_rdma_gin_put_comm::iflush, src/rdma/gin/nccl_ofi_gin.cpp:941-1003 */
+int oracle_gin_tx_iflush(oracle_gin_tx_t *tx, void *host_slots, uint64_t device_flush_buffer,
+			 uint64_t sentinel, int32_t *request)
+{
+	*request = -1;
+	if (tx->n_free < 1 + tx->num_rails) {
+		return -12;
+	}
+	volatile uint64_t *host = (volatile uint64_t *)host_slots;
+	for (uint32_t rail_id = 0; rail_id < tx->num_rails; rail_id++) { /* :957-962 */
+		host[rail_id * 8] = 0;
+	}
+	int fr = req_alloc(tx); /* :964-965 */
+	tx->reqs[fr].use = REQ_FLUSH;
+	tx->reqs[fr].host_buff = host;
+	tx->reqs[fr].sentinel = sentinel;
+	for (uint32_t rail_id = 0; rail_id < tx->num_rails; rail_id++) { /* :967-996 */
+		int rd = req_alloc(tx);
+		oreq_t *r = &tx->reqs[rd];
+		r->use = REQ_POST;
+		r->parent = -1; /* pending_flag = nullptr */
+		r->post.kind = ORACLE_GIN_POST_READ;
+		r->post.rail = rail_id;
+		r->post.context = (uint32_t)rd;
+		r->post.peer = 0xffffffffu; /* own rank's address: loop-back */
+		r->post.src = (uint64_t)(uintptr_t)host_slots + 64u * rail_id;
+		r->post.len = 64;
+		r->post.dest = device_flush_buffer;
+		int ret = req_post(tx, rd);
+		if (ret == -11) {
+			add_pending_req(tx, rd);
+		} else if (ret != 0) {
+			req_free(tx, rd); /* the reference leaves it out of the pool; see oracle_gin_tx_iget */
+			req_free(tx, fr);
+			return ret;
+		} else {
+			tx->st.posts++;
+		}
+	}
+	*request = fr;
+	return 0;
+}
+
 int oracle_gin_tx_send_ack(oracle_gin_tx_t *tx, uint32_t peer, uint64_t ack_msg)
 {
 	int ar = req_alloc(tx);
@@ -353,8 +398,20 @@ int oracle_gin_tx_progress(oracle_gin_tx_t *tx)
 int oracle_gin_tx_test(oracle_gin_tx_t *tx, int32_t request, int *done)
 {
 	*done = 0;
-	if (request < 0 || (uint32_t)request >= tx->max_requests || tx->reqs[request].use != REQ_OP) {
+	if (request < 0 || (uint32_t)request >= tx->max_requests ||
+	    (tx->reqs[request].use != REQ_OP && tx->reqs[request].use != REQ_FLUSH)) {
 		return -22;
+	}
+	if (tx->reqs[request].use == REQ_FLUSH) {
+		/* nccl_ofi_gin_iflush_req::test, src/rdma/gin/nccl_ofi_gin_reqs.cpp:373-394 */
+		for (uint32_t rail_id = 0; rail_id < tx->num_rails; rail_id++) {
+			if (tx->reqs[request].host_buff[rail_id * 8] != tx->reqs[request].sentinel) {
+				return 0;
+			}
+		}
+		*done = 1;
+		req_free(tx, request);
+		return 0;
 	}
 	for (int i = 0; i <= ORACLE_MAX_RAILS; i++) {
 		if (tx->reqs[request].reqs_pending[i]) {

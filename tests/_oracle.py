@@ -154,6 +154,7 @@ _ORACLE_PROTOS = {
     "oracle_gin_tx_iput_signal": (c_int, [ctypes.c_void_p, c_u32, ctypes.POINTER(GinWire),
                                           ctypes.POINTER(c_i32)]),
     "oracle_gin_tx_iget": (c_int, [ctypes.c_void_p, c_u32, ctypes.POINTER(GinWire), ctypes.POINTER(c_i32)]),
+    "oracle_gin_tx_iflush": (c_int, [ctypes.c_void_p, ctypes.c_void_p, c_u64, c_u64, ctypes.POINTER(c_i32)]),
     "oracle_gin_tx_send_ack": (c_int, [ctypes.c_void_p, c_u32, c_u64]),
     "oracle_gin_tx_progress": (c_int, [ctypes.c_void_p]),
     "oracle_gin_tx_test": (c_int, [ctypes.c_void_p, c_i32, ctypes.POINTER(c_int)]),

@@ -633,6 +633,32 @@ void run_gin_engine(uint64_t seed, uint32_t n_ops)
 			if (ra == 0) {
 				open.push_back(qa);
 			}
+		} else if (what < 58) { /* a flush: one read per rail into slots that a later step fills */
+			static uint64_t slots_a[32]; /* one array for both engines: the posts carry its address */
+			uint64_t *const slots_b = slots_a;
+			int32_t qa = -2, qb = -2;
+			const int ra = oracle_gin_tx_iflush(a, slots_a, 0x5000, 0xdeadbeefdeadbeefull, &qa);
+			SAME("iflush rc", ra, ofi_amd_gin_tx_iflush(b, slots_b, 0x5000, 0xdeadbeefdeadbeefull, &qb));
+			SAME("iflush request", qa, qb);
+			if (ra == 0) {
+				SAME("slots cleared", slots_a[0] | slots_a[8] | slots_a[16] | slots_a[24], 0);
+				/* the reads land at once or not at all before the request is tested */
+				const bool landed = rng.chance(70);
+				for (int r = 0; r < 4; r++) {
+					slots_a[8 * r] = slots_b[8 * r] = landed ? 0xdeadbeefdeadbeefull : 0;
+				}
+				int da = -1, db = -1;
+				SAME("flush test rc", oracle_gin_tx_test(a, qa, &da), ofi_amd_gin_tx_test(b, qb, &db));
+				SAME("flush done", da, db);
+				if (!da) {
+					for (int r = 0; r < 4; r++) {
+						slots_a[8 * r] = slots_b[8 * r] = 0xdeadbeefdeadbeefull;
+					}
+					SAME("flush test rc", oracle_gin_tx_test(a, qa, &da), ofi_amd_gin_tx_test(b, qb, &db));
+					SAME("flush done late", da, 1);
+					SAME("flush done late", db, 1);
+				}
+			}
 		} else if (what < 65) {
 			const uint64_t msg = rng.next();
 			const uint32_t peer = rng.below(8);

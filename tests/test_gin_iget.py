@@ -307,3 +307,87 @@ def test_reads_through_the_in_process_fabric(lib):
     assert lib.ofi_amd_gin_tx_test(tx, req, ctypes.byref(done)) == 0 and done.value == 1
     lib.ofi_amd_gin_tx_destroy(tx)
     lib.ofi_amd_loopfab_destroy(fab)
+
+
+# ---- iflush: the fence behind gets ----
+
+SENTINEL = 0xDEADBEEFDEADBEEF
+SELF = 0xFFFFFFFF
+
+
+def test_flush_posts_one_read_per_rail_and_is_done_by_the_sentinel(which, oracle, lib):
+    """iflush (src/rdma/gin/nccl_ofi_gin.cpp:941-1003) with send queues of one entry, rail 1 occupied
+    by a put's write (entries 0, 1).  The flush is entry 2; its reads are entries 3 (rail 0,
+    posted), 4 (rail 1, refused and queued), 5, 6 (rails 2, 3, posted).  The engine has cleared
+    the four slots.  The reads' completions free their entries but say nothing to the flush:
+    test() is done only when every slot holds the sentinel, whatever the completion queue said."""
+    e = Engine(which, oracle, lib, (1,))
+    f = e.fabric
+    slots = (ctypes.c_uint64 * 32)(*([0x1111] * 32))
+    base = ctypes.addressof(slots)
+    assert e.op([(1, 0)]) == (0, 0)
+    f.take_log()
+    req = ctypes.c_int32(-7)
+    assert e.fn("iflush")(e.tx, slots, 0xABC000, SENTINEL, ctypes.byref(req)) == 0 and req.value == 2
+    assert f.take_log() == [("post", R, 0, 0, 3), ("refused", R, 1, 0, 4), ("post", R, 2, 0, 5), ("post", R, 3, 0, 6)]
+    assert [slots[8 * r] for r in range(4)] == [0, 0, 0, 0] and slots[1] == 0x1111
+    assert e.stats()["requests"] == 7 and e.stats()["pending"] == 1
+    assert e.test(2) == (0, 0)
+    # every read that was posted completes; the flush is still not done: no sentinel yet
+    for rail in (0, 1, 2, 3):
+        f.complete(rail)
+    assert e.progress() == 0
+    assert [x for x in f.take_log() if x[0] != "cq_read"] == [("post", R, 1, 0, 4)]
+    assert e.test(2) == (0, 0)
+    assert e.stats()["requests"] == 3                                # the put, the flush and the retried read
+    for rail in (0, 2, 3, 1):
+        slots[8 * rail] = SENTINEL
+        assert e.test(2) == (0, 1 if rail == 1 else 0)
+    assert e.test(2)[0] == EINVAL                                   # freed by the test that saw it done
+    f.complete(1)
+    assert e.progress() == 0 and e.test(0) == (0, 1) and e.stats()["requests"] == 0
+    e.close()
+
+
+def test_flush_read_arguments_and_failure(which, oracle, lib):
+    """The reads go to the own rank (loop-back), 64 bytes from the device flush buffer into the
+    rail's slot.  A read that fails for good returns the flush request to the pool (:990-993)."""
+    seen = []
+    e = Engine(which, oracle, lib, (4, (2, EIO)), rails=3)
+    real_post = e.fabric.post
+
+    def post(fabric, p):
+        c = p.contents
+        seen.append((c.kind, c.rail, c.peer, c.src, c.len, c.dest, c.imm))
+        return real_post(fabric, p)
+    e.fabric._post = e.mod.FABRIC_POST_FN(post)
+    e.fabric.ops.post = e.fabric._post
+    # the engine copied the callbacks at create: make a new engine on the spying fabric
+    e2 = Engine.__new__(Engine)
+    e2.__dict__.update(e.__dict__)
+    if e.product:
+        e2.tx = ctypes.c_void_p()
+        assert lib.ofi_amd_gin_tx_create(3, 4, 4, 64, ctypes.byref(e.fabric.ops), ctypes.byref(e2.tx)) == 0
+    else:
+        e2.tx = ctypes.c_void_p(oracle.oracle_gin_tx_create(3, 4, 4, 64, ctypes.byref(e.fabric.ops)))
+    slots = (ctypes.c_uint64 * 24)()
+    base = ctypes.addressof(slots)
+    req = ctypes.c_int32(-7)
+    assert e2.fn("iflush")(e2.tx, slots, 0xABC000, SENTINEL, ctypes.byref(req)) == EIO and req.value == -1
+    assert seen == [(R, 0, SELF, base, 64, 0xABC000, 0), (R, 1, SELF, base + 64, 64, 0xABC000, 0)]
+    assert e2.stats()["requests"] == 1                              # the read on rail 0 is still out
+    e2.close()
+    e.close()
+
+
+def test_product_flush_argument_checks(lib, oracle):
+    e = Engine("product", oracle, lib, (4,), max_requests=4)
+    slots = (ctypes.c_uint64 * 32)()
+    req = ctypes.c_int32()
+    assert lib.ofi_amd_gin_tx_iflush(None, slots, 1, SENTINEL, ctypes.byref(req)) == EINVAL
+    assert lib.ofi_amd_gin_tx_iflush(e.tx, None, 1, SENTINEL, ctypes.byref(req)) == EINVAL
+    assert lib.ofi_amd_gin_tx_iflush(e.tx, ctypes.c_void_p(ctypes.addressof(slots) + 4), 1, SENTINEL,
+                                     ctypes.byref(req)) == EINVAL
+    assert lib.ofi_amd_gin_tx_iflush(e.tx, slots, 1, SENTINEL, ctypes.byref(req)) == -12   # 1 + 4 entries, 4 there
+    assert e.fabric.take_log() == []
+    e.close()

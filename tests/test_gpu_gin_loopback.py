@@ -206,11 +206,11 @@ def test_gets_land_bit_exact_beside_puts(lib, gpu):
     assert [int(x) for x in _gpu.to_host(d_cnt, np.uint64)] == counters
 
     assert stats.descriptors == nctx * ops and stats.signals == n_signals
-    assert stats.reads == want_reads
+    assert stats.reads == want_reads and stats.flush_reads == 4     # the fence behind the gets: one read per rail
     assert stats.bytes == sum(r[2] for r in replay if r) + sum(g[2] for g in gets)
     for c in range(nctx):
         assert comms[c].tx_head == n_puts // nctx                 # the puts only
-    assert stats.tx_completions == stats.writes + stats.signals + stats.acks + stats.reads
+    assert stats.tx_completions == stats.writes + stats.signals + stats.acks + stats.reads + stats.flush_reads
     assert stats.posts_refused > 0
     assert _gpu.fetch_async_errors(lib) == 0
     lib.ofi_amd_gin_rings_destroy(rings)
