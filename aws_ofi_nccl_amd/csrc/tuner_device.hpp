@@ -140,13 +140,70 @@ __device__ inline float model_cost(int platform, int coll, int algo, int proto, 
 	return __fadd_rn(__fmul_rn(latency, (float)pipe_ops), __fdiv_rn((float)size, bw));
 }
 
+/* The three protocols of one algorithm at once: cell for cell the operations of model_cost above,
+ * in the same order, with what the three cells share worked out once (the step counts and their
+ * conversions, the base bandwidth, the rank quotient and the log term).  size_f = (float)size,
+ * ranks_over_nodes = num_ranks / num_nodes (a grid knows it without dividing). */
+__device__ inline void model_cost_protos(int platform, int coll, int algo, int pipe_ops, float size_f,
+					 uint64_t num_ranks, uint64_t num_nodes, uint64_t ranks_over_nodes,
+					 double log2_nodes, int num_channels, int net_comp_overhead,
+					 float out[NUM_PROTOS])
+{
+	out[PROTO_LL] = out[PROTO_LL128] = out[PROTO_SIMPLE] = -1.0f;
+	if (coll != FUNC_ALLREDUCE || (algo != ALGO_RING && algo != ALGO_TREE && algo != ALGO_NVLS_TREE)) {
+		return;
+	}
+	const model_params_t params = model_params(platform);
+	const float net_lat_of[NUM_PROTOS] = { params.net_lat, params.net_lat,
+					       __fadd_rn(params.net_lat, (float)net_comp_overhead) };
+	const float rails_bw = __fmul_rn(params.internode_bw, (float)params.num_rails);
+	float latency[NUM_PROTOS], bw;
+	if (algo == ALGO_RING) {
+		const int num_steps = (int)(2 * (num_ranks - 1));
+		const int num_internode_steps = (int)(2 * num_nodes);
+		const float inter = (float)num_internode_steps, rest = (float)(num_steps - num_internode_steps);
+#pragma unroll
+		for (int proto = 0; proto < NUM_PROTOS; proto++) {
+			latency[proto] = __fadd_rn(__fmul_rn(inter, net_lat_of[proto]),
+						   __fmul_rn(rest, nvlink_lat(ALGO_RING, proto)));
+		}
+		bw = __fmul_rn(rails_bw, (float)num_channels);
+	} else if (algo == ALGO_NVLS_TREE) {
+#pragma unroll
+		for (int proto = 0; proto < NUM_PROTOS; proto++) {
+			const double t = __dadd_rn((double)nvlink_lat(ALGO_NVLS_TREE, proto),
+						   __dmul_rn(log2_nodes, (double)net_lat_of[proto]));
+			latency[proto] = (float)__dmul_rn(2.0, t);
+		}
+		const float half = __fdiv_rn(rails_bw, 2.0f);
+		bw = __fmul_rn(half < params.intranode_bw ? half : params.intranode_bw, (float)num_channels);
+	} else {
+		const float hops = (float)(2 * (ranks_over_nodes - 1));
+		const double log_term = __dmul_rn(2.0, log2_nodes);
+#pragma unroll
+		for (int proto = 0; proto < NUM_PROTOS; proto++) {
+			const float a = __fmul_rn(hops, nvlink_lat(ALGO_TREE, proto));
+			const double b = __dmul_rn(log_term, (double)net_lat_of[proto]);
+			latency[proto] = (float)__dadd_rn((double)a, b);
+		}
+		bw = __fdiv_rn(__fmul_rn(rails_bw, (float)num_channels), 2.0f);
+	}
+	const float bw_of[NUM_PROTOS] = { (float)__dmul_rn((double)bw, 0.5), (float)__dmul_rn((double)bw, 0.9375), bw };
+	const float pipe = (float)pipe_ops;
+#pragma unroll
+	for (int proto = 0; proto < NUM_PROTOS; proto++) {
+		out[proto] = __fadd_rn(__fmul_rn(latency[proto], pipe), __fdiv_rn(size_f, bw_of[proto]));
+	}
+}
+
 /* model_get_coll_info_internal_v3 (:154-234); with the NVLS-tree bit of `mask`
  * clear it is _v2 with nvlsSupport == 0 (:236-309).  The model never looks at
- * NCCL's cost table, so no other bit of the mask matters here. */
-__device__ inline void model_choose(int platform, int coll, uint64_t size, uint64_t ranks,
-				    uint64_t nodes, double log2_nodes, int pipe_ops, int num_channels,
-				    int net_comp_overhead, uint32_t mask, int &chosen_algo,
-				    int &chosen_proto)
+ * NCCL's cost table, so no other bit of the mask matters here.  cost_of(algo, proto) is the
+ * cell's cost, negative when not modelled. */
+template <typename F>
+__device__ __forceinline__ void model_choose_with(int platform, int coll, uint64_t size, uint64_t ranks,
+						  uint64_t nodes, uint32_t mask, F cost_of, int &chosen_algo,
+						  int &chosen_proto)
 {
 	chosen_algo = -1;
 	chosen_proto = -1;
@@ -173,8 +230,7 @@ __device__ inline void model_choose(int platform, int coll, uint64_t size, uint6
 			if (algo == ALGO_NVLS_TREE && proto != PROTO_SIMPLE) {
 				continue;
 			}
-			float c = model_cost(platform, coll, algo, proto, pipe_ops, size, ranks, nodes,
-					     log2_nodes, num_channels, net_comp_overhead);
+			float c = cost_of(algo, proto);
 			if (c < 0) {
 				continue;
 			}
@@ -185,6 +241,20 @@ __device__ inline void model_choose(int platform, int coll, uint64_t size, uint6
 			}
 		}
 	}
+}
+
+__device__ inline void model_choose(int platform, int coll, uint64_t size, uint64_t ranks,
+				    uint64_t nodes, double log2_nodes, int pipe_ops, int num_channels,
+				    int net_comp_overhead, uint32_t mask, int &chosen_algo,
+				    int &chosen_proto)
+{
+	model_choose_with(
+		platform, coll, size, ranks, nodes, mask,
+		[&](int algo, int proto) -> float {
+			return model_cost(platform, coll, algo, proto, pipe_ops, size, ranks, nodes, log2_nodes,
+					  num_channels, net_comp_overhead);
+		},
+		chosen_algo, chosen_proto);
 }
 
 /* ------------------------------------------------------------------ regions */

@@ -47,11 +47,22 @@ __global__ __launch_bounds__(256) void model_grid_kernel(grid_dims_t g,
 							 int8_t *__restrict__ choice)
 {
 	extern __shared__ double stage[]; /* [256][cells per point] when COST */
+	__shared__ int32_t column_of[NUM_ALGOS]; /* the plan's column of an algorithm, -1: none */
 	const uint32_t cpp = g.n_algos * NUM_PROTOS;
 	const uint32_t first = blockIdx.x * 256u;
 	const uint32_t p = first + threadIdx.x;
 	const ofi_amd_tuner_variant_t v = variants[blockIdx.y];
 	const bool live = p < points_per_variant;
+	if (COST && CHOICE) {
+		if (threadIdx.x < NUM_ALGOS) {
+			int32_t col = -1;
+			for (uint32_t ai = g.n_algos; ai-- > 0;) {
+				col = g.algos[ai] == (int32_t)threadIdx.x ? (int32_t)ai : col;
+			}
+			column_of[threadIdx.x] = col;
+		}
+		__syncthreads();
+	}
 	if (live) {
 		uint32_t r = p;
 		const uint32_t pi = r % g.n_ppn; r /= g.n_ppn;
@@ -59,36 +70,78 @@ __global__ __launch_bounds__(256) void model_grid_kernel(grid_dims_t g,
 		const uint32_t si = r % g.n_sizes; r /= g.n_sizes;
 		const uint32_t ci = r;
 		const uint64_t nodes = g.nodes[ni];
-		const uint64_t ranks = nodes * g.ppn[pi];
+		const uint64_t per_node = g.ppn[pi];
+		const uint64_t ranks = nodes * per_node;
 		if (COST) {
 			const bool modelled = platform_has_model(v.platform);
+			const float size_f = (float)g.sizes[si];
+			const int coll = g.colls[ci];
+			const double log2_nodes = g.log2_nodes[ni];
 			for (uint32_t ai = 0; ai < g.n_algos; ai++) {
+				float c[NUM_PROTOS] = { -1.0f, -1.0f, -1.0f };
+				if (modelled) {
+					/* ranks = nodes * per_node, so ranks / nodes is per_node */
+					model_cost_protos(v.platform, coll, g.algos[ai], v.pipe_ops, size_f, ranks, nodes, per_node,
+							  log2_nodes, v.num_channels, v.net_comp_overhead, c);
+				}
+#pragma unroll
 				for (uint32_t proto = 0; proto < NUM_PROTOS; proto++) {
-					float c = -1.0f;
-					if (modelled) {
-						c = model_cost(v.platform, g.colls[ci], g.algos[ai], (int)proto, v.pipe_ops,
-							       g.sizes[si], ranks, nodes, g.log2_nodes[ni],
-							       v.num_channels, v.net_comp_overhead);
-					}
-					stage[threadIdx.x * cpp + ai * NUM_PROTOS + proto] = (double)c;
+					stage[threadIdx.x * cpp + ai * NUM_PROTOS + proto] = (double)c[proto];
 				}
 			}
 		}
 		if (CHOICE) {
 			int algo, proto;
-			model_choose(v.platform, g.colls[ci], g.sizes[si], ranks, nodes, g.log2_nodes[ni], v.pipe_ops,
-				     v.num_channels, v.net_comp_overhead, kAllAllowed, algo, proto);
+			if (COST) {
+				/* the cells the decision looks at have just been worked out: it reads this thread's
+				 * row of the stage instead of evaluating the model again, and goes to the model
+				 * only for an algorithm the plan has no column for */
+				const double *cells = &stage[threadIdx.x * cpp];
+				model_choose_with(
+					v.platform, g.colls[ci], g.sizes[si], ranks, nodes, kAllAllowed,
+					[&](int a, int pr) -> float {
+						const int32_t col = column_of[a];
+						if (col >= 0) {
+							return (float)cells[col * NUM_PROTOS + pr]; /* exact: it was a float */
+						}
+						return model_cost(v.platform, g.colls[ci], a, pr, v.pipe_ops, g.sizes[si], ranks,
+								  nodes, g.log2_nodes[ni], v.num_channels, v.net_comp_overhead);
+					},
+					algo, proto);
+			} else {
+				model_choose(v.platform, g.colls[ci], g.sizes[si], ranks, nodes, g.log2_nodes[ni], v.pipe_ops,
+					     v.num_channels, v.net_comp_overhead, kAllAllowed, algo, proto);
+			}
 			const uint64_t at = ((uint64_t)blockIdx.y * points_per_variant + p) * 2u;
-			choice[at + 0] = (int8_t)algo;
-			choice[at + 1] = (int8_t)proto;
+			if ((reinterpret_cast<uintptr_t>(choice) & 1u) == 0) {
+				*reinterpret_cast<uint16_t *>(choice + at) =
+					(uint16_t)((uint8_t)(int8_t)algo | ((uint32_t)(uint8_t)(int8_t)proto << 8));
+			} else {
+				choice[at + 0] = (int8_t)algo;
+				choice[at + 1] = (int8_t)proto;
+			}
 		}
 	}
 	if (COST) {
 		__syncthreads();
 		const uint32_t valid = min(256u, points_per_variant - first);
 		double *out = cost + ((uint64_t)blockIdx.y * points_per_variant + first) * cpp;
-		for (uint32_t k = threadIdx.x; k < valid * cpp; k += 256u) {
-			__builtin_nontemporal_store(stage[k], &out[k]);
+		const uint32_t cells = valid * cpp;
+		if ((reinterpret_cast<uintptr_t>(out) & 15u) == 0) {
+			/* two cells per lane and store: 1 KiB per wavefront instruction */
+			typedef double double2_t __attribute__((ext_vector_type(2)));
+			const double2_t *from = reinterpret_cast<const double2_t *>(stage);
+			double2_t *to = reinterpret_cast<double2_t *>(out);
+			for (uint32_t k = threadIdx.x; k < cells / 2; k += 256u) {
+				__builtin_nontemporal_store(from[k], &to[k]);
+			}
+			if ((cells & 1u) && threadIdx.x == 0) {
+				out[cells - 1] = stage[cells - 1];
+			}
+		} else {
+			for (uint32_t k = threadIdx.x; k < cells; k += 256u) {
+				__builtin_nontemporal_store(stage[k], &out[k]);
+			}
 		}
 	}
 }
