@@ -9,6 +9,7 @@
 #include <vector>
 #include <cstring>
 
+#include "gin_derive.hpp"
 #include "gin_rings.hpp"
 
 namespace {
@@ -126,6 +127,8 @@ static int drain_contexts(ofi_amd_gin_rings_t *r, uint32_t c_begin, uint32_t c_e
 			uint64_t want = ops_per_context - done[k];
 			uint32_t limit = want < burst ? (uint32_t)want : burst;
 			uint64_t h = hash[k];
+			/* constant over the burst: the derivation keeps the counters below the rail count */
+			const bool fast = mode >= 2 && ofi_amd_gin::derive_fast_path(&comms[c]);
 
 			while (pos - start < limit &&
 			       __atomic_load_n(&seq[pos & mask], __ATOMIC_ACQUIRE) == pos + 1) {
@@ -141,9 +144,16 @@ static int drain_contexts(ofi_amd_gin_rings_t *r, uint32_t c_begin, uint32_t c_e
 					ofi_amd_gin_wire_t local;
 					ofi_amd_gin_wire_t *wire =
 						out_wire ? &out_wire[(size_t)c * ops_per_context + i] : &local;
-					int e = d->kind == OFI_AMD_GIN_KIND_GET
-							? ofi_amd_gin_iget(&comms[c], mrs, n_mrs, d, wire)
-							: ofi_amd_gin_iput_signal(&comms[c], mrs, n_mrs, d, wire);
+					/* the derivation is inlined here (gin_derive.hpp): the communicator's state
+					 * stays in registers from one descriptor of the burst to the next */
+					int e;
+					if (d->kind == OFI_AMD_GIN_KIND_GET) {
+						e = ofi_amd_gin_iget(&comms[c], mrs, n_mrs, d, wire);
+					} else if (fast) {
+						e = ofi_amd_gin::derive<true>(&comms[c], mrs, n_mrs, d, wire);
+					} else {
+						e = ofi_amd_gin_iput_signal(&comms[c], mrs, n_mrs, d, wire);
+					}
 					if (e != 0) {
 						rc = e;
 						break;
