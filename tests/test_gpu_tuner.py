@@ -211,6 +211,26 @@ def test_region_grid_shapes_around_the_workgroup_size(lib, oracle, gpu, n_sizes,
         lib.ofi_amd_tuner_plan_destroy(plan)
 
 
+def test_region_grid_on_changing_platform_lists(lib, oracle, gpu):
+    """One plan, platform lists that grow, shrink and change in place: the launch order the plan keeps
+    for a list (which entry, chunk and ranks-per-node value each workgroup takes) is rebuilt whenever
+    the list differs from the last call's, never reused for another list."""
+    colls = np.array([4, 2, 3], dtype=np.int32)
+    sizes = np.array(sorted({int(2 ** (k / 2)) for k in range(10, 70)}), dtype=np.uint64)
+    nodes = np.array([1, 2, 3, 4, 8, 16, 32, 64, 100], dtype=np.uint64)
+    ppn = np.array([1, 2, 4, 8], dtype=np.uint32)
+    plan = make_plan(lib, colls, sizes, nodes, ppn, np.array([1], dtype=np.int32))
+    cache = {}
+    for platforms in ([0, 1, 2, 3], [3], [1, 1, 0], [0, 1, 1], [2, 3, 0, 1, 0, 3, 2], [3], [0, 1, 2, 3]):
+        key = tuple(platforms)
+        if key not in cache:
+            cache[key] = oracle_region_grid(oracle, platforms, colls, sizes, nodes, ppn)
+        got = run_region(lib, plan, platforms, (len(platforms), 3, len(sizes), len(nodes), 4))
+        mism = np.argwhere((got != cache[key]).any(axis=-1))
+        assert len(mism) == 0, (platforms, mism[:10])
+    lib.ofi_amd_tuner_plan_destroy(plan)
+
+
 def test_bad_arguments(lib, gpu):
     colls, sizes, nodes, ppn, algos = synthetic.tuner_axes()
     plan = ctypes.c_void_p()
