@@ -18,8 +18,11 @@ nothing else of interest, which keeps counter runs short.  The shapes:
   striping  1m | 16m     1,000,000 / 16,000,000 message sizes, 4 rails
   model     64 | 256     tuner cost-model grids per launch
   region    64           tuner region grids per launch
-  eager     configured   65,536 rx buffers of 8,320 B, payloads 0..8,184 B, destinations at any
-                         byte alignment
+  eager     configured   65,536 rx buffers of 8,320 B, payloads 0..8,184 B, taken in a random
+                         order of slots, destinations at any byte alignment
+            slots        the same with the rx buffers taken in slot order
+            align<N>     the same as configured with every destination a multiple of N bytes
+                         (N = 16, 64 or 128); "slots+align<N>" combines the two
 """
 import argparse
 import ctypes
@@ -105,6 +108,13 @@ def main():
         rx_off = rng.permutation(n).astype(np.uint64) * np.uint64(stride)
         dst_off = (np.sort(rng.permutation((2 << 30) // 8448)[:n]).astype(np.uint64) * np.uint64(8448) +
                    rng.integers(0, 64, n).astype(np.uint64))
+        for word in (args.shape or "configured").split("+"):
+            if word == "slots":
+                rx_off = np.arange(n, dtype=np.uint64) * np.uint64(stride)
+            elif word in ("align16", "align64", "align128"):
+                dst_off &= ~np.uint64(int(word[5:]) - 1)
+            elif word != "configured":
+                ap.error("unknown shape")
         d_rx = torch.randint(0, 255, (n * stride,), dtype=torch.uint8, device="cuda")
         d_dst = torch.zeros(2 << 30, dtype=torch.uint8, device="cuda")
         d = [dev(x) for x in (rx_off, recv_len, dst_off, recv_len)]
