@@ -35,8 +35,10 @@
  * lanes may be clamped, loads it (94.4 -> 91.8 us on the configured batch: the
  * texture-address unit is busy 74 % of the kernel's time).  That dword always
  * contains at least one byte of the buffer, so nothing beyond the dword that
- * holds the last source byte is read.  The sub-16-byte tail goes out as single
- * bytes so that nothing outside [dst, dst+len) is written.
+ * holds the last source byte is read.  The rows cover whole 64-byte units of the
+ * destination; what is left of the buffer (up to 63 bytes) goes out as single
+ * bytes, one per lane, so that nothing outside [dst, dst+len) is written and the
+ * last, partial unit is written by one instruction.
  *
  * Flush: the wave waits until its own stores have left the CU (they are
  * write-through to the L2 of its XCD), then lane 0 re-reads the first 4 bytes
@@ -58,6 +60,9 @@
 #endif
 #ifndef OFI_BOUNCE_NEIGHBOUR
 #define OFI_BOUNCE_NEIGHBOUR 1 /* shifted path: the dword after a lane's 16 bytes comes from the next lane */
+#endif
+#ifndef OFI_BOUNCE_TAIL64
+#define OFI_BOUNCE_TAIL64 1 /* the byte-wise tail takes the whole last 64-byte unit */
 #endif
 #ifndef OFI_BOUNCE_GROUP
 #define OFI_BOUNCE_GROUP 32 /* consecutive workgroups that share an XCD */
@@ -205,9 +210,12 @@ __global__ __launch_bounds__(kBlock) void bounce_scatter_kernel(
 	uint8_t *d = arena + doff;
 
 	if (bytes != 0) {
-		const uint32_t nvec = bytes >> 4;
-		/* tail bytes first, so their latency overlaps the body; unpredicated (lanes
-		 * without a tail byte re-copy the buffer's last byte) to stay branch-free */
+		/* whole 64-byte units as 16-byte words, the rest (up to 63 bytes) singly, one per
+		 * lane: the last, partial unit of memory is then written by one instruction rather
+		 * than by the end of a row and by the tail.  Tail bytes first, so their latency
+		 * overlaps the body; unpredicated (lanes without a tail byte re-copy the buffer's
+		 * last byte) to stay branch-free */
+		const uint32_t nvec = OFI_BOUNCE_TAIL64 ? (bytes >> 6) << 2 : bytes >> 4;
 		const uint32_t tail_at = min((nvec << 4) + lane, bytes - 1u);
 		const uint8_t tail_byte = s[tail_at];
 
@@ -252,7 +260,7 @@ __device__ __forceinline__ void copy_any(const uint8_t *__restrict__ s, uint8_t 
 	if (rem != 0) {
 		const uint8_t *s2 = s + head;
 		uint8_t *d2 = d + head;
-		const uint32_t nvec = rem >> 4;
+		const uint32_t nvec = OFI_BOUNCE_TAIL64 ? (rem >> 6) << 2 : rem >> 4; /* as in the bounce copy */
 		const uint32_t tail_at = min((nvec << 4) + lane, rem - 1u);
 		const uint8_t tail_byte = s2[tail_at];
 		const uint32_t shift = (uint32_t)(reinterpret_cast<uintptr_t>(s2) & 3u);
