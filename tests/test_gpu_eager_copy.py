@@ -80,13 +80,15 @@ def test_random_alignment_and_truncation(lib, oracle, gpu, n, seed):
 
 
 def test_every_short_length_at_every_alignment(lib, oracle, gpu):
-    """lengths 0..80 x destination alignment 0..15 x source alignment (rx_off + 8) fixed by
-    the format: the head / body / tail split is exercised at each boundary"""
+    """lengths 0..200 x destination alignment 0..63 x source alignment (rx_off + 8) fixed by
+    the format: the head (up to the destination's first 64-byte boundary) / body (whole 64-byte
+    units) / tail (up to 63 bytes) split is exercised at each boundary, three bytes apart so
+    that a byte written outside a buffer lands in its neighbour or in the fill"""
     lens, offs = [], []
     pos = 0
-    for length in range(0, 81):
-        for align in range(16):
-            start = (pos + 15) // 16 * 16 + align
+    for length in range(0, 201):
+        for align in range(64):
+            start = (pos + 63) // 64 * 64 + align
             offs.append(start)
             lens.append(length)
             pos = start + length + 3
