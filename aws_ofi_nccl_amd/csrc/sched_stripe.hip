@@ -150,6 +150,23 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, uint32_t)
 	return v;
 }
 
+/* Which tile a workgroup takes.  Workgroups are dealt to the 8 XCDs in turn; with tile =
+ * workgroup number every XCD writes one tile's rows (96 KiB) out of every eight, with runs of
+ * 16 consecutive tiles per XCD each of them writes 1.5 MiB at a stretch.  Once the output no
+ * longer fits the last-level cache the longer stretches are faster (5,000,000 messages: 110.6 ->
+ * 102.9 us, 16,000,000: 324.6 -> 305.9 us; runs of 4, 64, 256 or an eighth of the batch per XCD:
+ * 307-312 us), below that they are slower (1,000,000: 22.4 -> 24.1 us, 4,200,000: 91.3 -> 97.0
+ * us), so they are used from 4.5 Mi messages on.  The grid is rounded up to whole rounds; a
+ * workgroup whose tile does not exist leaves at once. */
+constexpr uint32_t kXcdRunShift = 4;
+constexpr uint64_t kXcdRunBatch = 9ull << 19;
+__device__ __forceinline__ uint32_t tile_of_workgroup(uint32_t wg, uint32_t run_shift)
+{
+	/* XCDs take runs of 2^run_shift consecutive tiles in turn */
+	const uint32_t x = wg & 7u, t = wg >> 3;
+	return ((((t >> run_shift) << 3) + x) << run_shift) + (t & ((1u << run_shift) - 1u));
+}
+
 template <uint32_t PASSES>
 __global__ __launch_bounds__(kThreads) void stripe_count_kernel(
 	const uint64_t *__restrict__ sizes, uint32_t n, const ofi_amd_sched_state_t *__restrict__ state,
@@ -295,13 +312,17 @@ template <bool INLINE, uint32_t PASSES>
 __global__ __launch_bounds__(kThreads) void stripe_emit_kernel(
 	const uint64_t *__restrict__ sizes, uint32_t n, ofi_amd_sched_state_t *__restrict__ state,
 	uint64_t align, const uint32_t *__restrict__ tile_prefix, const uint32_t *__restrict__ seed0,
-	uint32_t *__restrict__ num_xfers, u32x4 *__restrict__ xfers)
+	uint32_t num_tiles, uint32_t xcd_run_shift, uint32_t *__restrict__ num_xfers, u32x4 *__restrict__ xfers)
 {
 	/* 256 rows of 96 bytes = 6 x 16 B each */
 	__shared__ u32x4 rows[kThreads * 6];
 	__shared__ uint32_t wave_sum[kThreads / 64];
 	const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-	const uint32_t base = blockIdx.x * (kThreads * PASSES);
+	const uint32_t tile = tile_of_workgroup(blockIdx.x, xcd_run_shift);
+	if (tile >= num_tiles) {
+		return;
+	}
+	const uint32_t base = tile * (kThreads * PASSES);
 	/* every pass's size is requested up front: the passes below then run out of registers
 	 * instead of each waiting for its own load */
 	uint64_t size_of[PASSES];
@@ -320,7 +341,7 @@ __global__ __launch_bounds__(kThreads) void stripe_emit_kernel(
 	if (INLINE) {
 		/* sum of the totals of the tiles before this one (packed halves, no overflow) */
 		uint32_t acc = 0;
-		for (uint32_t t = threadIdx.x; t < blockIdx.x; t += kThreads) {
+		for (uint32_t t = threadIdx.x; t < tile; t += kThreads) {
 			acc += tile_prefix[t];
 		}
 #pragma unroll
@@ -335,7 +356,7 @@ __global__ __launch_bounds__(kThreads) void stripe_emit_kernel(
 		__syncthreads();
 		seed = (((acc >> 16) % R) << 16) | ((acc & 0xffffu) % R);
 	} else {
-		seed = tile_prefix[blockIdx.x];
+		seed = tile_prefix[tile];
 	}
 	uint32_t carry_small = seed >> 16, carry_big = seed & 0xffffu; /* both < R */
 
@@ -423,7 +444,7 @@ __global__ __launch_bounds__(kThreads) void stripe_emit_kernel(
 		carry_big = mod_rails(carry_big + (tot & 0xffffu), p);
 		__syncthreads();
 	}
-	if (INLINE && blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
+	if (INLINE && tile == num_tiles - 1 && threadIdx.x == 0) {
 		/* the carries after the last tile are the counters the next batch starts from;
 		 * nobody reads them any more in this launch (the seed was snapshotted) */
 		state->rr_small_counter = carry_small;
@@ -490,14 +511,17 @@ void launch_batch(hipStream_t s, uint32_t tiles, const uint64_t *d_sizes, uint32
 {
 	hipLaunchKernelGGL(stripe_count_kernel<PASSES>, dim3(tiles), dim3(kThreads), 0, s, d_sizes, n, d_state,
 			   align, totals, seed0, err);
+	const uint32_t xcd_run_shift = n >= kXcdRunBatch ? kXcdRunShift : 0u;
+	const uint32_t xcd_run = 1u << xcd_run_shift;
+	const uint32_t emit_grid = (tiles + 8u * xcd_run - 1u) / (8u * xcd_run) * (8u * xcd_run);
 	if (tiles <= kInlineTiles) {
-		hipLaunchKernelGGL((stripe_emit_kernel<true, PASSES>), dim3(tiles), dim3(kThreads), 0, s, d_sizes, n,
-				   d_state, align, totals, seed0, d_num_xfers, d_xfers);
+		hipLaunchKernelGGL((stripe_emit_kernel<true, PASSES>), dim3(emit_grid), dim3(kThreads), 0, s, d_sizes, n,
+				   d_state, align, totals, seed0, tiles, xcd_run_shift, d_num_xfers, d_xfers);
 	} else {
 		hipLaunchKernelGGL(stripe_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, totals, tiles, d_state,
 				   prefix, err);
-		hipLaunchKernelGGL((stripe_emit_kernel<false, PASSES>), dim3(tiles), dim3(kThreads), 0, s, d_sizes, n,
-				   d_state, align, prefix, seed0, d_num_xfers, d_xfers);
+		hipLaunchKernelGGL((stripe_emit_kernel<false, PASSES>), dim3(emit_grid), dim3(kThreads), 0, s, d_sizes, n,
+				   d_state, align, prefix, seed0, tiles, xcd_run_shift, d_num_xfers, d_xfers);
 	}
 }
 
