@@ -297,6 +297,7 @@ PROTOTYPES = {
     "ofi_amd_eager_copy_batch": (ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_u32, c_vp, c_vp,
                                                 c_vp]),
     "ofi_amd_copy_table": (ctypes.c_int, [c_vp, c_vp, c_vp, c_u32, c_vp]),
+    "ofi_amd_copy_table_pieces": (ctypes.c_int, [c_vp, c_vp, c_vp, c_u32, c_u32, c_vp]),
     "ofi_amd_gin_loopback_run": (ctypes.c_int, [c_vp, c_u64, c_vp, c_vp, c_u32, ctypes.POINTER(GinSignalRegion), c_u32,
                                                 c_u32, c_u32, c_u32, c_u32, c_u32, c_vp,
                                                 ctypes.POINTER(GinLoopbackStats)]),

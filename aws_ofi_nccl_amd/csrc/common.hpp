@@ -62,6 +62,7 @@ enum : uint32_t {
 	ASYNC_ERR_BOUNCE_RANGE = 1u << 0, /* destination range outside arena or misaligned */
 	ASYNC_ERR_GIN_TIMEOUT = 1u << 1,  /* producer gave up on a full ring */
 	ASYNC_ERR_SCHED_STATE = 1u << 2,  /* scheduler state unusable (rails, stripe size) */
+	ASYNC_ERR_COPY_LENGTH = 1u << 3,  /* a copy-table entry longer than the stated maximum */
 };
 
 } // namespace ofi_amd

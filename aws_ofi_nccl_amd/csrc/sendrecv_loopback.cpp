@@ -17,7 +17,7 @@
 
 namespace {
 
-constexpr uint32_t kPiece = 256u << 10;  /* a long write is cut so that no wavefront copies more */
+constexpr uint32_t kPiece = 1u << 30;    /* a table entry's length is 32 bits: longer writes are cut */
 constexpr uint32_t kRxStride = 8320;     /* 8192 + header room, rounded to the 128-byte rx alignment */
 constexpr int64_t kEagerSendSize = 8192; /* OFI_NCCL_EAGER_MAX_SIZE default, src/nccl_ofi_rdma.cpp:6808 */
 
@@ -192,7 +192,7 @@ extern "C" int ofi_amd_sendrecv_loopback_run(const uint64_t *src_addrs, const ui
 		/* ---- the wire: one table of device copies for everything the sender handed out ---- */
 		uint64_t *src = t_src.as<uint64_t>(), *dst = t_dst.as<uint64_t>();
 		uint32_t *len = t_len.as<uint32_t>();
-		uint32_t n_copy = 0, n_eager = 0;
+		uint32_t n_copy = 0, n_eager = 0, longest = OFI_AMD_EAGER_HEADER_SIZE;
 		for (open_msg_t &m : open) {
 			const ofi_amd_send_action_t &a = m.action;
 			if (a.kind == OFI_AMD_SEND_EAGER) {
@@ -205,6 +205,7 @@ extern "C" int ofi_amd_sendrecv_loopback_run(const uint64_t *src_addrs, const ui
 					src[n_copy] = src_addrs[m.index];
 					dst[n_copy] = slot + OFI_AMD_EAGER_HEADER_SIZE;
 					len[n_copy++] = static_cast<uint32_t>(a.size);
+					longest = a.size > longest ? static_cast<uint32_t>(a.size) : longest;
 				}
 				rc = ofi_amd_recv_comm_eager_arrival(rcv, a.msg_seq_num, &a.hdr, static_cast<uint32_t>(a.size),
 								     n_eager);
@@ -218,6 +219,7 @@ extern "C" int ofi_amd_sendrecv_loopback_run(const uint64_t *src_addrs, const ui
 						src[n_copy] = src_addrs[m.index] + x.offset + off;
 						dst[n_copy] = a.remote_buff_offset + x.offset + off;
 						len[n_copy++] = static_cast<uint32_t>(n);
+						longest = n > longest ? static_cast<uint32_t>(n) : longest;
 					}
 					rc = ofi_amd_recv_comm_write_arrival(rcv, a.imm, x.msg_size);
 					st.rdma_writes++;
@@ -233,8 +235,10 @@ extern "C" int ofi_amd_sendrecv_loopback_run(const uint64_t *src_addrs, const ui
 			}
 		}
 		if (rc == 0 && n_copy) {
-			rc = ofi_amd_copy_table(t_src.dev_as<uint64_t>(), t_dst.dev_as<uint64_t>(), t_len.dev_as<uint32_t>(),
-						n_copy, stream);
+			/* a write is one table entry whatever its length: the launch gives every 8 KiB of it
+			 * a wavefront of its own */
+			rc = ofi_amd_copy_table_pieces(t_src.dev_as<uint64_t>(), t_dst.dev_as<uint64_t>(),
+						       t_len.dev_as<uint32_t>(), n_copy, longest, stream);
 			st.launches++;
 			st.copy_entries += n_copy;
 		}

@@ -80,7 +80,8 @@ int ofi_amd_gpu_stream_synchronize(void *stream);
  * a bit in a library-owned pinned word.  Fetch-and-clear it after synchronising:
  * bit 0 = bounce destination out of range / misaligned, bit 1 = GIN producer
  * timed out, bit 2 = scheduler state unusable (num_rails outside 1..4 or a zero
- * min_stripe_size; the batch is then left unwritten). */
+ * min_stripe_size; the batch is then left unwritten), bit 3 = an entry of
+ * ofi_amd_copy_table_pieces longer than max_len (its bytes beyond are not copied). */
 int ofi_amd_async_error_fetch(uint32_t *bits);
 
 /* ======================================================================
@@ -198,6 +199,18 @@ int ofi_amd_eager_copy_batch(const void *rx_base, const uint64_t *d_rx_off, cons
  */
 int ofi_amd_copy_table(const uint64_t *d_src_addr, const uint64_t *d_dst_addr, const uint32_t *d_len,
 		       uint32_t n, void *stream);
+
+/*
+ * The same copies for tables that hold long entries: one wavefront per 8 KiB piece of an
+ * entry rather than per entry, so that a few long RDMA writes (a rendezvous message's
+ * stripes: one fi_writedata per rail, src/nccl_ofi_rdma.cpp:2447-2479) are swept by the whole chip
+ * instead of by one wavefront each, and the caller need not cut them.  max_len >= every
+ * d_len[i]; the launch has n * ceil(max_len / 8192) wavefronts (-E2BIG beyond 2^31 - 1: split
+ * the table), those past the end of their entry leave at once.  An entry longer than max_len
+ * is copied up to that bound and reported through ofi_amd_async_error_fetch (bit 3).
+ */
+int ofi_amd_copy_table_pieces(const uint64_t *d_src_addr, const uint64_t *d_dst_addr, const uint32_t *d_len,
+			      uint32_t n, uint32_t max_len, void *stream);
 
 /* Flush only: d_flush[i] = 4 bytes at d_arena + d_dst_off[i], read with
  * device-scope acquire semantics (the C5 read-back without a copy). */

@@ -219,7 +219,7 @@ typedef struct {
 	uint64_t eager_messages;
 	uint64_t write_messages;
 	uint64_t rdma_writes;   /* stripes */
-	uint64_t copy_entries;  /* table entries of the wire launches (stripes cut to 256 KiB) */
+	uint64_t copy_entries;  /* table entries of the wire launches: one per eager header, eager payload and RDMA write */
 	uint64_t rounds;
 	uint64_t launches;
 	uint64_t send_again;    /* isend calls answered "call again" */

@@ -242,6 +242,53 @@ def test_copy_table_matches_a_host_replay(lib, gpu):
     assert lib.ofi_amd_copy_table(a_src.data_ptr(), a_dst.data_ptr(), d_len.data_ptr(), 0, _gpu.stream()) == 0
 
 
+def test_copy_table_in_pieces_matches_a_host_replay(lib, gpu):
+    """The same table through the launch that gives every 8 KiB of an entry its own wavefront: a few
+    long entries (up to 5 MiB) among many short and empty ones, any alignment; lengths at and
+    round the 8 KiB piece size; a maximum that is not a multiple of the piece size; an entry longer
+    than the stated maximum is copied up to it and reported."""
+    rng = np.random.default_rng(7)
+    edge = [0, 1, 63, 64, 65, 8191, 8192, 8193, 16383, 16384, 16385, 3 * 8192 + 100]
+    lens = np.concatenate([rng.integers(0, 300, 400), (2 ** rng.uniform(3, 22.3, 200)).astype(np.int64),
+                           np.array(edge * 3)]).astype(np.uint32)
+    n = len(lens)
+    src = rng.integers(0, 256, 32 << 20, dtype=np.uint8)
+    src_off = rng.integers(0, len(src) - int(lens.max()), n).astype(np.uint64)
+    gaps = rng.integers(0, 70, n).astype(np.uint64)
+    dst_off = (np.cumsum(lens.astype(np.uint64) + gaps) - lens.astype(np.uint64)).astype(np.uint64)
+    total = int(dst_off[-1] + lens[-1]) + 128
+    d_src = _gpu.to_dev(src)
+    a_src = _gpu.to_dev(src_off + np.uint64(d_src.data_ptr()))
+    d_len = _gpu.to_dev(lens)
+    want = np.full(total, 0x77, dtype=np.uint8)
+    for s, d, l in zip(src_off, dst_off, lens):
+        want[int(d):int(d) + int(l)] = src[int(s):int(s) + int(l)]
+    for max_len in (int(lens.max()), int(lens.max()) + 12345, 0xFFFFFFFF // 64):
+        d_dst = torch.full((total,), 0x77, dtype=torch.uint8, device="cuda")
+        a_dst = _gpu.to_dev(dst_off + np.uint64(d_dst.data_ptr()))
+        assert lib.ofi_amd_copy_table_pieces(a_src.data_ptr(), a_dst.data_ptr(), d_len.data_ptr(), n, max_len,
+                                             _gpu.stream()) == 0
+        _gpu.sync()
+        assert np.array_equal(d_dst.cpu().numpy(), want), max_len
+        assert _gpu.fetch_async_errors(lib) == 0
+    # a stated maximum of 20,000 bytes is three pieces: longer entries stop at 24,576 bytes, bit 3 is set
+    d_dst = torch.full((total,), 0x77, dtype=torch.uint8, device="cuda")
+    a_dst = _gpu.to_dev(dst_off + np.uint64(d_dst.data_ptr()))
+    assert lib.ofi_amd_copy_table_pieces(a_src.data_ptr(), a_dst.data_ptr(), d_len.data_ptr(), n, 20000,
+                                         _gpu.stream()) == 0
+    _gpu.sync()
+    cut = np.full(total, 0x77, dtype=np.uint8)
+    for s, d, l in zip(src_off, dst_off, lens):
+        l = min(int(l), 24576)
+        cut[int(d):int(d) + l] = src[int(s):int(s) + l]
+    assert np.array_equal(d_dst.cpu().numpy(), cut)
+    assert _gpu.fetch_async_errors(lib) == 8
+    assert lib.ofi_amd_copy_table_pieces(None, a_dst.data_ptr(), d_len.data_ptr(), 1, 64, _gpu.stream()) == -22
+    assert lib.ofi_amd_copy_table_pieces(a_src.data_ptr(), a_dst.data_ptr(), d_len.data_ptr(), 0, 64, _gpu.stream()) == 0
+    assert lib.ofi_amd_copy_table_pieces(a_src.data_ptr(), a_dst.data_ptr(), d_len.data_ptr(), 1 << 20, 0xFFFFFFFF,
+                                         _gpu.stream()) == -7   # 2^20 entries x 2^19 pieces: split the table
+
+
 def test_bad_arguments(lib, gpu):
     rings = ctypes.c_void_p()
     assert lib.ofi_amd_gin_rings_create(1, 256, ctypes.byref(rings)) == 0

@@ -104,8 +104,8 @@ def test_power_of_two_sweep_large_messages(lib, gpu, size, count):
         assert bool((dsts[i][size // 2:] == 0x4DCD).all()), (i, "wrote past the receive buffer")
     assert stats.messages == count and stats.payload_bytes == size * count
     assert stats.write_messages == count and stats.rdma_writes == 4 * count and stats.eager_messages == 0
-    # every stripe is cut into 256 KiB table entries: size / 4 rails / 256 KiB each
-    assert stats.copy_entries == count * 4 * (size // 4 // (256 << 10))
+    # one table entry per RDMA write: a stripe is not cut (the copy launch gives each 8 KiB a wavefront)
+    assert stats.copy_entries == count * 4
 
 
 def test_receiver_first_sends_everything_as_writes(lib, gpu):
