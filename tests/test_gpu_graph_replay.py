@@ -75,6 +75,8 @@ def test_graph_of_hot_path_launches_replays_exactly(lib, oracle, gpu):
     d_tsrc = _gpu.to_dev(t_src_off + np.uint64(d_src.data_ptr()))
     d_tdst = _gpu.to_dev(t_dst_off + np.uint64(d_tarena.data_ptr()))
     d_tlen = _gpu.to_dev(t_len)
+    d_parena = torch.zeros_like(d_tarena)    # the same table through the launch with a wavefront per 8 KiB
+    d_pdst = _gpu.to_dev(t_dst_off + np.uint64(d_parena.data_ptr()))
     want_tarena = np.zeros(d_tarena.numel(), dtype=np.uint8)
     for a, b, l in zip(t_src_off, t_dst_off, t_len):
         want_tarena[int(b):int(b) + int(l)] = src[int(a):int(a) + int(l)]
@@ -84,6 +86,8 @@ def test_graph_of_hot_path_launches_replays_exactly(lib, oracle, gpu):
                                             d_earena.data_ptr(), d_edst.data_ptr(), d_elen.data_ptr(), n_e,
                                             d_copied.data_ptr(), None, sp) == 0
         assert lib.ofi_amd_copy_table(d_tsrc.data_ptr(), d_tdst.data_ptr(), d_tlen.data_ptr(), n_t, sp) == 0
+        assert lib.ofi_amd_copy_table_pieces(d_tsrc.data_ptr(), d_pdst.data_ptr(), d_tlen.data_ptr(), n_t, 70000,
+                                             sp) == 0
         assert lib.ofi_amd_sched_batch(d_state.data_ptr(), d_sizes.data_ptr(), n_msg, 128, d_num.data_ptr(),
                                        d_xf.data_ptr(), sp) == 0
         assert lib.ofi_amd_bounce_scatter(d_src.data_ptr(), d_src.numel(), d_arena.data_ptr(), w["arena_bytes"],
@@ -112,6 +116,7 @@ def test_graph_of_hot_path_launches_replays_exactly(lib, oracle, gpu):
         d_arena.zero_()
         d_earena.zero_()
         d_tarena.zero_()
+        d_parena.zero_()
         d_copied.zero_()
         d_flush.zero_()
         d_num.fill_(-1)
@@ -130,6 +135,7 @@ def test_graph_of_hot_path_launches_replays_exactly(lib, oracle, gpu):
         assert np.array_equal(d_earena.cpu().numpy(), want_earena), replay
         assert np.array_equal(_gpu.to_host(d_copied, np.uint32), e_len), replay
         assert np.array_equal(d_tarena.cpu().numpy(), want_tarena), replay
+        assert np.array_equal(d_parena.cpu().numpy(), want_tarena), replay
         assert np.array_equal(_gpu.to_host(d_flush, np.uint32), want_flush), replay
         with np.errstate(over="ignore"):
             counters += per_replay
