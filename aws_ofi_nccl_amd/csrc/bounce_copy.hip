@@ -55,14 +55,10 @@
 #include "common.hpp"
 #include "ofi_amd_hotpath.h"
 
+/* Both were swept on the configured batch: 2 or 4 wavefronts per workgroup and XCD runs of 8 to
+ * 256 measure the same or slower. */
 #ifndef OFI_BOUNCE_WAVES
 #define OFI_BOUNCE_WAVES 1 /* buffers (= wavefronts) per workgroup */
-#endif
-#ifndef OFI_BOUNCE_NEIGHBOUR
-#define OFI_BOUNCE_NEIGHBOUR 1 /* shifted path: the dword after a lane's 16 bytes comes from the next lane */
-#endif
-#ifndef OFI_BOUNCE_TAIL64
-#define OFI_BOUNCE_TAIL64 1 /* the byte-wise tail takes the whole last 64-byte unit */
 #endif
 #ifndef OFI_BOUNCE_GROUP
 #define OFI_BOUNCE_GROUP 32 /* consecutive workgroups that share an XCD */
@@ -80,11 +76,6 @@ constexpr int kWavesPerBlock = OFI_BOUNCE_WAVES;
 constexpr int kBlock = 64 * kWavesPerBlock;
 constexpr uint32_t kXcds = 8;
 constexpr uint32_t kGroup = OFI_BOUNCE_GROUP;
-#ifndef OFI_BOUNCE_LDS
-#define OFI_BOUNCE_LDS 0
-#endif
-/* Unused LDS requested per workgroup: caps the workgroups resident on a CU (160 KiB each). */
-constexpr uint32_t kLdsPerBlock = OFI_BOUNCE_LDS;
 constexpr uint32_t kRows = 8;              /* rows of 64 x 16 bytes per trip: 8 KiB per wave */
 constexpr uint32_t kTripVec = kRows * 64u; /* 16-byte words per trip */
 
@@ -112,11 +103,10 @@ __device__ __forceinline__ void copy_rows(const uint8_t *__restrict__ s, uint8_t
 		}
 		const uint8_t *p = s + ((uint64_t)j << 4);
 		v[k] = load16_dword_aligned(p);
-		if (SHIFTED && (!OFI_BOUNCE_NEIGHBOUR || k == R - 1)) {
+		if (SHIFTED && k == R - 1) {
 			x[k] = *reinterpret_cast<const uint32_t *>(p + 16);
 		}
 	}
-#if OFI_BOUNCE_NEIGHBOUR
 	if (SHIFTED) {
 		/* The dword that follows a lane's 16 bytes is the first dword of the next lane's: it
 		 * comes over from the neighbour (one wave-wide DPP shift; lane 63 takes lane 0 of the
@@ -130,7 +120,6 @@ __device__ __forceinline__ void copy_rows(const uint8_t *__restrict__ s, uint8_t
 			x[k] = lane == 63u ? wrap : from_next;
 		}
 	}
-#endif
 #pragma unroll
 	for (int k = 0; k < R; k++) {
 		uint32_t j = (uint32_t)k * 64u + lane;
@@ -215,7 +204,7 @@ __global__ __launch_bounds__(kBlock) void bounce_scatter_kernel(
 		 * than by the end of a row and by the tail.  Tail bytes first, so their latency
 		 * overlaps the body; unpredicated (lanes without a tail byte re-copy the buffer's
 		 * last byte) to stay branch-free */
-		const uint32_t nvec = OFI_BOUNCE_TAIL64 ? (bytes >> 6) << 2 : bytes >> 4;
+		const uint32_t nvec = (bytes >> 6) << 2;
 		const uint32_t tail_at = min((nvec << 4) + lane, bytes - 1u);
 		const uint8_t tail_byte = s[tail_at];
 
@@ -260,7 +249,7 @@ __device__ __forceinline__ void copy_any(const uint8_t *__restrict__ s, uint8_t 
 	if (rem != 0) {
 		const uint8_t *s2 = s + head;
 		uint8_t *d2 = d + head;
-		const uint32_t nvec = OFI_BOUNCE_TAIL64 ? (rem >> 6) << 2 : rem >> 4; /* as in the bounce copy */
+		const uint32_t nvec = (rem >> 6) << 2; /* as in the bounce copy */
 		const uint32_t tail_at = min((nvec << 4) + lane, rem - 1u);
 		const uint8_t tail_byte = s2[tail_at];
 		const uint32_t shift = (uint32_t)(reinterpret_cast<uintptr_t>(s2) & 3u);
@@ -452,7 +441,7 @@ int ofi_amd_bounce_scatter(const void *d_src, uint64_t src_bytes, void *d_arena,
 	uint32_t blocks = (n + kWavesPerBlock - 1) / kWavesPerBlock;
 	const uint32_t round = kXcds * kGroup; /* whole rounds over the XCDs */
 	blocks = (blocks + round - 1) / round * round;
-	hipLaunchKernelGGL(bounce_scatter_kernel, dim3(blocks), dim3(kBlock), kLdsPerBlock, as_stream(stream),
+	hipLaunchKernelGGL(bounce_scatter_kernel, dim3(blocks), dim3(kBlock), 0, as_stream(stream),
 			   static_cast<const uint8_t *>(d_src), src_bytes, static_cast<uint8_t *>(d_arena),
 			   arena_bytes, d_src_off, d_dst_off, d_len, n, d_flush, err);
 	OFI_AMD_HIP_TRY(hipGetLastError());
