@@ -15,6 +15,10 @@ nothing else of interest, which keeps counter runs short.  The shapes:
                          the reference point that scales FETCH_SIZE / WRITE_SIZE
   fill      <MiB>        torch's fill of that many MiB (default 100): what the chip sustains when a
                          kernel only writes
+  table     <MiB>        --buffers (default 64) copies of that many MiB each (default 16), sources and
+                         destinations 4 KiB-aligned and apart: whole entries through
+                         ofi_amd_copy_table_pieces (a wavefront per 8 KiB), or with --cut the same
+                         bytes as 256 KiB entries through ofi_amd_copy_table (a wavefront per entry)
   striping  1m | 16m     1,000,000 / 16,000,000 message sizes, 4 rails
   model     64 | 256     tuner cost-model grids per launch
   region    64           tuner region grids per launch
@@ -35,10 +39,12 @@ SEED = 1234
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--kernel", required=True, choices=["bounce", "copy", "fill", "striping", "model", "region", "eager"])
+    ap.add_argument("--kernel", required=True, choices=["bounce", "copy", "fill", "table", "striping", "model", "region", "eager"])
     ap.add_argument("--shape", default=None)
     ap.add_argument("--launches", type=int, default=30)
-    ap.add_argument("--buffers", type=int, default=65536, help="bounce aligned8k / dense8k: buffer count")
+    ap.add_argument("--buffers", type=int, default=None,
+                    help="bounce aligned8k / dense8k: buffer count (default 65,536); table: entries (default 64)")
+    ap.add_argument("--cut", action="store_true", help="table: 256 KiB entries, one wavefront each")
     ap.add_argument("--no-flush", action="store_true", help="bounce / eager: no read-back")
     ap.add_argument("--graph", action="store_true",
                     help="record one call into a HIP graph and replay it --launches times")
@@ -68,7 +74,7 @@ def main():
         w = synthetic.bounce_workload(SEED)
         n = len(w["len"])
         if shape in ("aligned8k", "dense8k"):
-            n = args.buffers
+            n = args.buffers or 65536
             if not 0 < n <= (2 << 30) // 8192:
                 ap.error("--buffers out of range")
             length = np.full(n, 8192, dtype=np.uint32)
@@ -101,6 +107,23 @@ def main():
         d_fill = torch.empty(int(args.shape or "100") << 20, dtype=torch.uint8, device="cuda")
         step = lambda: d_fill.fill_(7)
         print("bytes written per launch: %d" % d_fill.numel())
+    elif args.kernel == "table":
+        entries, each = args.buffers or 64, int(args.shape or "16") << 20
+        if not 0 < entries * each <= 64 << 30:
+            ap.error("--buffers x --shape out of range")
+        d_from = torch.randint(0, 255, (entries * each,), dtype=torch.uint8, device="cuda")
+        d_to = torch.zeros(entries * each, dtype=torch.uint8, device="cuda")
+        piece = (256 << 10) if args.cut else each
+        starts = np.arange(0, entries * each, piece, dtype=np.uint64)
+        d_s, d_d = dev(starts + np.uint64(d_from.data_ptr())), dev(starts + np.uint64(d_to.data_ptr()))
+        d_l = dev(np.full(len(starts), piece, dtype=np.uint32))
+        if args.cut:
+            step = lambda: m.check(lib.ofi_amd_copy_table(d_s.data_ptr(), d_d.data_ptr(), d_l.data_ptr(), len(starts),
+                                                          stream), "copy_table")
+        else:
+            step = lambda: m.check(lib.ofi_amd_copy_table_pieces(d_s.data_ptr(), d_d.data_ptr(), d_l.data_ptr(),
+                                                                 len(starts), piece, stream), "copy_table_pieces")
+        print("bytes copied per launch: %d in %d table entries" % (entries * each, len(starts)))
     elif args.kernel == "eager":
         n, stride = 65536, 8320
         rng = np.random.default_rng(SEED)
