@@ -55,13 +55,24 @@
 #include "common.hpp"
 #include "ofi_amd_hotpath.h"
 
-/* Both were swept on the configured batch: 2 or 4 wavefronts per workgroup and XCD runs of 8 to
- * 256 measure the same or slower. */
+/* Swept on the configured batch over thousands of launches in a row (1, 2, 4, 8 or 16
+ * wavefronts per workgroup, XCD runs of 8 to 128 buffers): 8 wavefronts per workgroup with runs
+ * of 32 buffers per XCD was the fastest (91.1 us per launch; 1 x 32: 92.7, 4 x 8: 91.8,
+ * 16 x 2: 92.6). */
 #ifndef OFI_BOUNCE_WAVES
-#define OFI_BOUNCE_WAVES 1 /* buffers (= wavefronts) per workgroup */
+#define OFI_BOUNCE_WAVES 8 /* buffers (= wavefronts) per workgroup */
+#endif
+#ifndef OFI_EAGER_WAVES
+#define OFI_EAGER_WAVES 1
+#endif
+#ifndef OFI_EAGER_GROUP
+#define OFI_EAGER_GROUP 32
+#endif
+#ifndef OFI_TABLE_WAVES
+#define OFI_TABLE_WAVES 1
 #endif
 #ifndef OFI_BOUNCE_GROUP
-#define OFI_BOUNCE_GROUP 32 /* consecutive workgroups that share an XCD */
+#define OFI_BOUNCE_GROUP 4 /* consecutive workgroups that share an XCD */
 #endif
 
 namespace {
@@ -74,6 +85,9 @@ struct __attribute__((packed, aligned(4))) dword_aligned_u32x4 {
 
 constexpr int kWavesPerBlock = OFI_BOUNCE_WAVES;
 constexpr int kBlock = 64 * kWavesPerBlock;
+constexpr int kEagerWaves = OFI_EAGER_WAVES;
+constexpr uint32_t kEagerGroup = OFI_EAGER_GROUP;
+constexpr int kTableWaves = OFI_TABLE_WAVES;
 constexpr uint32_t kXcds = 8;
 constexpr uint32_t kGroup = OFI_BOUNCE_GROUP;
 constexpr uint32_t kRows = 8;              /* rows of 64 x 16 bytes per trip: 8 KiB per wave */
@@ -82,6 +96,20 @@ constexpr uint32_t kTripVec = kRows * 64u; /* 16-byte words per trip */
 __device__ __forceinline__ u32x4 load16_dword_aligned(const uint8_t *p)
 {
 	return reinterpret_cast<const dword_aligned_u32x4 *>(p)->v;
+}
+
+/*
+ * Every access to a destination carries the same cache policy, the streaming one: the 16-byte
+ * stores of the rows, the single head and tail bytes and the read-back of the flush.  With the
+ * rows streaming and the tail bytes and the read-back as ordinary accesses, the same batch
+ * launched over and over on the same buffers slowed down by 6 % within 2,000 launches (91 ->
+ * 97 us; fewer and fewer of those ordinary lines leave the L2 between launches, and a read
+ * sweep of 16 MiB of other memory brought the first rate back); with one policy the rate does
+ * not move (91 us from the first launch to the 20,000th).
+ */
+__device__ __forceinline__ void store_byte_streaming(uint8_t *p, uint8_t v)
+{
+	__builtin_nontemporal_store(v, p);
 }
 
 /*
@@ -214,14 +242,13 @@ __global__ __launch_bounds__(kBlock) void bounce_scatter_kernel(
 		} else {
 			copy_words<true>(s - shift, d, nvec, shift, lane);
 		}
-		d[tail_at] = tail_byte;
+		store_byte_streaming(d + tail_at, tail_byte);
 	}
 
 	if (flush != nullptr) {
 		__builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
 		if (lane == 0) {
-			flush[buf] = __hip_atomic_load(reinterpret_cast<const uint32_t *>(d),
-						       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+			flush[buf] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(d));
 		}
 	}
 }
@@ -258,9 +285,9 @@ __device__ __forceinline__ void copy_any(const uint8_t *__restrict__ s, uint8_t 
 		} else {
 			copy_words<true>(s2 - shift, d2, nvec, shift, lane);
 		}
-		d2[tail_at] = tail_byte;
+		store_byte_streaming(d2 + tail_at, tail_byte);
 	}
-	d[head_at] = head_byte;
+	store_byte_streaming(d + head_at, head_byte);
 }
 
 /*
@@ -268,7 +295,7 @@ __device__ __forceinline__ void copy_any(const uint8_t *__restrict__ s, uint8_t 
  * payload, which goes to a receive buffer at any alignment, truncated to that buffer's
  * length (rdma_eager_copy_req::post, src/nccl_ofi_rdma.cpp:2729-2776).
  */
-__global__ __launch_bounds__(kBlock) void eager_copy_kernel(
+__global__ __launch_bounds__(64 * kEagerWaves) void eager_copy_kernel(
 	const uint8_t *__restrict__ rx_base, const uint64_t *__restrict__ rx_off,
 	const uint32_t *__restrict__ recv_len, uint8_t *__restrict__ dst_base,
 	const uint64_t *__restrict__ dst_off, const uint32_t *__restrict__ dst_len, uint32_t n,
@@ -278,8 +305,8 @@ __global__ __launch_bounds__(kBlock) void eager_copy_kernel(
 	const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 	const uint32_t xcd = blockIdx.x % kXcds;
 	const uint32_t turn = blockIdx.x / kXcds;
-	const uint32_t wg = ((turn / kGroup) * kXcds + xcd) * kGroup + turn % kGroup;
-	const uint32_t buf = wg * kWavesPerBlock + wave;
+	const uint32_t wg = ((turn / kEagerGroup) * kXcds + xcd) * kEagerGroup + turn % kEagerGroup;
+	const uint32_t buf = wg * kEagerWaves + wave;
 	if (buf >= n) {
 		return;
 	}
@@ -299,8 +326,7 @@ __global__ __launch_bounds__(kBlock) void eager_copy_kernel(
 		 * then the four are combined inside the quad */
 		uint32_t word = 0;
 		if (lane < min(bytes, 4u)) {
-			word = (uint32_t)__hip_atomic_load(d + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)
-			       << (8u * lane);
+			word = (uint32_t)__builtin_nontemporal_load(d + lane) << (8u * lane);
 		}
 		word |= __shfl_xor(word, 1, 64);
 		word |= __shfl_xor(word, 2, 64);
@@ -311,13 +337,13 @@ __global__ __launch_bounds__(kBlock) void eager_copy_kernel(
 }
 
 /* One wavefront per (source address, destination address, length) entry. */
-__global__ __launch_bounds__(kBlock) void copy_table_kernel(const uint64_t *__restrict__ src_addr,
+__global__ __launch_bounds__(64 * kTableWaves) void copy_table_kernel(const uint64_t *__restrict__ src_addr,
 							     const uint64_t *__restrict__ dst_addr,
 							     const uint32_t *__restrict__ len, uint32_t n)
 {
 	const uint32_t lane = threadIdx.x & 63u;
 	const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-	const uint32_t i = blockIdx.x * kWavesPerBlock + wave;
+	const uint32_t i = blockIdx.x * kTableWaves + wave;
 	if (i >= n) {
 		return;
 	}
@@ -462,10 +488,10 @@ int ofi_amd_eager_copy_batch(const void *rx_base, const uint64_t *d_rx_off, cons
 	if (!rx_base || !d_rx_off || !d_recv_len || !d_dst_off || !d_dst_len || n > (1u << 30)) {
 		return -EINVAL;
 	}
-	uint32_t blocks = (n + kWavesPerBlock - 1) / kWavesPerBlock;
-	const uint32_t round = kXcds * kGroup;
+	uint32_t blocks = (n + kEagerWaves - 1) / kEagerWaves;
+	const uint32_t round = kXcds * kEagerGroup;
 	blocks = (blocks + round - 1) / round * round;
-	hipLaunchKernelGGL(eager_copy_kernel, dim3(blocks), dim3(kBlock), 0, as_stream(stream),
+	hipLaunchKernelGGL(eager_copy_kernel, dim3(blocks), dim3(64 * kEagerWaves), 0, as_stream(stream),
 			   static_cast<const uint8_t *>(rx_base), d_rx_off, d_recv_len,
 			   static_cast<uint8_t *>(dst_base), d_dst_off, d_dst_len, n, d_copied, d_flush);
 	OFI_AMD_HIP_TRY(hipGetLastError());
@@ -485,7 +511,7 @@ int ofi_amd_copy_table(const uint64_t *d_src_addr, const uint64_t *d_dst_addr, c
 	if (!d_src_addr || !d_dst_addr || !d_len || n > (1u << 30)) {
 		return -EINVAL;
 	}
-	hipLaunchKernelGGL(copy_table_kernel, dim3((n + kWavesPerBlock - 1) / kWavesPerBlock), dim3(kBlock), 0,
+	hipLaunchKernelGGL(copy_table_kernel, dim3((n + kTableWaves - 1) / kTableWaves), dim3(64 * kTableWaves), 0,
 			   as_stream(stream), d_src_addr, d_dst_addr, d_len, n);
 	OFI_AMD_HIP_TRY(hipGetLastError());
 	return 0;

@@ -48,6 +48,13 @@ def main():
     ap.add_argument("--no-flush", action="store_true", help="bounce / eager: no read-back")
     ap.add_argument("--graph", action="store_true",
                     help="record one call into a HIP graph and replay it --launches times")
+    ap.add_argument("--busy-seconds", type=float, default=0.0,
+                    help="before the launches, keep the device busy this long with plain device copies of 256 MiB "
+                         "(another kernel, so that a profiler filtering by kernel name counts only the launches)")
+    ap.add_argument("--per-launch", action="store_true",
+                    help="an event between every two launches: prints the median launch period of the first 100, "
+                         "of every tenth of the run and of the last 1,000 (how the rate moves while the device "
+                         "stays busy)")
     args = ap.parse_args()
 
     import numpy as np
@@ -191,6 +198,31 @@ def main():
         step = graph.replay
         step()
         torch.cuda.synchronize()
+    if args.busy_seconds > 0:
+        import time
+        d_a = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+        d_b = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < args.busy_seconds:
+            for _ in range(200):
+                d_b.copy_(d_a)
+            torch.cuda.synchronize()
+    if args.per_launch:
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.launches + 1)]
+        marks[0].record()
+        for k in range(args.launches):
+            step()
+            marks[k + 1].record()
+        torch.cuda.synchronize()
+        us = np.array([marks[k].elapsed_time(marks[k + 1]) * 1e3 for k in range(args.launches)])
+        print("%s %s: %d launches back to back, %.2f s; median launch period in us:" % (
+            args.kernel, args.shape or "", args.launches, us.sum() / 1e6))
+        print("  first %d: %.2f" % (min(100, len(us)), np.median(us[:100])))
+        for t in range(10):
+            part = us[len(us) * t // 10:len(us) * (t + 1) // 10]
+            print("  tenth %d: %.2f (min %.2f, mean %.2f)" % (t + 1, np.median(part), part.min(), part.mean()))
+        print("  last %d: %.2f" % (min(1000, len(us)), np.median(us[-1000:])))
+        return 0
     e0.record()
     for _ in range(args.launches):
         step()
