@@ -56,6 +56,24 @@ def per_launch_ms(fn, reps, torch):
     return t[len(t) // 2], t[0]
 
 
+def sustained(fn, seconds, est_ms, torch, np):
+    """At least `seconds` of launches back to back, an event after every launch, so that each launch
+    period is known: the figure is the median of the last half, when whatever moves with the time
+    the device has been busy (clocks, caches, memory state) has settled."""
+    n = max(200, int(seconds * 1e3 / est_ms) + 1)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
+    torch.cuda.synchronize()
+    marks[0].record()
+    for k in range(n):
+        fn()
+        marks[k + 1].record()
+    torch.cuda.synchronize()
+    ms = np.array([marks[k].elapsed_time(marks[k + 1]) for k in range(n)])
+    return {"launches": n, "seconds": float(ms.sum() / 1e3), "ms_median_last_half": float(np.median(ms[n // 2:])),
+            "ms_median_first_100": float(np.median(ms[:100])), "ms_median_last_1000": float(np.median(ms[-1000:])),
+            "ms_max_last_half": float(ms[n // 2:].max())}
+
+
 def run_threads(fn, parts):
     """fn(part) on one thread per part (oracle calls run outside the interpreter lock); seconds."""
     import threading
@@ -112,6 +130,11 @@ def bench_bounce(lib, oracle, torch, np, args):
     wall_ms, ev_ms = timed_steps(step, args.steps, args.warmup, torch)
     med_ms, min_ms = per_launch_ms(step, max(10, args.steps), torch)
     algo_bytes = 2 * w["src_bytes"] + 8 * n          # payload read + write, 4 B flush read + 4 B write
+    sus = None
+    if args.sustain_seconds > 0:
+        sus = sustained(step, args.sustain_seconds, med_ms, torch, np)
+        sus["achieved"] = algo_bytes / sus["ms_median_last_half"] / 1e6
+        sus["frac"] = sus["achieved"] / HBM_PEAK_GBS
     # result check of the timed configuration: every flush word and every byte of the 2 GiB arena
     # (the untouched ones included) against the oracle's, compared on the device
     arena = np.zeros(w["arena_bytes"], dtype=np.uint8)
@@ -125,11 +148,18 @@ def bench_bounce(lib, oracle, torch, np, args):
     del d_want
     # plain device copy of the same payload, as the practical ceiling
     d_tmp = torch.empty(w["src_bytes"], dtype=torch.uint8, device="cuda")
-    _, copy_ms = timed_steps(lambda: d_tmp.copy_(d_src[:w["src_bytes"]]), args.steps, 3, torch)
+    copy_step = lambda: d_tmp.copy_(d_src[:w["src_bytes"]])
+    _, copy_ms = timed_steps(copy_step, args.steps, 3, torch)
     out = {"ms_wall": wall_ms, "ms_kernel": ev_ms, "algo_bytes": algo_bytes,
-           "gbs": algo_bytes / ev_ms / 1e6, "gbs_wall": algo_bytes / wall_ms / 1e6,
+           "gbs": algo_bytes / med_ms / 1e6, "gbs_wall": algo_bytes / wall_ms / 1e6,
            "device_copy_gbs": 2 * w["src_bytes"] / copy_ms / 1e6, "parity_ok": ok, "buffers": n,
-           "payload_bytes": w["src_bytes"], "ms_kernel_median": med_ms, "ms_kernel_min": min_ms}
+           "payload_bytes": w["src_bytes"], "ms_kernel_median": med_ms, "ms_kernel_min": min_ms,
+           "sustained": sus}
+    if args.sustain_seconds > 0:
+        c = sustained(copy_step, args.sustain_seconds, copy_ms, torch, np)
+        c["achieved"] = 2 * w["src_bytes"] / c["ms_median_last_half"] / 1e6
+        c["frac"] = c["achieved"] / HBM_PEAK_GBS
+        out["sustained_device_copy"] = c
     cpu = None
     if not args.skip_cpu:
         reps = max(2, min(40, int(8.0 / max(first_cpu_s, 1e-3))))
@@ -224,6 +254,16 @@ def bench_eager(lib, oracle, torch, np, args):
         wall_ms, ev_ms = timed_steps(step, max(3, args.steps // 4), 2, torch)
         out[key] = {"ms_kernel": ev_ms, "payload_gbs": payload / ev_ms / 1e6,
                     "read_plus_written_gbs": 2 * payload / ev_ms / 1e6}
+        if key == "rx_pool_in_hbm":
+            med_ms, min_ms = per_launch_ms(step, max(10, args.steps), torch)
+            out[key].update({"ms_kernel_back_to_back": ev_ms, "ms_kernel": med_ms, "ms_kernel_min": min_ms,
+                             "payload_gbs": payload / med_ms / 1e6, "read_plus_written_gbs": 2 * payload / med_ms / 1e6,
+                             "hbm_frac": 2 * payload / med_ms / 1e6 / HBM_PEAK_GBS})
+            if args.sustain_seconds > 0:
+                c = sustained(step, args.sustain_seconds, med_ms, torch, np)
+                c["achieved"] = 2 * payload / c["ms_median_last_half"] / 1e6
+                c["frac"] = c["achieved"] / HBM_PEAK_GBS
+                out[key]["sustained"] = c
     # result check on a strided sample of the buffers against the oracle's copy
     idx = np.arange(0, n, 97)
     want = np.zeros(len(idx) * 8192, dtype=np.uint8)
@@ -665,6 +705,8 @@ def main():
     ap.add_argument("--skip-extra", action="store_true", help="only the bounce-copy step")
     ap.add_argument("--extra", default="eager,striping,tuner,gin,sendrecv", help="which other paths to time")
     ap.add_argument("--skip-cpu", action="store_true", help="no CPU baselines")
+    ap.add_argument("--sustain-seconds", type=float, default=2.0,
+                    help="length of the back-to-back leg behind roofline.sustained (0: skip it)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU only: this path has no collective or sharded leg "
@@ -709,8 +751,11 @@ def main():
                    "arena_bytes": 2 << 30},
         "roofline": {"bound": "hbm", "achieved": bounce["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": bounce["gbs"] / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": traffic_source,
-                     "kernel": "bounce_scatter_kernel", "kernel_ms": bounce["ms_kernel"],
+                     "kernel": "bounce_scatter_kernel", "kernel_ms": bounce["ms_kernel_median"],
                      "kernel_ms_median": bounce["ms_kernel_median"], "kernel_ms_min": bounce["ms_kernel_min"],
+                     "kernel_ms_back_to_back": bounce["ms_kernel"],
+                     "sustained": bounce["sustained"],
+                     "sustained_device_copy": bounce.get("sustained_device_copy"),
                      "algorithmic_bytes_per_launch": bounce["algo_bytes"],
                      "device_copy_GBps_same_payload": bounce["device_copy_gbs"]},
         "cpu_baseline": cpu,

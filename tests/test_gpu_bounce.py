@@ -284,7 +284,7 @@ def test_gpu_glue(lib, gpu):
     assert lib.ofi_amd_gpu_get_device_for_addr(host.ctypes.data, ctypes.byref(dev)) < 0 and dev.value == -1
 
 
-def test_dma_buf_export_of_device_memory(lib, gpu):
+def test_dma_buf_export_of_device_memory(lib, gpu, capsys):
     """nccl_net_ofi_gpu_get_dma_buf_fd (src/nccl_ofi_rocm.cpp:129-139), called as the reference
     calls it for its flush buffer (src/nccl_ofi_rdma.cpp:3842-3845: a page-aligned address, one
     system page) and for a whole registration: a dma-buf file descriptor and offset 0.  Where the
@@ -295,6 +295,7 @@ def test_dma_buf_export_of_device_memory(lib, gpu):
     assert lib.ofi_amd_gpu_mem_alloc(ctypes.byref(p), 4 << 20) == 0 and p.value % page == 0
     have = lib.ofi_amd_gpu_have_dma_buf_attr()
     assert have in (0, 1)
+    links = []
     for addr, size in ((p.value, page), (p.value + 16 * page, 1 << 20), (p.value, 4 << 20)):
         fd, off = ctypes.c_int(-1), ctypes.c_size_t(99)
         rc = lib.ofi_amd_gpu_get_dma_buf_fd(ctypes.c_void_p(addr), size, ctypes.byref(fd), ctypes.byref(off))
@@ -306,6 +307,7 @@ def test_dma_buf_export_of_device_memory(lib, gpu):
         assert st.st_ino > 0
         link = os.readlink("/proc/self/fd/%d" % fd.value)
         assert "dmabuf" in link, link                            # an anonymous dma-buf inode
+        links.append(link)
         try:
             end = os.lseek(fd.value, 0, os.SEEK_END)             # dma-buf files report their size
             assert end >= size, (end, size)
@@ -314,6 +316,9 @@ def test_dma_buf_export_of_device_memory(lib, gpu):
         os.close(fd.value)
         with pytest.raises(OSError):
             os.fstat(fd.value)                                   # the caller owns the descriptor: closed means gone
+    # which branch ran is part of the result: say so whatever pytest captures
+    with capsys.disabled():
+        print("\n[dma-buf] ofi_amd_gpu_have_dma_buf_attr() = %d; exported descriptors: %s" % (have, links or "none"))
     # the exported memory is untouched and still usable
     data = np.arange(256, dtype=np.uint8)
     back = np.zeros(256, dtype=np.uint8)

@@ -354,6 +354,26 @@ def test_configured_shape_full_size(lib, oracle, gpu):
     lib.ofi_amd_gin_rings_destroy(rings)
 
 
+def test_configured_shape_full_size_derived_stream(lib, oracle, gpu):
+    """The same configured run with the proxy's full work per descriptor: every one of the
+    256,000,000 puts goes through the iputSignal derivation (sequence number, immediate data,
+    stripes, metadata), and every 224-byte wire record is folded, in order, into the checksum that
+    the oracle computes over its own derivation of the same stream.  One proxy thread, as the
+    configuration says; the oracle needs some fifteen seconds on one core."""
+    nctx, cap, ops = 256, 4096, 1_000_000
+    omrs, pmrs = _oracle.default_mrs(), _oracle.default_mrs(m.GinMr)
+    rings = make_rings(lib, nctx, cap)
+    comms = (m.GinComm * nctx)()
+    for c in range(nctx):
+        assert lib.ofi_amd_gin_comm_init(ctypes.byref(comms[c]), c % 1024, 4, 131072, 64, 1) == 0
+    rc, stats, _, _ = produce_and_drain(lib, rings, nctx, ops, mode=3, comms=comms, mrs=pmrs, timeout_ms=30000)
+    assert rc == 0 and lib.ofi_amd_gin_producer_status(rings) == 0
+    assert stats.descriptors == nctx * ops and stats.signals == nctx * (ops // 64)
+    want = oracle.oracle_gin_stream_checksum(SEED, nctx, ops, 1, 64, 1, 1, 1, 4, 131072, 64, 1, omrs)
+    assert stats.checksum == want
+    lib.ofi_amd_gin_rings_destroy(rings)
+
+
 def test_producer_gives_up_when_nobody_drains(lib, gpu):
     """Failure path forced from the host: more ops than slots, no consumer, a tiny spin limit.
     Every wave reaches its exit, the kernel ends, the status word reports the timeout."""

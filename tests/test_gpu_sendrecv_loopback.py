@@ -108,6 +108,44 @@ def test_power_of_two_sweep_large_messages(lib, gpu, size, count):
     assert stats.copy_entries == count * 4
 
 
+@pytest.mark.parametrize("size", [2 << 20, 64 << 20, 1 << 30])
+def test_sixty_four_in_flight_above_one_mebibyte(lib, gpu, size):
+    """The configured depth at the sizes where a message is striped writes: 64 messages open at
+    once, each with a source and a receive buffer of its own (2 x 64 GiB at 1 GiB, which the
+    288 GB of the part hold), random 16-bit words (bf16 bit patterns) generated on the device.
+    Every received byte and the guard words behind each receive buffer are compared on the
+    device (tests/functional/nccl_message_transfer.cpp:45-56 checks the same on the host)."""
+    count, guard = 64, 32
+    free_bytes, _ = torch.cuda.mem_get_info()
+    if 2 * count * (size + 2 * guard) + (4 << 30) > free_bytes:
+        pytest.skip("needs %d GiB of free device memory" % ((2 * count * size) >> 30))
+    src = torch.empty(count * (size // 2), dtype=torch.int16, device="cuda")
+    gen = torch.Generator(device="cuda").manual_seed(size)
+    for k in range(count):
+        src[k * (size // 2):(k + 1) * (size // 2)].random_(-32768, 32767, generator=gen)
+    stride = size // 2 + guard
+    dst = torch.full((count * stride,), 0x4DCD, dtype=torch.int16, device="cuda")
+    pool = torch.zeros(64 * RX_STRIDE, dtype=torch.uint8, device="cuda")
+    a_src = np.array([src.data_ptr() + k * size for k in range(count)], dtype=np.uint64)
+    a_dst = np.array([dst.data_ptr() + 2 * k * stride for k in range(count)], dtype=np.uint64)
+    a_size = np.full(count, size, dtype=np.uint64)
+    stats = m.SendrecvLoopbackStats()
+    torch.cuda.synchronize()
+    rc = lib.ofi_amd_sendrecv_loopback_run(a_src.ctypes.data, a_dst.ctypes.data, a_size.ctypes.data,
+                                           a_size.ctypes.data, None, count, 64, 4, 1, pool.data_ptr(),
+                                           pool.numel(), 0, _gpu.stream(), ctypes.byref(stats))
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    for k in range(count):
+        got = dst[k * stride:(k + 1) * stride]
+        assert torch.equal(got[:size // 2], src[k * (size // 2):(k + 1) * (size // 2)]), (k, size)
+        assert bool((got[size // 2:] == 0x4DCD).all()), (k, "wrote past the receive buffer")
+    assert stats.rounds == 1 and stats.messages == count and stats.payload_bytes == size * count
+    assert stats.write_messages == count and stats.rdma_writes == 4 * count and stats.eager_messages == 0
+    del src, dst
+    torch.cuda.empty_cache()
+
+
 def test_receiver_first_sends_everything_as_writes(lib, gpu):
     sizes = [8, 100, 1024, 8184, 8185, 70000, 300000, 1 << 20] * 8
     st = run(lib, sizes, sizes, 64, flags=1, seed=3)
