@@ -109,7 +109,8 @@ class GinLoopbackStats(ctypes.Structure):
                 ("signals", c_u64), ("work_items", c_u64), ("acks", c_u64), ("launches", c_u64),
                 ("seconds", ctypes.c_double), ("posts_refused", c_u64), ("post_retries", c_u64),
                 ("tx_completions", c_u64), ("pending_max", c_u32), ("requests_max", c_u32), ("reads", c_u64),
-                ("flush_reads", c_u64)]
+                ("flush_reads", c_u64), ("ns_pop_derive", c_u64), ("ns_tx_post", c_u64), ("ns_wire", c_u64),
+                ("ns_progress", c_u64), ("ns_rx", c_u64), ("ns_launch_wait", c_u64)]
 
 
 class GinSignalWork(ctypes.Structure):

@@ -364,7 +364,8 @@ constexpr uint32_t kPieceRunShift = 7;
 __global__ __launch_bounds__(64) void copy_table_pieces_kernel(const uint64_t *__restrict__ src_addr,
 							       const uint64_t *__restrict__ dst_addr,
 							       const uint32_t *__restrict__ len, uint32_t n,
-							       uint32_t pieces_per_entry, uint32_t *__restrict__ err)
+							       uint32_t pieces_per_entry, uint32_t max_len,
+							       uint32_t *__restrict__ err)
 {
 	const uint32_t lane = threadIdx.x;
 	const uint32_t xcd = blockIdx.x % kXcds, turn = blockIdx.x / kXcds;
@@ -374,11 +375,12 @@ __global__ __launch_bounds__(64) void copy_table_pieces_kernel(const uint64_t *_
 	if (e >= n) {
 		return;
 	}
-	const uint32_t bytes = len[e];
-	const uint64_t off = (uint64_t)piece * kPieceBytes;
-	if (piece == pieces_per_entry - 1u && bytes > (uint64_t)pieces_per_entry * kPieceBytes && lane == 0) {
+	const uint32_t stated = len[e];
+	if (piece == 0 && stated > max_len && lane == 0) {
 		atomicOr(err, ofi_amd::ASYNC_ERR_COPY_LENGTH); /* longer than the caller said: the rest stays uncopied */
 	}
+	const uint32_t bytes = min(stated, max_len);
+	const uint64_t off = (uint64_t)piece * kPieceBytes;
 	if (off >= bytes) {
 		return;
 	}
@@ -541,7 +543,7 @@ int ofi_amd_copy_table_pieces(const uint64_t *d_src_addr, const uint64_t *d_dst_
 		return -ENOMEM;
 	}
 	hipLaunchKernelGGL(copy_table_pieces_kernel, dim3((uint32_t)blocks), dim3(64), 0, as_stream(stream), d_src_addr,
-			   d_dst_addr, d_len, n, (uint32_t)pieces_per_entry, err);
+			   d_dst_addr, d_len, n, (uint32_t)pieces_per_entry, max_len, err);
 	OFI_AMD_HIP_TRY(hipGetLastError());
 	return 0;
 }

@@ -92,6 +92,16 @@ inline int derive(ofi_amd_gin_comm_t *c, const ofi_amd_gin_mr_t *mrs, uint32_t n
 		 * cannot, so a full window is handed back to the caller. */
 		return (sop > kSignalAdd || bad_handle) ? -EINVAL : -EAGAIN;
 	}
+	if (!POW2) {
+		/* a communicator edited by hand since comm_init: out-of-range rails are an error, not
+		 * an index (the mask / shift path is only entered with all of this in range) */
+		if (c->num_rails < 1 || c->num_rails > OFI_AMD_MAX_NUM_RAILS || c->next_rail_id >= c->num_rails ||
+		    c->pinned_rail_id >= (int32_t)OFI_AMD_MAX_NUM_RAILS ||
+		    (c->sched.num_rails >= 1 && c->pinned_rail_id >= c->sched.num_rails)) {
+			std::memset(out, 0, sizeof(*out));
+			return -EINVAL;
+		}
+	}
 	const uint32_t seq = head & kImmSeqMask; /* :588 */
 	const bool aggregate = (d->opt_flags & kOptAggregate) != 0;
 	const bool has_signal = sop != 0;
@@ -129,7 +139,10 @@ inline int derive(ofi_amd_gin_comm_t *c, const ofi_amd_gin_mr_t *mrs, uint32_t n
 						: ofi_amd::div_pow2_or_slow(size - 1, st.min_stripe_size));
 		const uint32_t capped = (uint32_t)(want < R ? want : R);
 		const uint32_t n = small ? 1u : ofi_amd::kStripeCount[R - 1][capped - 1];
-		const uint32_t rr_small = st.rr_small_counter, rr_big = st.rr_counter;
+		/* counters at or beyond the rail count are taken modulo it, as the scheduler's own
+		 * increment would leave them */
+		const uint32_t rr_small = POW2 ? st.rr_small_counter : st.rr_small_counter % R;
+		const uint32_t rr_big = POW2 ? st.rr_counter : st.rr_counter % R;
 		const uint32_t first = small ? rr_small : rr_big;
 		st.rr_small_counter = small ? step(rr_small, 1) : rr_small;
 		st.rr_counter = small ? rr_big : step(rr_big, n);
@@ -237,9 +250,15 @@ inline int derive(ofi_amd_gin_comm_t *c, const ofi_amd_gin_mr_t *mrs, uint32_t n
  * counters below the rail count (derive keeps them there) */
 inline bool derive_fast_path(const ofi_amd_gin_comm_t *c)
 {
+	/* The struct is the caller's: a rail count outside 1..4, a zero stripe size or a pin or
+	 * rail cursor beyond the rail count (none of which comm_init or the derivation produce)
+	 * would index the stripe and key tables out of range, so they never take this path. */
 	const uint32_t R = (uint32_t)c->sched.num_rails;
-	return (R & (R - 1)) == 0 && c->sched.rr_small_counter < R && c->sched.rr_counter < R &&
-	       (c->sched.min_stripe_size & (c->sched.min_stripe_size - 1)) == 0;
+	return R >= 1 && R <= OFI_AMD_MAX_NUM_RAILS && (R & (R - 1)) == 0 && c->sched.rr_small_counter < R &&
+	       c->sched.rr_counter < R && c->sched.min_stripe_size != 0 &&
+	       (c->sched.min_stripe_size & (c->sched.min_stripe_size - 1)) == 0 &&
+	       c->pinned_rail_id < (int32_t)R && c->num_rails >= 1 && c->num_rails <= OFI_AMD_MAX_NUM_RAILS &&
+	       c->next_rail_id < c->num_rails;
 }
 
 } // namespace ofi_amd_gin

@@ -10,15 +10,15 @@
 #include <cerrno>
 #include <chrono>
 #include <cstring>
-#include <deque>
 #include <new>
 #include <vector>
 
+#include "gin_derive.hpp"
 #include "gin_rings.hpp"
 
 namespace {
 
-constexpr uint32_t kPiece = 64u << 10; /* long writes are cut so that no wavefront copies more */
+constexpr uint64_t kPiece = 1ull << 31; /* a table entry's length is 32 bits: longer writes take several */
 constexpr uint64_t kSentinel = 0xdeadbeefdeadbeefull; /* NCCL_OFI_GIN_FLUSH_SENTINEL_VAL */
 
 /* One launch pair's worth of copies and signal work, in pinned host memory the GPU reads in place. */
@@ -31,6 +31,7 @@ struct batch_t {
 	uint64_t *done_slot = nullptr;
 	void *d_done_slot = nullptr;
 	uint32_t n_copy = 0, n_work = 0;
+	uint32_t max_len = 0; /* longest entry of the copy table */
 	bool launched = false;
 };
 
@@ -64,20 +65,33 @@ int alloc_batch(batch_t &b, uint32_t cap_copy, uint32_t cap_work)
 	return rc;
 }
 
-/* A completion on its way from the "NIC" to the receiver. */
+/* A completion on its way from the "NIC" to the receiver: a write's immediate data, or the slot
+ * of a metadata message in the side table (one event in seventy is one, so the 32 bytes do not
+ * travel with every event). */
 struct event_t {
 	uint32_t peer;
-	uint32_t is_meta;
 	uint32_t imm;
-	uint64_t meta[4];
+	int32_t meta_slot; /* -1: a write completion */
 };
+struct meta_msg_t {
+	uint64_t word[4];
+};
+
+/* Where the proxy thread's time goes: the time-stamp counter is read around the stages of every
+ * 17th operation (reading it around all of them would be a tenth of the time measured) and
+ * around every launch, and the sums are scaled to the whole run when it ends. */
+struct stage_clock_t {
+	uint64_t pop_derive = 0, tx_post = 0, wire = 0, progress = 0, rx = 0, launch_wait = 0;
+	static uint64_t now() { return __builtin_ia32_rdtsc(); }
+};
+constexpr uint32_t kSampleEvery = 17; /* a prime: no beat with the caller's progress interval */
 
 struct lcg_t {
 	uint64_t s;
-	uint32_t next(uint32_t n)
+	uint32_t next(uint32_t n) /* n < 2^31; multiply-shift instead of a division per event */
 	{
 		s = s * 6364136223846793005ull + 1442695040888963407ull;
-		return (uint32_t)((s >> 33) % n);
+		return (uint32_t)(((s >> 33) * n) >> 31);
 	}
 };
 
@@ -106,16 +120,26 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 	ofi_amd_gin_rx_t *rx = nullptr;
 	ofi_amd_loopfab_t *fab = nullptr;
 	ofi_amd_gin_tx_t *tx = nullptr;
-	std::deque<int32_t> open_ops; /* operations whose posts have not all completed, oldest first */
 	constexpr uint32_t kPool = 1u << 16;
+	/* operations whose posts have not all completed, oldest first: positions into a power-of-two
+	 * array of kPool entries (an open operation holds a pool entry, so there are never more) */
+	std::vector<int32_t> open_ops;
+	uint32_t open_head = 0, open_tail = 0;
 	std::vector<uint32_t> comm_ids;
 	std::vector<event_t> in_flight;
+	std::vector<meta_msg_t> meta_msgs; /* metadata messages in flight, and the free slots among them */
+	std::vector<int32_t> meta_free;
 	std::vector<uint64_t> done;
 	int rc = 0;
 	try {
 		comm_ids.resize(nctx);
+		open_ops.assign(kPool, -1);
 		done.assign(nctx, 0);
 		in_flight.reserve(reorder_window + 8);
+		meta_msgs.resize(reorder_window + 8);
+		for (int32_t k = (int32_t)meta_msgs.size(); k > 0; k--) {
+			meta_free.push_back(k - 1);
+		}
 	} catch (...) {
 		return -ENOMEM;
 	}
@@ -165,15 +189,26 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 	ofi_amd_gin_ack_t acks[64];
 
 	/* copies first, then the signals that were released while they were queued */
-	auto flush = [&]() -> int {
+	stage_clock_t sc;
+	bool sampling = false; /* this operation's stages are being timed */
+	auto flush_inner = [&]() -> int {
 		batch_t &b = batches[cur];
 		if (b.n_copy == 0 && b.n_work == 0) {
 			return 0;
 		}
 		int e = 0;
 		if (b.n_copy) {
-			e = ofi_amd_copy_table(static_cast<const uint64_t *>(b.d_src), static_cast<const uint64_t *>(b.d_dst),
-					       static_cast<const uint32_t *>(b.d_len), b.n_copy, stream);
+			/* one table entry per write, every 8 KiB of it a wavefront of its own; a launch holds
+			 * at most 2^31 - 1 wavefronts, so a table with very long entries goes in parts */
+			const uint64_t per_entry = ((uint64_t)b.max_len + 8191u) / 8192u;
+			const uint64_t most = per_entry ? (0x7fff0000ull / per_entry) : b.n_copy;
+			const uint32_t part = most < 1 ? 1u : (most < b.n_copy ? (uint32_t)most : b.n_copy);
+			for (uint32_t at = 0; at < b.n_copy && e == 0; at += part) {
+				const uint32_t cnt = b.n_copy - at < part ? b.n_copy - at : part;
+				e = ofi_amd_copy_table_pieces(static_cast<const uint64_t *>(b.d_src) + at,
+							      static_cast<const uint64_t *>(b.d_dst) + at,
+							      static_cast<const uint32_t *>(b.d_len) + at, cnt, b.max_len, stream);
+			}
 		}
 		if (e == 0 && b.n_work) {
 			e = ofi_amd_gin_signal_apply(static_cast<const ofi_amd_gin_signal_work_t *>(b.d_work), b.n_work,
@@ -205,18 +240,38 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 			next.launched = false;
 		}
 		next.n_copy = next.n_work = 0;
+		next.max_len = 0;
 		return 0;
 	};
+	/* launches and the wait for the other table pair are timed every time, and taken out of the
+	 * sampled stage they interrupt */
+	uint64_t flush_ticks_in_sample = 0;
+	auto flush = [&]() -> int {
+		const uint64_t f0 = stage_clock_t::now();
+		const int e = flush_inner();
+		const uint64_t dt = stage_clock_t::now() - f0;
+		sc.launch_wait += dt;
+		if (sampling) {
+			flush_ticks_in_sample += dt;
+		}
+		return e;
+	};
 
-	/* hands one completion to the receiver and collects what that releases */
+	/* hands one completion to the receiver */
 	auto deliver = [&](const event_t &ev) -> int {
-		int e = ev.is_meta ? ofi_amd_gin_rx_metadata(rx, ev.peer, ev.meta)
-				   : ofi_amd_gin_rx_write_completion(rx, ev.peer, ev.imm);
-		if (e != 0) {
+		if (ev.meta_slot >= 0) {
+			const int e = ofi_amd_gin_rx_metadata(rx, ev.peer, meta_msgs[(size_t)ev.meta_slot].word);
+			meta_free.push_back(ev.meta_slot);
 			return e;
 		}
+		return ofi_amd_gin_rx_write_completion(rx, ev.peer, ev.imm);
+	};
+	/* collects what the completions delivered so far have released: the target sends its ACKs
+	 * back through the same endpoint (send_ack, :267-315), the signal work joins the batch (its
+	 * payloads' copies entered the table when their writes left the fabric, so it is behind them) */
+	auto collect = [&]() -> int {
+		int e = 0;
 		for (;;) {
-			/* the target sends its ACKs back through the same endpoint (send_ack, :267-315) */
 			const uint32_t n = ofi_amd_gin_rx_take_acks(rx, acks, 64);
 			for (uint32_t i = 0; i < n && e == 0; i++) {
 				e = ofi_amd_gin_tx_send_ack(tx, acks[i].peer, acks[i].msg);
@@ -243,7 +298,11 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 		return 0;
 	};
 
-	auto deliver_some = [&](uint32_t keep) -> int {
+	uint32_t uncollected = 0; /* completions delivered since the receiver's ACKs and signal work were fetched */
+	auto deliver_some_inner = [&](uint32_t keep) -> int {
+		if (in_flight.size() <= keep) {
+			return 0;
+		}
 		while (in_flight.size() > keep) {
 			const uint32_t k = rng.next((uint32_t)in_flight.size());
 			const event_t ev = in_flight[k];
@@ -253,8 +312,26 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 			if (e != 0) {
 				return e;
 			}
+			uncollected++;
+		}
+		/* what the receiver has released is fetched every 16 completions, and whenever the
+		 * caller waits for everything in flight to arrive */
+		if (uncollected >= 16 || keep == 0) {
+			uncollected = 0;
+			return collect();
 		}
 		return 0;
+	};
+
+	auto deliver_some = [&](uint32_t keep) -> int {
+		if (!sampling) {
+			return deliver_some_inner(keep);
+		}
+		const uint64_t r0 = stage_clock_t::now();
+		const uint64_t fl0 = flush_ticks_in_sample;
+		const int e = deliver_some_inner(keep);
+		sc.rx += stage_clock_t::now() - r0 - (flush_ticks_in_sample - fl0);
+		return e;
 	};
 
 	/* The wire and the initiator's progress: what the fabric has transmitted is executed (a write
@@ -264,13 +341,13 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 	 * operations. */
 	ofi_amd_gin_post_t wire_posts[64];
 	auto pump = [&]() -> int {
+		const uint64_t p0 = sampling ? stage_clock_t::now() : 0;
+		const uint64_t fl0 = flush_ticks_in_sample;
 		for (;;) {
 			const uint32_t n = ofi_amd_loopfab_take_transmitted(fab, wire_posts, 64);
 			for (uint32_t i = 0; i < n; i++) {
 				const ofi_amd_gin_post_t &p = wire_posts[i];
-				event_t ev;
-				std::memset(&ev, 0, sizeof(ev));
-				ev.peer = p.peer;
+				event_t ev{p.peer, 0, -1};
 				if (p.kind == OFI_AMD_GIN_POST_WRITE || p.kind == OFI_AMD_GIN_POST_READ) {
 					/* a read is the same copy the other way, and the target hears nothing of it */
 					const bool read = p.kind == OFI_AMD_GIN_POST_READ;
@@ -296,6 +373,7 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 						b.src[b.n_copy] = (read ? p.dest : p.src) + off;
 						b.dst[b.n_copy] = (read ? landing : p.dest) + off;
 						b.len[b.n_copy] = (uint32_t)len;
+						b.max_len = (uint32_t)len > b.max_len ? (uint32_t)len : b.max_len;
 						b.n_copy++;
 					}
 					if (read && p.peer == OFI_AMD_GIN_PEER_SELF) {
@@ -310,8 +388,13 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 						in_flight.push_back(ev);
 					}
 				} else if (p.kind == OFI_AMD_GIN_POST_META) {
-					ev.is_meta = 1;
-					std::memcpy(ev.meta, p.msg, sizeof(ev.meta));
+					if (meta_free.empty()) { /* more in flight than the window: grow the table */
+						meta_free.push_back((int32_t)meta_msgs.size());
+						meta_msgs.emplace_back();
+					}
+					ev.meta_slot = meta_free.back();
+					meta_free.pop_back();
+					std::memcpy(meta_msgs[(size_t)ev.meta_slot].word, p.msg, sizeof(p.msg));
 					in_flight.push_back(ev);
 				} else {
 					/* gin_ack_msg_t: rx_consumed in bits 12..25 (handle_ack_completion, :1843-1869) */
@@ -323,19 +406,25 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 				break;
 			}
 		}
+		const uint64_t p1 = sampling ? stage_clock_t::now() : 0;
 		int e = ofi_amd_gin_tx_progress(tx);
-		while (e == 0 && !open_ops.empty()) {
+		while (e == 0 && open_head != open_tail) {
 			int done = 0;
-			e = ofi_amd_gin_tx_test(tx, open_ops.front(), &done);
+			e = ofi_amd_gin_tx_test(tx, open_ops[open_head & (kPool - 1)], &done);
 			if (e != 0 || !done) {
 				break;
 			}
-			open_ops.pop_front();
+			open_head++;
+		}
+		if (sampling) {
+			sc.wire += p1 - p0 - (flush_ticks_in_sample - fl0);
+			sc.progress += stage_clock_t::now() - p1;
 		}
 		return e;
 	};
 
 	const auto t0 = clock::now();
+	const uint64_t tsc0 = stage_clock_t::now();
 	auto last_progress = t0;
 	uint64_t remaining = (uint64_t)nctx * ops_per_context;
 	uint32_t idle = 0;
@@ -344,50 +433,79 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 	while (remaining > 0 && rc == 0) {
 		bool progressed = false;
 		for (uint32_t c = 0; c < nctx && rc == 0; c++) {
-			for (uint32_t burst = 0; burst < 256 && done[c] < ops_per_context; burst++) {
-				ofi_amd_gin_desc_t d;
-				if (ofi_amd_gin_ring_pop(r, c, &d) != 1) {
+			/* constant over the burst: the derivation keeps the counters below the rail count */
+			const bool fast = ofi_amd_gin::derive_fast_path(&comms[c]);
+			auto derive_one = [&](const ofi_amd_gin_desc_t &d, ofi_amd_gin_wire_t *wire) -> int {
+				if (d.kind == OFI_AMD_GIN_KIND_GET) {
+					return ofi_amd_gin_iget(&comms[c], mrs, n_mrs, &d, wire);
+				}
+				return fast ? ofi_amd_gin::derive<true>(&comms[c], mrs, n_mrs, &d, wire)
+					    : ofi_amd_gin_iput_signal(&comms[c], mrs, n_mrs, &d, wire);
+			};
+			/* a burst is read in place and its slots are handed back together afterwards, in
+			 * position order (nccl_ofi_mpsc_ring::pop, include/nccl_ofi_mpsc_ring.h:124-144, for a
+			 * run of positions): no copy of the record, no store per operation into a line
+			 * the producers poll */
+			const uint32_t cap = r->capacity, mask = cap - 1;
+			uint32_t *ring_seq = r->sequences + (size_t)c * cap;
+			const ofi_amd_gin_desc_t *ring_rec = r->records + (size_t)c * cap;
+			const uint32_t start = r->dequeue_pos[c];
+			const uint64_t want = ops_per_context - done[c];
+			const uint32_t most = cap / 2 < 256 ? cap / 2 : 256;
+			const uint32_t limit = want < most ? (uint32_t)want : most;
+			uint32_t pos = start;
+			for (; pos - start < limit; pos++) {
+				sampling = (st.descriptors % kSampleEvery) == 0;
+				const uint64_t s0 = sampling ? stage_clock_t::now() : 0;
+				if (__atomic_load_n(&ring_seq[pos & mask], __ATOMIC_ACQUIRE) != pos + 1) {
 					break;
 				}
+				const ofi_amd_gin_desc_t &d = ring_rec[pos & mask];
 				ofi_amd_gin_wire_t wire;
-				rc = ofi_amd_gin_derive(&comms[c], mrs, n_mrs, &d, &wire);
-				const auto w0 = clock::now();
+				rc = derive_one(d, &wire);
+				if (sampling) {
+					sc.pop_derive += stage_clock_t::now() - s0;
+				}
+				const auto w0 = rc == -EAGAIN ? clock::now() : clock::time_point();
 				while (rc == -EAGAIN) {
 					/* window closed (await_tx_window, :518-537, progresses until it opens): let
 					 * everything in flight arrive, which brings the ACKs */
 					rc = pump();
 					if (rc == 0) rc = deliver_some(0);
 					if (rc == 0) rc = pump();
-					if (rc == 0) rc = ofi_amd_gin_derive(&comms[c], mrs, n_mrs, &d, &wire);
+					if (rc == 0) rc = derive_one(d, &wire);
 					if (rc == -EAGAIN &&
 					    std::chrono::duration_cast<std::chrono::milliseconds>(clock::now() - w0).count() >
 						    (long long)timeout_ms) {
 						rc = -ETIMEDOUT;
 					}
 				}
-				/* room in the request pool for this operation and the ACKs it may trigger */
-				while (rc == 0) {
-					(void)ofi_amd_gin_tx_stats(tx, &ts);
-					if (ts.requests + 64 <= kPool) {
-						break;
+				/* room in the request pool for this operation and the ACKs it may trigger: an
+				 * operation takes at most 6 entries and an ACK one, so looking every 1,024
+				 * operations with 16,384 entries to spare is enough */
+				if ((st.descriptors & 1023u) == 0) {
+					while (rc == 0) {
+						(void)ofi_amd_gin_tx_stats(tx, &ts);
+						if (ts.requests + 16384 <= kPool) {
+							break;
+						}
+						rc = pump();
+						if (rc == 0) rc = deliver_some(0);
 					}
-					rc = pump();
-					if (rc == 0) rc = deliver_some(0);
 				}
 				if (rc != 0) {
 					break;
 				}
 				int32_t req = -1;
+				const uint64_t s1 = sampling ? stage_clock_t::now() : 0;
 				rc = d.kind == OFI_AMD_GIN_KIND_GET ? ofi_amd_gin_tx_iget(tx, c, &wire, &req)
 								   : ofi_amd_gin_tx_iput_signal(tx, c, &wire, &req);
 				if (rc != 0) {
 					break;
 				}
-				try {
-					open_ops.push_back(req);
-				} catch (...) {
-					rc = -ENOMEM;
-					break;
+				open_ops[open_tail++ & (kPool - 1)] = req;
+				if (sampling) {
+					sc.tx_post += stage_clock_t::now() - s1;
 				}
 				st.signals += wire.has_meta;
 				/* NCCL's proxy submits what it has and then calls ginProgress: a progress call
@@ -404,7 +522,13 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 				remaining--;
 				st.descriptors++;
 				progressed = true;
+				sampling = false;
 			}
+			sampling = false;
+			for (uint32_t p = start; p != pos; p++) {
+				__atomic_store_n(&ring_seq[p & mask], p + cap, __ATOMIC_RELEASE);
+			}
+			r->dequeue_pos[c] = pos;
 		}
 		if (progressed) {
 			idle = 0;
@@ -430,7 +554,7 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 			break;
 		}
 		(void)ofi_amd_gin_tx_stats(tx, &ts);
-		if (open_ops.empty() && in_flight.empty() && ts.requests == 0) {
+		if (open_head == open_tail && in_flight.empty() && ts.requests == 0) {
 			break;
 		}
 		if (std::chrono::duration_cast<std::chrono::milliseconds>(clock::now() - d0).count() >
@@ -483,6 +607,17 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 		rc = sync_rc;
 	}
 	st.seconds = std::chrono::duration<double>(clock::now() - t0).count();
+	{
+		/* ticks -> nanoseconds from this run's own two clocks; sampled stages scaled up */
+		const double ns_per_tick = st.seconds * 1e9 / (double)(stage_clock_t::now() - tsc0);
+		const double k = ns_per_tick * kSampleEvery;
+		st.ns_pop_derive = (uint64_t)(sc.pop_derive * k);
+		st.ns_tx_post = (uint64_t)(sc.tx_post * k);
+		st.ns_wire = (uint64_t)(sc.wire * k);
+		st.ns_progress = (uint64_t)(sc.progress * k);
+		st.ns_rx = (uint64_t)(sc.rx * k);
+		st.ns_launch_wait = (uint64_t)(sc.launch_wait * ns_per_tick);
+	}
 	if (stats) {
 		*stats = st;
 	}

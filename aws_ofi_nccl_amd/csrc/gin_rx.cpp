@@ -21,16 +21,18 @@ namespace {
 constexpr uint32_t kSeqMask = (1u << 13) - 1;    /* GIN_IMM_SEQ_MASK */
 constexpr uint32_t kCursorMask = (1u << 14) - 1; /* GIN_RX_CONSUMED_MASK */
 
-struct rx_req {
-	bool present = false;
-	bool metadata_received = false;
-	bool is_ack_requested = false;
-	uint32_t num_seg_completions = 0;
-	uint32_t total_segments = 0;
-	uint32_t meta_seq = 0;
+struct rx_req { /* 32 bytes: two to a cache line, walked in sequence order */
+	uint8_t present = 0;
+	uint8_t metadata_received = 0;
+	uint8_t is_ack_requested = 0;
+	uint8_t num_seg_completions = 0; /* at most 5: four writes and the metadata message */
+	uint8_t total_segments = 0;
+	uint8_t pad = 0;
+	uint16_t meta_seq = 0;
 	uint64_t base = 0, offset = 0, value = 0;
 	bool complete() const { return present && num_seg_completions == total_segments; }
 };
+static_assert(sizeof(rx_req) == 32, "rx_req");
 
 struct rx_peer {
 	uint32_t comm_id = 0;
@@ -62,7 +64,7 @@ void retire(ofi_amd_gin_rx *rx, uint32_t peer)
 		}
 		if (!req->metadata_received) {
 			/* a put without signal: consume the sequence number, nothing to deliver */
-			ack_requested |= req->is_ack_requested;
+			ack_requested |= req->is_ack_requested != 0;
 			pc.rx_consumed = (pc.rx_consumed + 1) & kCursorMask;
 			pc.next_delivered_seq = (pc.next_delivered_seq + 1) & kSeqMask;
 			*req = rx_req();
@@ -79,7 +81,7 @@ void retire(ofi_amd_gin_rx *rx, uint32_t peer)
 		for (;;) {
 			folded.value += cur->value;
 			folded.run_len++;
-			ack_requested |= cur->is_ack_requested;
+			ack_requested |= cur->is_ack_requested != 0;
 			pc.rx_consumed = (pc.rx_consumed + 1) & kCursorMask;
 			pc.next_delivered_seq = (pc.next_delivered_seq + 1) & kSeqMask;
 
@@ -167,16 +169,16 @@ int ofi_amd_gin_rx_write_completion(ofi_amd_gin_rx_t *rx, uint32_t peer, uint32_
 		rx_req &req = rx->peers[peer].reqs[seq];
 		if (!req.present) {
 			req = rx_req();
-			req.present = true;
+			req.present = 1;
 			req.num_seg_completions = 1;
-			req.total_segments = total;
+			req.total_segments = (uint8_t)total;
 			req.is_ack_requested = ack;
 		} else {
-			req.is_ack_requested |= ack;
+			req.is_ack_requested |= (uint8_t)ack;
 			req.num_seg_completions += 1;
 		}
 		if (req.num_seg_completions == req.total_segments) {
-			req.meta_seq = seq;
+			req.meta_seq = (uint16_t)seq;
 			retire(rx, peer);
 		}
 	} catch (...) {
@@ -198,16 +200,16 @@ int ofi_amd_gin_rx_metadata(ofi_amd_gin_rx_t *rx, uint32_t peer, const uint64_t 
 		rx_req &req = rx->peers[peer].reqs[seq];
 		if (!req.present) {
 			req = rx_req();
-			req.present = true;
+			req.present = 1;
 			req.num_seg_completions = 1;
-			req.total_segments = total;
+			req.total_segments = (uint8_t)total;
 			req.is_ack_requested = ack;
 		} else {
 			req.num_seg_completions += 1;
-			req.is_ack_requested |= ack;
+			req.is_ack_requested |= (uint8_t)ack;
 		}
-		req.metadata_received = true;
-		req.meta_seq = seq;
+		req.metadata_received = 1;
+		req.meta_seq = (uint16_t)seq;
 		req.base = meta[1];
 		req.offset = meta[2];
 		req.value = meta[3];

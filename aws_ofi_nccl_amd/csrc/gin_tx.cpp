@@ -54,6 +54,10 @@ struct ofi_amd_gin_tx {
 		}
 		*idx = free_list.back();
 		free_list.pop_back();
+		request_t &r = pool[*idx]; /* what a user does not set itself starts clean; `post` is always set whole */
+		r.slot = 0;
+		r.parent = kNoParent;
+		r.pending_mask = 0;
 		st.requests++;
 		if (st.requests > st.requests_max) {
 			st.requests_max = st.requests;
@@ -63,7 +67,7 @@ struct ofi_amd_gin_tx {
 
 	void release(uint32_t idx)
 	{
-		pool[idx] = request_t();
+		pool[idx].use = kFree; /* the rest is rewritten by whoever takes the entry next */
 		free_list.push_back(idx);
 		st.requests--;
 	}
@@ -436,16 +440,40 @@ int ofi_amd_gin_tx_stats(const ofi_amd_gin_tx_t *tx, ofi_amd_gin_tx_stats_t *out
 
 /* ---------------------------------------------------------------- the in-process fabric ---- */
 
+/* Fixed-size queue over a power-of-two array: positions only grow, the index is the position
+ * masked. */
+template <typename T>
+struct ring_t {
+	std::vector<T> slot;
+	uint32_t mask = 0, head = 0, tail = 0; /* head: oldest entry, tail: next free position */
+	void reset(uint32_t capacity)
+	{
+		uint32_t n = 1;
+		while (n < capacity) {
+			n <<= 1;
+		}
+		slot.assign(n, T());
+		mask = n - 1;
+		head = tail = 0;
+	}
+	uint32_t size() const { return tail - head; }
+	bool empty() const { return tail == head; }
+	T &at(uint32_t k) { return slot[(head + k) & mask]; } /* k-th oldest */
+	void push(const T &v) { slot[tail++ & mask] = v; }
+	void pop() { head++; }
+};
+
 struct ofi_amd_loopfab {
 	struct rail_t {
-		std::deque<ofi_amd_gin_post_t> sq; /* posted, completion not read yet */
-		uint32_t transmitted = 0;          /* of which the doorbell has rung for */
-		uint32_t taken = 0;                /* of which handed to the wire */
-		uint32_t readable = 0;             /* of which the completion can be read */
+		ring_t<ofi_amd_gin_post_t> sq; /* posted, completion not read yet: at most sq_depth */
+		uint32_t transmitted = 0;      /* of which the doorbell has rung for */
+		uint32_t taken = 0;            /* of which handed to the wire */
+		uint32_t readable = 0;         /* of which the completion can be read */
 	};
 	uint32_t num_rails = 0, sq_depth = 0;
 	std::vector<rail_t> rails;
-	std::deque<uint32_t> rung; /* rails in the order their doorbells rang, one entry per transmitted post */
+	ring_t<uint8_t> rung; /* rails in the order their doorbells rang, one entry per transmitted post:
+			       * at most num_rails * sq_depth */
 
 	static int post(void *self, const ofi_amd_gin_post_t *p)
 	{
@@ -457,17 +485,13 @@ struct ofi_amd_loopfab {
 		if (r.sq.size() >= f->sq_depth) {
 			return -EAGAIN;
 		}
-		try {
-			r.sq.push_back(*p);
-			/* a provider never leaves a full queue unsubmitted */
-			if (!p->more || r.sq.size() >= f->sq_depth) {
-				while (r.transmitted < r.sq.size()) {
-					f->rung.push_back(p->rail);
-					r.transmitted++;
-				}
+		r.sq.push(*p);
+		/* a provider never leaves a full queue unsubmitted */
+		if (!p->more || r.sq.size() >= f->sq_depth) {
+			while (r.transmitted < r.sq.size()) {
+				f->rung.push((uint8_t)p->rail);
+				r.transmitted++;
 			}
-		} catch (...) {
-			return -ENOMEM;
 		}
 		return 0;
 	}
@@ -481,8 +505,8 @@ struct ofi_amd_loopfab {
 		rail_t &r = f->rails[rail];
 		uint32_t n = 0;
 		while (n < max && r.readable > 0) {
-			contexts[n++] = r.sq.front().context;
-			r.sq.pop_front(); /* the send-queue entry is free again */
+			contexts[n++] = r.sq.at(0).context;
+			r.sq.pop(); /* the send-queue entry is free again */
 			r.readable--;
 			r.taken--;
 			r.transmitted--;
@@ -502,8 +526,16 @@ int ofi_amd_loopfab_create(uint32_t num_rails, uint32_t sq_depth, ofi_amd_loopfa
 	if (!f) {
 		return -ENOMEM;
 	}
+	if (sq_depth > (1u << 20)) {
+		delete f;
+		return -EINVAL;
+	}
 	try {
 		f->rails.resize(num_rails);
+		for (auto &r : f->rails) {
+			r.sq.reset(sq_depth);
+		}
+		f->rung.reset(num_rails * sq_depth);
 	} catch (...) {
 		delete f;
 		return -ENOMEM;
@@ -539,16 +571,12 @@ int ofi_amd_loopfab_ring_all(ofi_amd_loopfab_t *f)
 	if (!f) {
 		return -EINVAL;
 	}
-	try {
-		for (uint32_t rail = 0; rail < f->num_rails; rail++) {
-			ofi_amd_loopfab::rail_t &r = f->rails[rail];
-			while (r.transmitted < r.sq.size()) {
-				f->rung.push_back(rail);
-				r.transmitted++;
-			}
+	for (uint32_t rail = 0; rail < f->num_rails; rail++) {
+		ofi_amd_loopfab::rail_t &r = f->rails[rail];
+		while (r.transmitted < r.sq.size()) {
+			f->rung.push((uint8_t)rail);
+			r.transmitted++;
 		}
-	} catch (...) {
-		return -ENOMEM;
 	}
 	return 0;
 }
@@ -560,9 +588,9 @@ uint32_t ofi_amd_loopfab_take_transmitted(ofi_amd_loopfab_t *f, ofi_amd_gin_post
 	}
 	uint32_t n = 0;
 	while (n < cap && !f->rung.empty()) {
-		ofi_amd_loopfab::rail_t &r = f->rails[f->rung.front()];
-		f->rung.pop_front();
-		out[n++] = r.sq[r.taken];
+		ofi_amd_loopfab::rail_t &r = f->rails[f->rung.at(0)];
+		f->rung.pop();
+		out[n++] = r.sq.at(r.taken);
 		r.taken++;
 		r.readable++; /* executed on the spot by the caller: the completion is there */
 	}

@@ -99,6 +99,13 @@ int ofi_amd_gin_iget(ofi_amd_gin_comm_t *c, const ofi_amd_gin_mr_t *mrs, uint32_
 	const uint64_t local = mrs[d->dst_mr].local_base + d->dst_off;
 	const uint64_t from = remote.remote_address_offset + d->src_off;
 	for (int k = 0; k < n; k++) {
+		if (xfers[k].rail_id >= OFI_AMD_MAX_NUM_RAILS) {
+			/* a round-robin counter edited beyond the rail count: an error, not a key index */
+			std::memset(out, 0, sizeof(*out));
+			return -EINVAL;
+		}
+	}
+	for (int k = 0; k < n; k++) {
 		ofi_amd_gin_write_t &r = out->writes[k];
 		r.rail = xfers[k].rail_id;
 		r.src = local + xfers[k].offset;

@@ -575,7 +575,7 @@ def bench_gin(lib, oracle, torch, np, args):
     t0 = time.perf_counter()
     m.check(lib.ofi_amd_gin_produce_seeded(rings, SEED, l_ops, 1, 64, 1, 1, 0, _gpu.stream()), "produce")
     rc = lib.ofi_amd_gin_loopback_run(rings, l_ops, ctypes.cast(comms, ctypes.c_void_p),
-                                      ctypes.cast(mrs, ctypes.c_void_p), 3, regions, 1, 32, 4096, 0, 1, 20000,
+                                      ctypes.cast(mrs, ctypes.c_void_p), 3, regions, 1, 32, 16384, 0, 1, 20000,
                                       ctypes.c_void_p(side.cuda_stream), ctypes.byref(lstats))
     torch.cuda.synchronize()
     secs = time.perf_counter() - t0
@@ -586,7 +586,10 @@ def bench_gin(lib, oracle, torch, np, args):
                        "payload_gbs": lstats.bytes / secs / 1e9, "payload_bytes": lstats.bytes,
                        "rdma_writes": lstats.writes, "copy_launches": lstats.launches, "acks": lstats.acks,
                        "signals": lstats.signals,
-                       "signals_counted_in_hbm_ok": signals_seen == l_ctx * (l_ops // 64), "proxy_threads": 1}
+                       "signals_counted_in_hbm_ok": signals_seen == l_ctx * (l_ops // 64), "proxy_threads": 1,
+                       "ns_per_put": secs / lstats.descriptors * 1e9,
+                       "ns_per_put_by_stage": {k: getattr(lstats, "ns_" + k) / lstats.descriptors for k in (
+                           "pop_derive", "tx_post", "wire", "progress", "rx", "launch_wait")}}
     lib.ofi_amd_gin_rings_destroy(rings)
     del d_srcbuf, d_dstbuf
     torch.cuda.empty_cache()

@@ -207,7 +207,8 @@ int ofi_amd_copy_table(const uint64_t *d_src_addr, const uint64_t *d_dst_addr, c
  * instead of by one wavefront each, and the caller need not cut them.  max_len >= every
  * d_len[i]; the launch has n * ceil(max_len / 8192) wavefronts (-E2BIG beyond 2^31 - 1: split
  * the table), those past the end of their entry leave at once.  An entry longer than max_len
- * is copied up to that bound and reported through ofi_amd_async_error_fetch (bit 3).
+ * is copied up to exactly max_len bytes (nothing of it when max_len is 0) and reported through
+ * ofi_amd_async_error_fetch (bit 3).
  */
 int ofi_amd_copy_table_pieces(const uint64_t *d_src_addr, const uint64_t *d_dst_addr, const uint32_t *d_len,
 			      uint32_t n, uint32_t max_len, void *stream);
@@ -673,7 +674,7 @@ int ofi_amd_gin_signal_apply(const ofi_amd_gin_signal_work_t *d_work, uint32_t n
  *   3. executes what the fabric transmits: each RDMA write as a (source, destination, length)
  *      copy -- source mrs[src_mr].local_base + src_off, destination the write's `dest` (give
  *      the destination MR's remote_address_offset the device address of the target buffer) --
- *      long writes cut into 64 KiB pieces; the write completions and the metadata message go
+ *      one table entry per write; the write completions and the metadata message go
  *      to a receiver (ofi_amd_gin_rx_*, one peer per context), up to reorder_window events
  *      out of order; each RDMA read of a get as the copy the other way -- from the read's
  *      `dest` (the remote MR's remote_address_offset + offset) into the local buffer -- of
@@ -682,7 +683,7 @@ int ofi_amd_gin_signal_apply(const ofi_amd_gin_signal_work_t *d_work, uint32_t n
  *   4. sends the receiver's ACKs back through the same engine and fabric; an ACK that arrives
  *      moves the sender's window (ofi_amd_gin_apply_ack),
  * and every batch_writes queued copies (and at the end) launches, in this order on `stream`,
- * ofi_amd_copy_table for the copies and ofi_amd_gin_signal_apply for the signals the
+ * ofi_amd_copy_table_pieces for the copies and ofi_amd_gin_signal_apply for the signals the
  * receiver has released: a signal is applied after the payloads it covers.  `stream` must
  * not be the stream the producing kernel runs on (that kernel waits for this call to drain
  * its rings; work queued behind it would never start).  What the
@@ -692,7 +693,7 @@ int ofi_amd_gin_signal_apply(const ofi_amd_gin_signal_work_t *d_work, uint32_t n
 typedef struct {
 	uint64_t descriptors;
 	uint64_t writes;          /* RDMA writes derived */
-	uint64_t copy_entries;    /* after cutting long writes */
+	uint64_t copy_entries;    /* copy-table entries: one per write and per read */
 	uint64_t bytes;           /* payload bytes moved */
 	uint64_t signals;         /* put-signal operations */
 	uint64_t work_items;      /* folded signal deliveries applied */
@@ -706,6 +707,14 @@ typedef struct {
 	uint32_t requests_max;    /* most request-pool entries in use */
 	uint64_t reads;           /* RDMA reads of gets */
 	uint64_t flush_reads;     /* reads of the flush that fences them (one per rail), 0 without gets */
+	/* where the calling thread's time went, nanoseconds over the whole run (the first five from
+	 * time stamps around the stages of every 16th operation, scaled up) */
+	uint64_t ns_pop_derive;   /* ring pop + ofi_amd_gin_derive */
+	uint64_t ns_tx_post;      /* ofi_amd_gin_tx_iput_signal / _iget: pool entries, posts into the fabric */
+	uint64_t ns_wire;         /* taking transmitted posts off the fabric, copy-table entries, events */
+	uint64_t ns_progress;     /* ofi_amd_gin_tx_progress (CQ drain, retries) + test of the oldest operations */
+	uint64_t ns_rx;           /* receiver: completions, metadata, ACKs back into the engine, signal work */
+	uint64_t ns_launch_wait;  /* copy / signal launches and the wait for the other table pair's sentinel */
 } ofi_amd_gin_loopback_stats_t;
 
 int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *rings, uint64_t ops_per_context,

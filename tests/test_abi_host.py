@@ -127,6 +127,63 @@ def test_proxy_derivation_matches_oracle(lib, oracle, ack_model, agg_mask, signa
         assert lib.ofi_amd_gin_iput_signal(ctypes.byref(pc), pmrs, 3, ctypes.byref(pd), ctypes.byref(pw)) == 0
 
 
+def test_proxy_derivation_survives_a_communicator_edited_by_hand(lib):
+    """ofi_amd_gin_comm_t is the caller's struct.  Fields that comm_init and the derivation never
+    produce -- a rail count outside 1..4, a zero stripe size, a pin or a rail cursor beyond the rail
+    count, round-robin counters beyond it -- must end in an error or in rails inside the table,
+    never in a read past the stripe-count or key tables (the build under AddressSanitizer in
+    tests/test_host_sanitizers.py runs the same code)."""
+    mrs = _oracle.default_mrs(m.GinMr)
+    base = m.GinComm()
+    assert lib.ofi_amd_gin_comm_init(ctypes.byref(base), 3, 4, 131072, 64, 1) == 0
+    state = bytes(base)
+    d_small = m.GinDesc(0, 0, 4096, 8, 0, 1, 0, 0, 0, 0, 1, 2, 1)
+    d_big = m.GinDesc(0, 0, 1 << 20, 8, 0, 1, 0, 0, 0, 0, 1, 2, 1)
+    d_signal_only = m.GinDesc(0, 0, 0, 8, 0, 1, 1, 0, 0, 0, 1, 2, 2)
+    w = m.GinWire()
+
+    def edited(**fields):
+        c = m.GinComm.from_buffer_copy(state)
+        for k, v in fields.items():
+            if k.startswith("sched_"):
+                setattr(c.sched, k[6:], v)
+            else:
+                setattr(c, k, v)
+        return c
+
+    for d in (d_small, d_big):
+        for fields in ({"sched_num_rails": 8}, {"sched_num_rails": 16}, {"sched_num_rails": 0},
+                       {"sched_num_rails": -1}, {"sched_min_stripe_size": 0}):
+            c = edited(**fields)
+            assert lib.ofi_amd_gin_iput_signal(ctypes.byref(c), mrs, 3, ctypes.byref(d), ctypes.byref(w)) == \
+                -errno.ENOMEM, fields                       # no schedule, as the reference's nullptr schedule
+        for fields in ({"pinned_rail_id": 4}, {"pinned_rail_id": 1 << 20}, {"num_rails": 0}, {"num_rails": 9},
+                       {"next_rail_id": 4}):
+            c = edited(**fields)
+            assert lib.ofi_amd_gin_iput_signal(ctypes.byref(c), mrs, 3, ctypes.byref(d), ctypes.byref(w)) == \
+                -errno.EINVAL, fields
+            assert bytes(w) == bytes(224)
+        # counters beyond the rail count are reduced, not used as indices
+        for fields in ({"sched_rr_small_counter": 4}, {"sched_rr_counter": 7}, {"sched_rr_counter": 0xFFFFFFFF},
+                       {"sched_rr_small_counter": 1 << 30, "sched_rr_counter": 1 << 31}):
+            c = edited(**fields)
+            assert lib.ofi_amd_gin_iput_signal(ctypes.byref(c), mrs, 3, ctypes.byref(d), ctypes.byref(w)) == 0, fields
+            assert 1 <= w.num_writes <= 4 and all(w.writes[k].rail < 4 for k in range(w.num_writes))
+            assert c.sched.rr_small_counter < 4 and c.sched.rr_counter < 4
+    for fields in ({"num_rails": 0}, {"next_rail_id": 9}, {"pinned_rail_id": 5}):
+        c = edited(**fields)
+        assert lib.ofi_amd_gin_iput_signal(ctypes.byref(c), mrs, 3, ctypes.byref(d_signal_only),
+                                           ctypes.byref(w)) == -errno.EINVAL, fields
+    # three rails (the general path from the start): same answers
+    assert lib.ofi_amd_gin_comm_init(ctypes.byref(base), 3, 3, 131072, 64, 1) == 0
+    state = bytes(base)
+    c = edited(sched_rr_counter=5, sched_rr_small_counter=3)
+    assert lib.ofi_amd_gin_iput_signal(ctypes.byref(c), mrs, 3, ctypes.byref(d_big), ctypes.byref(w)) == 0
+    assert all(w.writes[k].rail < 3 for k in range(w.num_writes))
+    c = edited(pinned_rail_id=3)
+    assert lib.ofi_amd_gin_iput_signal(ctypes.byref(c), mrs, 3, ctypes.byref(d_big), ctypes.byref(w)) == -errno.EINVAL
+
+
 def test_proxy_rejects_bad_arguments(lib):
     c = m.GinComm()
     assert lib.ofi_amd_gin_comm_init(ctypes.byref(c), 1024, 4, 131072, 64, 1) == -errno.EINVAL

@@ -271,18 +271,29 @@ def test_copy_table_in_pieces_matches_a_host_replay(lib, gpu):
         _gpu.sync()
         assert np.array_equal(d_dst.cpu().numpy(), want), max_len
         assert _gpu.fetch_async_errors(lib) == 0
-    # a stated maximum of 20,000 bytes is three pieces: longer entries stop at 24,576 bytes, bit 3 is set
+    # a stated maximum that is not a multiple of the 8 KiB piece: longer entries stop at exactly that
+    # many bytes (also those that would still fit the last piece) and bit 3 is set; 0 copies nothing
+    for max_len in (20000, 8192, 100, 0):
+        d_dst = torch.full((total,), 0x77, dtype=torch.uint8, device="cuda")
+        a_dst = _gpu.to_dev(dst_off + np.uint64(d_dst.data_ptr()))
+        assert lib.ofi_amd_copy_table_pieces(a_src.data_ptr(), a_dst.data_ptr(), d_len.data_ptr(), n, max_len,
+                                             _gpu.stream()) == 0
+        _gpu.sync()
+        cut = np.full(total, 0x77, dtype=np.uint8)
+        for s, d, l in zip(src_off, dst_off, lens):
+            l = min(int(l), max_len)
+            cut[int(d):int(d) + l] = src[int(s):int(s) + l]
+        assert np.array_equal(d_dst.cpu().numpy(), cut), max_len
+        assert _gpu.fetch_async_errors(lib) == 8
+    # every entry within the bound although longer than the bound rounded down to pieces: no report
+    short = np.minimum(lens, 20000).astype(np.uint32)
+    d_short = _gpu.to_dev(short)
     d_dst = torch.full((total,), 0x77, dtype=torch.uint8, device="cuda")
     a_dst = _gpu.to_dev(dst_off + np.uint64(d_dst.data_ptr()))
-    assert lib.ofi_amd_copy_table_pieces(a_src.data_ptr(), a_dst.data_ptr(), d_len.data_ptr(), n, 20000,
+    assert lib.ofi_amd_copy_table_pieces(a_src.data_ptr(), a_dst.data_ptr(), d_short.data_ptr(), n, 20000,
                                          _gpu.stream()) == 0
     _gpu.sync()
-    cut = np.full(total, 0x77, dtype=np.uint8)
-    for s, d, l in zip(src_off, dst_off, lens):
-        l = min(int(l), 24576)
-        cut[int(d):int(d) + l] = src[int(s):int(s) + l]
-    assert np.array_equal(d_dst.cpu().numpy(), cut)
-    assert _gpu.fetch_async_errors(lib) == 8
+    assert _gpu.fetch_async_errors(lib) == 0
     assert lib.ofi_amd_copy_table_pieces(None, a_dst.data_ptr(), d_len.data_ptr(), 1, 64, _gpu.stream()) == -22
     assert lib.ofi_amd_copy_table_pieces(a_src.data_ptr(), a_dst.data_ptr(), d_len.data_ptr(), 0, 64, _gpu.stream()) == 0
     assert lib.ofi_amd_copy_table_pieces(a_src.data_ptr(), a_dst.data_ptr(), d_len.data_ptr(), 1 << 20, 0xFFFFFFFF,
