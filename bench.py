@@ -567,30 +567,44 @@ def bench_gin(lib, oracle, torch, np, args):
     for c in range(l_ctx):
         lib.ofi_amd_gin_comm_init(ctypes.byref(comms[c]), c, 4, 131072, 64, 0)
     regions = (m.GinSignalRegion * 1)(m.GinSignalRegion(0x7F5500000000, 4096, d_cnt.data_ptr()))
-    rings = ctypes.c_void_p()
-    m.check(lib.ofi_amd_gin_rings_create(l_ctx, cap, ctypes.byref(rings)), "rings_create")
     side = torch.cuda.Stream()
-    lstats = m.GinLoopbackStats()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    m.check(lib.ofi_amd_gin_produce_seeded(rings, SEED, l_ops, 1, 64, 1, 1, 0, _gpu.stream()), "produce")
-    rc = lib.ofi_amd_gin_loopback_run(rings, l_ops, ctypes.cast(comms, ctypes.c_void_p),
-                                      ctypes.cast(mrs, ctypes.c_void_p), 3, regions, 1, 32, 16384, 0, 1, 20000,
-                                      ctypes.c_void_p(side.cuda_stream), ctypes.byref(lstats))
-    torch.cuda.synchronize()
-    secs = time.perf_counter() - t0
-    if rc != 0 or lib.ofi_amd_gin_producer_status(rings) != 0:
-        raise RuntimeError("gin loopback rc=%d" % rc)
-    signals_seen = int(d_cnt.sum().item())
-    out["loopback"] = {"contexts": l_ctx, "ops_per_context": l_ops, "puts_per_s": lstats.descriptors / secs,
-                       "payload_gbs": lstats.bytes / secs / 1e9, "payload_bytes": lstats.bytes,
-                       "rdma_writes": lstats.writes, "copy_launches": lstats.launches, "acks": lstats.acks,
-                       "signals": lstats.signals,
-                       "signals_counted_in_hbm_ok": signals_seen == l_ctx * (l_ops // 64), "proxy_threads": 1,
-                       "ns_per_put": secs / lstats.descriptors * 1e9,
-                       "ns_per_put_by_stage": {k: getattr(lstats, "ns_" + k) / lstats.descriptors for k in (
-                           "pop_derive", "tx_post", "wire", "progress", "rx", "launch_wait")}}
-    lib.ofi_amd_gin_rings_destroy(rings)
+    # a progress call after every operation (the strictest caller), and after every 64th: the
+    # reference's own test posts 64 puts and 64 put-signals before its first progress call
+    # (tests/functional/rma.cpp:213-246).  Two passes each; the first warms the pinned tables up.
+    for key, interval in (("loopback", 1), ("loopback_progress_every_64", 64)):
+        best = None
+        for _ in range(2):
+            for c in range(l_ctx):
+                lib.ofi_amd_gin_comm_init(ctypes.byref(comms[c]), c, 4, 131072, 64, 0)
+            d_cnt.zero_()
+            rings = ctypes.c_void_p()
+            m.check(lib.ofi_amd_gin_rings_create(l_ctx, cap, ctypes.byref(rings)), "rings_create")
+            lstats = m.GinLoopbackStats()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            m.check(lib.ofi_amd_gin_produce_seeded(rings, SEED, l_ops, 1, 64, 1, 1, 0, _gpu.stream()), "produce")
+            rc = lib.ofi_amd_gin_loopback_run(rings, l_ops, ctypes.cast(comms, ctypes.c_void_p),
+                                              ctypes.cast(mrs, ctypes.c_void_p), 3, regions, 1, 32, 16384, 0,
+                                              interval, 20000, ctypes.c_void_p(side.cuda_stream),
+                                              ctypes.byref(lstats))
+            torch.cuda.synchronize()
+            secs = time.perf_counter() - t0
+            if rc != 0 or lib.ofi_amd_gin_producer_status(rings) != 0:
+                raise RuntimeError("gin loopback rc=%d" % rc)
+            signals_seen = int(d_cnt.sum().item())
+            lib.ofi_amd_gin_rings_destroy(rings)
+            res = {"contexts": l_ctx, "ops_per_context": l_ops, "progress_call_every": interval,
+                   "puts_per_s": lstats.descriptors / secs,
+                   "payload_gbs": lstats.bytes / secs / 1e9, "payload_bytes": lstats.bytes,
+                   "rdma_writes": lstats.writes, "copy_launches": lstats.launches, "acks": lstats.acks,
+                   "signals": lstats.signals,
+                   "signals_counted_in_hbm_ok": signals_seen == l_ctx * (l_ops // 64), "proxy_threads": 1,
+                   "ns_per_put": secs / lstats.descriptors * 1e9,
+                   "ns_per_put_by_stage": {k: getattr(lstats, "ns_" + k) / lstats.descriptors for k in (
+                       "pop_derive", "tx_post", "wire", "progress", "rx", "launch_wait")}}
+            if best is None or res["puts_per_s"] > best["puts_per_s"]:
+                best = res
+        out[key] = best
     del d_srcbuf, d_dstbuf
     torch.cuda.empty_cache()
     if not args.skip_cpu:
@@ -765,6 +779,10 @@ def main():
         "parity_ok": bounce["parity_ok"],
         "gin_puts_per_s": extra.get("gin", {}).get("drain", {}).get("descs_per_s"),
         "gin_puts_per_s_4_proxy_threads": extra.get("gin", {}).get("drain_4_proxy_threads", {}).get("descs_per_s"),
+        # one proxy thread running the whole iputSignal derivation per descriptor (ring transport alone above)
+        "gin_derive_puts_per_s": extra.get("gin", {}).get("drain_and_derive_wire", {}).get("descs_per_s"),
+        # the same through the transmit engine, the in-process fabric, the receiver and the device copies
+        "gin_end_to_end_puts_per_s": extra.get("gin", {}).get("loopback", {}).get("puts_per_s"),
         "extra": extra,
     }
     print(json.dumps(line))

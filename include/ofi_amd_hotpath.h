@@ -463,10 +463,14 @@ typedef struct {
  *   mode 0: pop + fold every descriptor into the checksum;
  *   mode 1: also store the descriptors: out_desc[c * ops_per_context + i];
  *   mode 2: also run the derivation per context (comms[c], mrs[0..n_mrs); ofi_amd_gin_derive:
- *           iputSignal's for puts, iget's for gets);
- *           out_wire (may be NULL) receives the wire records at
- *           [c * ops_per_context + i].  The checksum is that of mode 0: what a proxy
- *           does with a record (the posts) is not this library's, and checking is
+ *           iputSignal's for puts, iget's for gets).  out_wire receives the wire records at
+ *           [c * ops_per_context + i]; with out_wire NULL they go round a 64-record array of the
+ *           proxy thread's own and are complete in memory there (a post step would read them
+ *           from it), so the timed work is the whole derivation either way.  The checksum is
+ *           that of mode 0, the descriptors alone: what a proxy does with a record (the posts)
+ *           is not this call's, and folding every record into the checksum is checking, not
+ *           proxy work.  (Before mode 3 existed, mode 2 folded the records in: a caller that
+ *           compared mode 2 checksums gets the mode 0 value now and the former value from mode 3.)
  *   mode 3: mode 2, and every wire record is folded into the checksum after its
  *           descriptor (the parity check of the derived stream at any size).
  * A descriptor whose handles lie outside mrs ends the call with -EINVAL.
