@@ -265,7 +265,7 @@ class TunerVariant(ctypes.Structure):
                 ("net_comp_overhead", c_i32)]
 
 
-# name -> (restype, argtypes); every symbol include/ofi_amd_hotpath.h declares
+# name -> (restype, argtypes); every symbol the headers under include/ declare
 PROTOTYPES = {
     "ofi_amd_gpu_init": (ctypes.c_int, []),
     "ofi_amd_gpu_get_device_for_addr": (ctypes.c_int, [c_vp, ctypes.POINTER(ctypes.c_int)]),
@@ -352,6 +352,26 @@ PROTOTYPES = {
     "ofi_amd_gin_tx_progress": (ctypes.c_int, [c_vp]),
     "ofi_amd_gin_tx_test": (ctypes.c_int, [c_vp, c_i32, ctypes.POINTER(ctypes.c_int)]),
     "ofi_amd_gin_tx_stats": (ctypes.c_int, [c_vp, ctypes.POINTER(GinTxStats)]),
+    # include/ofi_amd_rma_abi.h: set-up, then the data-path members of ncclRma_v15_t (int = ncclResult_t)
+    "ofi_amd_rma_ctx_create": (ctypes.c_int, [c_u32, c_u32, c_u64, c_u64, ctypes.POINTER(GinFabricOps), c_u32,
+                                              c_u32, ctypes.POINTER(c_vp)]),
+    "ofi_amd_rma_ctx_destroy": (ctypes.c_int, [c_vp]),
+    "ofi_amd_rma_mr_create": (ctypes.c_int, [c_vp, c_u64, c_vp, c_vp, c_vp, ctypes.POINTER(c_vp)]),
+    "ofi_amd_rma_mr_destroy": (ctypes.c_int, [c_vp]),
+    "ofi_amd_rma_set_flush_buffers": (ctypes.c_int, [c_vp, c_vp, c_u64, c_u64]),
+    "ofi_amd_rma_ack_received": (ctypes.c_int, [c_vp, c_u32, c_u64]),
+    "ofi_amd_rma_peer_state": (ctypes.POINTER(GinComm), [c_vp, c_u32]),
+    "ofi_amd_rma_tx_stats": (ctypes.c_int, [c_vp, ctypes.POINTER(GinTxStats)]),
+    "ofi_amd_rma_iput": (ctypes.c_int, [c_vp, ctypes.c_int, c_u64, c_vp, ctypes.c_size_t, c_u64, c_vp, c_u32, c_u32,
+                                        ctypes.POINTER(c_vp)]),
+    "ofi_amd_rma_iputSignal": (ctypes.c_int, [c_vp, ctypes.c_int, c_u64, c_vp, ctypes.c_size_t, c_u64, c_vp, c_u32,
+                                              c_u64, c_vp, c_u64, c_u32, ctypes.c_bool, c_u32,
+                                              ctypes.POINTER(c_vp)]),
+    "ofi_amd_rma_iget": (ctypes.c_int, [c_vp, ctypes.c_int, c_u64, c_vp, ctypes.c_size_t, c_u64, c_vp, c_u32, c_u32,
+                                        ctypes.POINTER(c_vp)]),
+    "ofi_amd_rma_iflush": (ctypes.c_int, [c_vp, ctypes.c_int, c_vp, c_u32, ctypes.POINTER(c_vp)]),
+    "ofi_amd_rma_test": (ctypes.c_int, [c_vp, c_vp, ctypes.POINTER(ctypes.c_int)]),
+    "ofi_amd_rma_rmaProgress": (ctypes.c_int, [c_vp]),
     "ofi_amd_loopfab_create": (ctypes.c_int, [c_u32, c_u32, ctypes.POINTER(c_vp)]),
     "ofi_amd_loopfab_destroy": (ctypes.c_int, [c_vp]),
     "ofi_amd_loopfab_ops": (ctypes.c_int, [c_vp, ctypes.POINTER(GinFabricOps)]),

@@ -71,6 +71,12 @@ def build_oracle():
                           stderr=subprocess.STDOUT, text=True)
     if proc.returncode != 0:
         raise RuntimeError("oracle build failed:\n%s" % proc.stdout)
+    # the reference-side glue of INTEGRATION.md against the reference's headers (a test binary; only
+    # where the reference tree is present)
+    proc = subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "host")], stdout=subprocess.PIPE,
+                          stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("tests/host build failed:\n%s" % proc.stdout)
 
 
 if __name__ == "__main__":

@@ -289,8 +289,9 @@ typedef struct {
 
 typedef struct ofi_amd_gin_rings ofi_amd_gin_rings_t;
 
-/* n_contexts rings of `capacity` (power of two, >= 64) descriptors each, in
- * pinned host memory: record array (64 B each) + sequence array (u32 each). */
+/* n_contexts rings of `capacity` descriptors each (a power of two, 256 .. 2^24: a workgroup of
+ * the seeded producer reserves 256 slots at a time; -EINVAL otherwise), in pinned host memory:
+ * record array (64 B each) + sequence array (u32 each). */
 int ofi_amd_gin_rings_create(uint32_t n_contexts, uint32_t capacity, ofi_amd_gin_rings_t **out);
 int ofi_amd_gin_rings_destroy(ofi_amd_gin_rings_t *rings);
 /*

@@ -1,0 +1,230 @@
+/*
+ * The glue a maintainer of the reference would add on top of the C ABI, compiled for real:
+ * the replacement of src/nccl_ofi_rocm.cpp and an nccl_ofi_device_copy implementation, both
+ * as they are printed in INTEGRATION.md (sections 1 and 2; tests/test_integration_glue.py
+ * checks that the text between the markers below is the text printed there), built against
+ * the reference's own headers where they lie (include/nccl_ofi_rocm.h,
+ * include/nccl_ofi_device_copy.h) and linked against libofi_amd_hotpath.so.
+ *
+ *   integration_glue link   the forwards that answer without a GPU
+ *   integration_glue gpu    the patterns of the reference's tests/unit/gdrcopy.cpp:15-133 (a
+ *                           2 MiB buffer written and read back whole, a 10-byte buffer written
+ *                           and read back byte by byte) through the C++ class, plus offsets
+ *                           and sizes around the class's CPU-store / copy-engine switch
+ */
+#include <cerrno>
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+// [section 1]
+// src/nccl_ofi_rocm.cpp (replacement)
+#include <cstddef>
+#include "nccl_ofi_rocm.h"
+#include "ofi_amd_hotpath.h"
+
+int nccl_net_ofi_gpu_init(void)                                   { return ofi_amd_gpu_init(); }
+int nccl_net_ofi_get_gpu_device_for_addr(void *p, int *dev)       { return ofi_amd_gpu_get_device_for_addr(p, dev); }
+int nccl_net_ofi_gpu_flush_gpudirect_rdma_writes(void)            { return ofi_amd_gpu_flush_gpudirect_rdma_writes(); } // -EPERM, as today
+int nccl_net_ofi_gpu_mem_alloc(void **p, size_t n)                { return ofi_amd_gpu_mem_alloc(p, n); }
+int nccl_net_ofi_gpu_mem_free(void *p)                            { return ofi_amd_gpu_mem_free(p); }
+int nccl_net_ofi_gpu_mem_copy_host_to_device(void *d, void *s, size_t n) { return ofi_amd_gpu_mem_copy_host_to_device(d, s, n); }
+int nccl_net_ofi_gpu_get_dma_buf_fd(void *p, size_t n, int *fd, size_t *off) { return ofi_amd_gpu_get_dma_buf_fd(p, n, fd, off); }
+bool nccl_net_ofi_gpu_have_dma_buf_attr(void)                     { return ofi_amd_gpu_have_dma_buf_attr() != 0; }
+bool nccl_net_ofi_gpu_have_gdr_support_attr(void)                 { return ofi_amd_gpu_have_gdr_support_attr() != 0; }
+// [end of section 1]
+
+// [section 2]
+#include "nccl_ofi_device_copy.h"
+
+class nccl_ofi_device_copy_amd : public nccl_ofi_device_copy {
+	struct Handle : RegHandle { ofi_amd_devcopy_region_t *r; };
+public:
+	int register_region(void *ptr, size_t size, RegHandle *&out) override {
+		auto *h = new Handle;
+		int rc = ofi_amd_devcopy_register(ptr, size, &h->r);
+		if (rc) { delete h; return rc; }
+		out = h; return 0;
+	}
+	int copy_to_device(const void *host, const RegHandle &h, size_t off, size_t n) override {
+		return ofi_amd_devcopy_to_device(host, static_cast<const Handle &>(h).r, off, n);
+	}
+	int copy_from_device(const RegHandle &h, size_t off, void *host, size_t n) override {
+		return ofi_amd_devcopy_from_device(static_cast<const Handle &>(h).r, off, host, n);
+	}
+	bool forced_pcie_copy() override { return ofi_amd_devcopy_forced_pcie_copy() != 0; }
+	int deregister_region(RegHandle *h) override {
+		int rc = ofi_amd_devcopy_deregister(static_cast<Handle *>(h)->r); delete static_cast<Handle *>(h); return rc;
+	}
+};
+// [end of section 2]
+
+/* The data-path members of the reference's ncclRma_v15_t take this library's functions as they
+ * are: a mismatch in any parameter list is a compile error here. */
+#include "nccl/net.h"
+#include "nccl/rma_v15.h"
+#include "ofi_amd_rma_abi.h"
+
+static ncclRma_v15_t rma_table_with_this_librarys_data_path()
+{
+	ncclRma_v15_t t = {};
+	t.name = "Libfabric";
+	t.iput = ofi_amd_rma_iput;
+	t.iputSignal = ofi_amd_rma_iputSignal;
+	t.iget = ofi_amd_rma_iget;
+	t.iflush = ofi_amd_rma_iflush;
+	t.test = ofi_amd_rma_test;
+	t.rmaProgress = ofi_amd_rma_rmaProgress;
+	return t;
+}
+
+#define CHECK(cond)                                                                       \
+	do {                                                                              \
+		if (!(cond)) {                                                            \
+			fprintf(stderr, "%s:%d: check failed: %s\n", __FILE__, __LINE__, #cond); \
+			return 1;                                                         \
+		}                                                                         \
+	} while (0)
+
+static int link_checks()
+{
+	/* answers that do not depend on a device */
+	CHECK(nccl_net_ofi_gpu_flush_gpudirect_rdma_writes() == -EPERM); /* src/nccl_ofi_rocm.cpp:53-56 */
+	CHECK(nccl_net_ofi_gpu_have_gdr_support_attr() == false);        /* :78-81 */
+	nccl_ofi_device_copy_amd copy;
+	nccl_ofi_device_copy &iface = copy;
+	CHECK(iface.forced_pcie_copy() == false);
+	/* one put through the table's pointers over the in-process fabric, polled to completion */
+	{
+		const ncclRma_v15_t table = rma_table_with_this_librarys_data_path();
+		ofi_amd_loopfab_t *fab = nullptr;
+		ofi_amd_gin_fabric_ops_t ops;
+		CHECK(ofi_amd_loopfab_create(4, 64, &fab) == 0 && ofi_amd_loopfab_ops(fab, &ops) == 0);
+		ofi_amd_rma_ctx_t *rma = nullptr;
+		CHECK(ofi_amd_rma_ctx_create(2, 4, 131072, 64, &ops, 256, 0, &rma) == 0);
+		const uint64_t addr[2] = {0x7e0000000000ull, 0x7e0100000000ull}, keys[8] = {1, 2, 3, 4, 5, 6, 7, 8};
+		ofi_amd_rma_mr_t *mr = nullptr;
+		CHECK(ofi_amd_rma_mr_create(rma, 0x7f0000000000ull, addr, addr, keys, &mr) == 0);
+		void *request = nullptr;
+		CHECK(table.iput(rma, 0, 16, mr, 5000, 32, mr, 1, ncclRmaOptFlagsDefault, &request) == ncclSuccess && request);
+		ofi_amd_gin_post_t sent[4];
+		CHECK(ofi_amd_loopfab_take_transmitted(fab, sent, 4) == 1);
+		CHECK(sent[0].kind == OFI_AMD_GIN_POST_WRITE && sent[0].len == 5000 && sent[0].src == 0x7f0000000010ull &&
+		      sent[0].dest == addr[1] + 32 && sent[0].key == keys[4 + sent[0].rail]);
+		int done = 0;
+		CHECK(table.test(rma, request, &done) == ncclSuccess && done == 0);
+		CHECK(table.rmaProgress(rma) == ncclSuccess);
+		CHECK(table.test(rma, request, &done) == ncclSuccess && done == 1);
+		CHECK(table.iput(rma, 0, 0, mr, 8, 0, mr, 7, 0, &request) == ncclInternalError); /* no such rank */
+		CHECK(ofi_amd_rma_mr_destroy(mr) == 0 && ofi_amd_rma_ctx_destroy(rma) == 0 && ofi_amd_loopfab_destroy(fab) == 0);
+	}
+	const int init = nccl_net_ofi_gpu_init();
+	if (init == -ENODEV) {
+		/* no GPU here: every device call says so, through the glue as through the C ABI */
+		void *p = nullptr;
+		CHECK(nccl_net_ofi_gpu_mem_alloc(&p, 64) == -ENODEV);
+		nccl_ofi_device_copy::RegHandle *h = nullptr;
+		char byte = 0;
+		CHECK(iface.register_region(&byte, 1, h) == -ENODEV && h == nullptr);
+		printf("link: ok (no device)\n");
+		return 0;
+	}
+	CHECK(init == 0);
+	printf("link: ok (device present)\n");
+	return 0;
+}
+
+static int gpu_checks()
+{
+	CHECK(nccl_net_ofi_gpu_init() == 0);
+	nccl_ofi_device_copy_amd amd;
+	nccl_ofi_device_copy &gdr = amd;
+
+	{ /* test_large_buffer, tests/unit/gdrcopy.cpp:15-74 */
+		constexpr size_t buff_size = 2 * 1024 * 1024UL;
+		void *ptr = nullptr;
+		CHECK(nccl_net_ofi_gpu_mem_alloc(&ptr, buff_size) == 0);
+		int dev = -1;
+		CHECK(nccl_net_ofi_get_gpu_device_for_addr(ptr, &dev) == 0 && dev >= 0);
+		nccl_ofi_device_copy::RegHandle *handle = nullptr;
+		CHECK(gdr.register_region(ptr, buff_size, handle) == 0);
+		std::vector<char> host_buff(buff_size, 'A'), dst_host_buff(buff_size, 0);
+		CHECK(gdr.copy_to_device(host_buff.data(), *handle, 0, buff_size) == 0);
+		CHECK(gdr.copy_from_device(*handle, 0, dst_host_buff.data(), buff_size) == 0);
+		CHECK(memcmp(host_buff.data(), dst_host_buff.data(), buff_size) == 0);
+		CHECK(gdr.deregister_region(handle) == 0);
+		CHECK(nccl_net_ofi_gpu_mem_free(ptr) == 0);
+	}
+	{ /* test_small_buffer, :76-133 */
+		constexpr size_t buff_size = 10;
+		void *ptr = nullptr;
+		CHECK(nccl_net_ofi_gpu_mem_alloc(&ptr, buff_size) == 0);
+		nccl_ofi_device_copy::RegHandle *handle = nullptr;
+		CHECK(gdr.register_region(ptr, buff_size, handle) == 0);
+		for (size_t i = 0; i < buff_size; ++i) {
+			uint8_t v = (uint8_t)i;
+			CHECK(gdr.copy_to_device(&v, *handle, i, 1) == 0);
+		}
+		for (size_t i = 0; i < buff_size; ++i) {
+			uint8_t v = 0xff;
+			CHECK(gdr.copy_from_device(*handle, i, &v, 1) == 0);
+			CHECK(v == i);
+		}
+		CHECK(gdr.deregister_region(handle) == 0);
+		CHECK(nccl_net_ofi_gpu_mem_free(ptr) == 0);
+	}
+	{ /* either side of the switch between CPU stores / loads and the copy engine, at odd offsets,
+	   * against a host-to-device copy through the other path of the glue */
+		constexpr size_t buff_size = 16u << 20;
+		void *ptr = nullptr;
+		CHECK(nccl_net_ofi_gpu_mem_alloc(&ptr, buff_size) == 0);
+		nccl_ofi_device_copy::RegHandle *handle = nullptr;
+		CHECK(gdr.register_region(ptr, buff_size, handle) == 0);
+		std::vector<uint8_t> pattern(buff_size), back(buff_size);
+		for (size_t i = 0; i < buff_size; i++) {
+			pattern[i] = (uint8_t)(i * 2654435761u >> 24);
+		}
+		std::vector<uint8_t> zero(buff_size, 0);
+		CHECK(nccl_net_ofi_gpu_mem_copy_host_to_device(ptr, zero.data(), buff_size) == 0);
+		const size_t sizes[] = {1, 255, 256, 257, 4096, (2u << 20) - 1, 2u << 20, (2u << 20) + 1, 3u << 20};
+		size_t at = 3;
+		for (size_t n : sizes) {
+			CHECK(at + n <= buff_size);
+			CHECK(gdr.copy_to_device(pattern.data() + at, *handle, at, n) == 0);
+			CHECK(gdr.copy_from_device(*handle, at, back.data() + at, n) == 0);
+			CHECK(memcmp(pattern.data() + at, back.data() + at, n) == 0);
+			at += n + 5;
+		}
+		/* out of range: refused, nothing written */
+		CHECK(gdr.copy_to_device(pattern.data(), *handle, buff_size - 4, 8) == -EINVAL);
+		CHECK(gdr.copy_from_device(*handle, buff_size, back.data(), 1) == -EINVAL);
+		CHECK(gdr.deregister_region(handle) == 0);
+		CHECK(nccl_net_ofi_gpu_mem_free(ptr) == 0);
+	}
+	{ /* the dma-buf forward, called as the reference calls it for a registration */
+		void *ptr = nullptr;
+		CHECK(nccl_net_ofi_gpu_mem_alloc(&ptr, 1u << 20) == 0);
+		if (nccl_net_ofi_gpu_have_dma_buf_attr()) {
+			int fd = -1;
+			size_t off = 99;
+			CHECK(nccl_net_ofi_gpu_get_dma_buf_fd(ptr, 1u << 20, &fd, &off) == 0 && fd >= 0 && off == 0);
+		}
+		CHECK(nccl_net_ofi_gpu_mem_free(ptr) == 0);
+	}
+	printf("gpu: ok\n");
+	return 0;
+}
+
+int main(int argc, char **argv)
+{
+	if (argc == 2 && strcmp(argv[1], "link") == 0) {
+		return link_checks();
+	}
+	if (argc == 2 && strcmp(argv[1], "gpu") == 0) {
+		return gpu_checks();
+	}
+	fprintf(stderr, "usage: %s link|gpu\n", argv[0]);
+	return 2;
+}

@@ -14,7 +14,8 @@ import aws_ofi_nccl_amd as m
 from aws_ofi_nccl_amd import synthetic
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADERS = [os.path.join(ROOT, "include", h) for h in ("ofi_amd_hotpath.h", "ofi_amd_wire.h", "ofi_amd_sendrecv.h")]
+HEADERS = [os.path.join(ROOT, "include", h) for h in ("ofi_amd_hotpath.h", "ofi_amd_wire.h", "ofi_amd_sendrecv.h",
+                                                      "ofi_amd_rma_abi.h")]
 
 
 def declared_symbols():
