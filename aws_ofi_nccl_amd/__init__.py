@@ -290,6 +290,7 @@ PROTOTYPES = {
     "ofi_amd_gpu_host_free": (ctypes.c_int, [c_vp]),
     "ofi_amd_gpu_host_get_device_pointer": (ctypes.c_int, [ctypes.POINTER(c_vp), c_vp]),
     "ofi_amd_sched_batch": (ctypes.c_int, [c_vp, c_vp, c_u64, c_u64, c_vp, c_vp, c_vp]),
+    "ofi_amd_sched_stream_release": (ctypes.c_int, [c_vp]),
     "ofi_amd_sched_batch_noalloc": (ctypes.c_int, [c_vp, c_vp, c_u64, c_u64, c_vp, c_vp, c_vp]),
     "ofi_amd_sched_get_schedule": (ctypes.c_int, [ctypes.POINTER(SchedState), c_u64, c_u64,
                                                   ctypes.POINTER(XferInfo)]),
@@ -308,6 +309,7 @@ PROTOTYPES = {
     "ofi_amd_flush_test": (ctypes.c_int, [c_vp, c_u32, c_u64]),
     "ofi_amd_flush_read": (ctypes.c_int, [c_vp, c_vp, c_u32, c_vp, c_vp]),
     "ofi_amd_devcopy_register": (ctypes.c_int, [c_vp, ctypes.c_size_t, ctypes.POINTER(c_vp)]),
+    "ofi_amd_devcopy_cpu_mapped": (ctypes.c_int, [c_vp]),
     "ofi_amd_devcopy_to_device": (ctypes.c_int, [c_vp, c_vp, ctypes.c_size_t, ctypes.c_size_t]),
     "ofi_amd_devcopy_from_device": (ctypes.c_int, [c_vp, ctypes.c_size_t, c_vp,
                                                    ctypes.c_size_t]),

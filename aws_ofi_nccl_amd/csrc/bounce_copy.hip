@@ -51,6 +51,8 @@
 #include <new>
 
 #include <immintrin.h>
+#include <sys/mman.h>
+#include <unistd.h>
 
 #include "common.hpp"
 #include "ofi_amd_hotpath.h"
@@ -433,8 +435,10 @@ __global__ __launch_bounds__(64) void flush_post_kernel(const uint64_t *__restri
  * mmap-ing (gdrcopy_RegHandle::mapped_ptr, include/nccl_ofi_gdrcopy.h:54-74) is the device
  * pointer itself. */
 struct ofi_amd_devcopy_region {
-	uint8_t *base;   /* device address = CPU-visible mapping */
+	uint8_t *base;   /* device address (= CPU-visible mapping where cpu_mapped) */
 	size_t size;
+	bool cpu_mapped; /* the CPU can store to and load from `base`: large BAR and the range is in the
+			  * process's address space; otherwise every copy goes through the copy engine */
 };
 
 /* CPU stores into the mapping are write-combined: 0.2-0.4 us for anything up to a page and
@@ -622,14 +626,25 @@ int ofi_amd_devcopy_register(void *device_ptr, size_t size, ofi_amd_devcopy_regi
 	if (attr.type != hipMemoryTypeDevice) {
 		return -EINVAL;
 	}
-	/* the CPU reaches device memory only where the whole of it sits behind the PCIe BAR */
+	/* The CPU reaches device memory only where the whole of it sits behind the PCIe BAR, and
+	 * then only allocations that the runtime has mapped into the process at their device
+	 * address (hipMalloc memory is; an imported or virtual-memory allocation need not be):
+	 * the first and the last page of the range are asked of the kernel.  Without either,
+	 * the region still registers and its copies take the copy engine at every size, as the
+	 * interface promises nothing about the path. */
 	int large_bar = 0;
 	if (hipDeviceGetAttribute(&large_bar, hipDeviceAttributeIsLargeBar, attr.device) != hipSuccess) {
 		(void)hipGetLastError();
-		return -ENOTSUP;
+		large_bar = 0;
 	}
-	if (!large_bar) {
-		return -ENOTSUP;
+	bool mapped = large_bar != 0;
+	if (mapped) {
+		const long page = sysconf(_SC_PAGESIZE);
+		const uintptr_t first = reinterpret_cast<uintptr_t>(device_ptr) & ~(uintptr_t)(page - 1);
+		const uintptr_t last = (reinterpret_cast<uintptr_t>(device_ptr) + size - 1) & ~(uintptr_t)(page - 1);
+		unsigned char vec = 0;
+		mapped = mincore(reinterpret_cast<void *>(first), (size_t)page, &vec) == 0 &&
+			 mincore(reinterpret_cast<void *>(last), (size_t)page, &vec) == 0;
 	}
 	auto *h = new (std::nothrow) ofi_amd_devcopy_region;
 	if (!h) {
@@ -637,6 +652,7 @@ int ofi_amd_devcopy_register(void *device_ptr, size_t size, ofi_amd_devcopy_regi
 	}
 	h->base = static_cast<uint8_t *>(device_ptr);
 	h->size = size;
+	h->cpu_mapped = mapped;
 	*out = h;
 	return 0;
 }
@@ -647,7 +663,7 @@ int ofi_amd_devcopy_to_device(const void *host_ptr, ofi_amd_devcopy_region_t *h,
 	if (!h || !host_ptr || offset > h->size || size > h->size - offset) {
 		return -EINVAL;
 	}
-	if (size <= kCpuStoreMax) {
+	if (h->cpu_mapped && size <= kCpuStoreMax) {
 		/* gdr_copy_to_mapping: CPU stores through the mapping, then drain the
 		 * write-combining buffers so that the bytes are on their way before the caller
 		 * rings any doorbell */
@@ -665,7 +681,7 @@ int ofi_amd_devcopy_from_device(ofi_amd_devcopy_region_t *h, size_t offset, void
 	if (!h || !host_ptr || offset > h->size || size > h->size - offset) {
 		return -EINVAL;
 	}
-	if (size <= kCpuLoadMax) {
+	if (h->cpu_mapped && size <= kCpuLoadMax) {
 		/* gdr_copy_from_mapping: CPU loads through the mapping */
 		std::memcpy(host_ptr, h->base + offset, size);
 		_mm_lfence();
@@ -673,6 +689,11 @@ int ofi_amd_devcopy_from_device(ofi_amd_devcopy_region_t *h, size_t offset, void
 	}
 	OFI_AMD_HIP_TRY(hipMemcpy(host_ptr, h->base + offset, size, hipMemcpyDeviceToHost));
 	return 0;
+}
+
+int ofi_amd_devcopy_cpu_mapped(const ofi_amd_devcopy_region_t *h)
+{
+	return h ? (h->cpu_mapped ? 1 : 0) : -EINVAL;
 }
 
 int ofi_amd_devcopy_forced_pcie_copy(void)

@@ -478,7 +478,25 @@ constexpr int kMaxDevices = 64;
 std::mutex g_scratch_lock;
 uint32_t *g_scratch_ptr[kMaxDevices]; /* device address of `scratch` on each GPU, once looked up */
 
-/* Device address of the current GPU's copy of `scratch` (each GPU has its own). */
+/* Device address of the current GPU's copy of `scratch` as ofi_amd_gpu_init() has recorded it;
+ * no runtime call that could allocate.  -ENXIO when the address has not been looked up. */
+int cached_scratch_of_current_device(uint32_t **out)
+{
+	int dev = -1;
+	OFI_AMD_HIP_TRY(hipGetDevice(&dev));
+	if (dev < 0 || dev >= kMaxDevices) {
+		return -ENODEV;
+	}
+	std::lock_guard<std::mutex> g(g_scratch_lock);
+	if (!g_scratch_ptr[dev]) {
+		return -ENXIO;
+	}
+	*out = g_scratch_ptr[dev];
+	return 0;
+}
+
+/* Device address of the current GPU's copy of `scratch` (each GPU has its own), looked up on
+ * first use: set-up only. */
 int scratch_of_current_device(uint32_t **out)
 {
 	int dev = -1;
@@ -615,6 +633,29 @@ int ofi_amd_sched_batch(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes,
 	return 0;
 }
 
+int ofi_amd_sched_stream_release(void *stream)
+{
+	int rc = require_device();
+	if (rc != 0) {
+		return rc;
+	}
+	workspace_t ws;
+	{
+		std::lock_guard<std::mutex> g(g_ws_lock);
+		auto it = g_ws_by_stream.find(stream);
+		if (it == g_ws_by_stream.end()) {
+			return 0; /* nothing was ever allocated for it */
+		}
+		ws = it->second;
+		g_ws_by_stream.erase(it);
+	}
+	/* launches queued on the stream may still read the scratch */
+	OFI_AMD_HIP_TRY(hipStreamSynchronize(as_stream(stream)));
+	(void)hipFree(ws.totals);
+	(void)hipFree(ws.prefix);
+	return 0;
+}
+
 int ofi_amd_sched_batch_noalloc(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes, uint64_t n,
 				uint64_t align, uint32_t *d_num_xfers, ofi_amd_xfer_info_t *d_xfers,
 				void *stream)
@@ -640,7 +681,7 @@ int ofi_amd_sched_batch_noalloc(ofi_amd_sched_state_t *d_state, const uint64_t *
 		return -ENXIO; /* ofi_amd_gpu_init() allocates it; this call must not */
 	}
 	uint32_t *base = nullptr;
-	rc = scratch_of_current_device(&base);
+	rc = cached_scratch_of_current_device(&base); /* -ENXIO: ofi_amd_gpu_init() looks the address up; this call must not */
 	if (rc != 0) {
 		return rc;
 	}

@@ -393,18 +393,25 @@ double log2_coord(double v)
  * not remembered: the next caller tries again. */
 int device_region_tables(region_tables_t *out)
 {
+	/* one copy of the tables per GPU, uploaded to whichever is current on first use there */
+	constexpr int kMaxDevices = 64;
 	static std::mutex lock;
-	static region_tables_t tables;
-	static bool built = false;
+	static region_tables_t tables[kMaxDevices];
+	static bool built[kMaxDevices];
+	int dev = -1;
+	if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+		(void)hipGetLastError();
+		return -ENODEV;
+	}
 	std::lock_guard<std::mutex> g(lock);
-	if (!built) {
-		const int status = build_region_tables(&tables);
+	if (!built[dev]) {
+		const int status = build_region_tables(&tables[dev]);
 		if (status != 0) {
 			return status;
 		}
-		built = true;
+		built[dev] = true;
 	}
-	*out = tables;
+	*out = tables[dev];
 	return 0;
 }
 

@@ -67,12 +67,25 @@ struct staging_t {
 	uint32_t cap = 0;
 	hipStream_t stream = nullptr;
 };
-staging_t g_stage;
+/* one per GPU: a stream and pinned staging belong to the device that was current when they
+ * were made, and a process may drive several */
+constexpr int kMaxDevices = 64;
+staging_t g_stages[kMaxDevices];
+
+staging_t *stage_of_current_device()
+{
+	int dev = -1;
+	if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+		(void)hipGetLastError();
+		return nullptr;
+	}
+	return &g_stages[dev];
+}
 
 } // namespace
 
 /* stream and staging for `want` questions; the caller holds g_stage.lock */
-static int ensure_staging(uint32_t want)
+static int ensure_staging(staging_t &g_stage, uint32_t want)
 {
 	if (!g_stage.stream) {
 		OFI_AMD_HIP_TRY(hipStreamCreateWithFlags(&g_stage.stream, hipStreamNonBlocking));
@@ -108,8 +121,12 @@ extern "C" int ofi_amd_tuner_query_prepare(uint32_t capacity)
 	if (rc != 0) {
 		return rc;
 	}
-	std::lock_guard<std::mutex> g(g_stage.lock);
-	return ensure_staging(capacity);
+	staging_t *stage = stage_of_current_device();
+	if (!stage) {
+		return -ENODEV;
+	}
+	std::lock_guard<std::mutex> g(stage->lock);
+	return ensure_staging(*stage, capacity);
 }
 
 extern "C" int ofi_amd_tuner_query(const ofi_amd_tuner_query_t *queries, uint32_t n,
@@ -141,8 +158,13 @@ extern "C" int ofi_amd_tuner_query(const ofi_amd_tuner_query_t *queries, uint32_
 		return rc;
 	}
 
+	staging_t *stage = stage_of_current_device();
+	if (!stage) {
+		return -ENODEV;
+	}
+	staging_t &g_stage = *stage;
 	std::lock_guard<std::mutex> g(g_stage.lock);
-	rc = ensure_staging(n);
+	rc = ensure_staging(g_stage, n);
 	if (rc != 0) {
 		return rc;
 	}

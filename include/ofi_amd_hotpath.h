@@ -121,6 +121,10 @@ typedef struct {
 int ofi_amd_sched_batch(ofi_amd_sched_state_t *d_state, const uint64_t *d_sizes, uint64_t n,
 			uint64_t align, uint32_t *d_num_xfers, ofi_amd_xfer_info_t *d_xfers,
 			void *stream);
+/* ofi_amd_sched_batch keeps a few KiB of device scratch per stream it has been called with
+ * (the reference's scheduler keeps a freelist per instance, src/nccl_ofi_scheduler.cpp:135-190).
+ * A caller that destroys a stream hands the scratch back first: waits for the stream, frees. */
+int ofi_amd_sched_stream_release(void *stream);
 
 /*
  * ofi_amd_sched_batch for callers that cannot allocate device memory: code under HIP graph
@@ -241,14 +245,19 @@ int ofi_amd_flush_test(const void *slots_host, uint32_t num_rails, uint64_t sent
  * small synchronous host<->device copies at an offset, done by the CPU through a mapping of
  * the device memory as GDRCopy does (src/nccl_ofi_gdrcopy.cpp:108-179).  On a large-BAR
  * system (hipDeviceAttributeIsLargeBar) device memory is CPU-addressable at its device
- * address, which is the mapping; register returns -ENOTSUP where it is not -- there is no
- * second path.  copy_to_device up to 2 MiB is CPU stores plus a store fence (0.2-0.4 us up to
- * a page, 20 GB/s beyond), copy_from_device up to 256 bytes CPU loads (2.5 us per 64 bytes);
- * larger copies, where the copy engine wins, go through it.  As with GDRCopy, neither call
+ * address, which is the mapping.  copy_to_device up to 2 MiB is then CPU stores plus a store
+ * fence (0.2-0.4 us up to a page, 20 GB/s beyond), copy_from_device up to 256 bytes CPU loads
+ * (2.5 us per 64 bytes); larger copies, where the copy engine wins, go through it.  Where the
+ * device has no large BAR, or the runtime has not mapped the registered range into the
+ * process, the region registers all the same and every copy takes the copy engine
+ * (11-14 us at the least).  As with GDRCopy, neither call
  * waits for GPU work: a store is seen by work submitted after the call returns, a load sees
  * the results of work that has completed. */
 typedef struct ofi_amd_devcopy_region ofi_amd_devcopy_region_t;
 int ofi_amd_devcopy_register(void *device_ptr, size_t size, ofi_amd_devcopy_region_t **out);
+/* 1: small copies of this region are CPU stores / loads through the mapping; 0: every copy takes
+ * the copy engine (no large BAR, or the range is not mapped into the process) */
+int ofi_amd_devcopy_cpu_mapped(const ofi_amd_devcopy_region_t *region);
 int ofi_amd_devcopy_to_device(const void *host_ptr, ofi_amd_devcopy_region_t *h, size_t offset,
 			      size_t size);
 int ofi_amd_devcopy_from_device(ofi_amd_devcopy_region_t *h, size_t offset, void *host_ptr,

@@ -245,3 +245,44 @@ def test_batches_on_two_streams_do_not_share_scratch(lib, oracle, gpu):
         assert np.array_equal(_gpu.to_host(d_xf, np.uint64).reshape(n, 4, 3), want_xf)
         st = read_state(d_state)
         assert (st.rr_small_counter, st.rr_counter) == (ost.rr_small_counter, ost.rr_counter)
+
+
+def test_stream_scratch_is_handed_back_and_made_again(lib, oracle, gpu):
+    """ofi_amd_sched_stream_release: the per-stream scratch goes back to the device (the runtime's
+    count of free memory does not fall over many streams used once each), a stream nothing was
+    allocated for is fine, and a released stream can be used again with the same results."""
+    n = 300_001
+    sizes = synthetic.stripe_sizes(77, n)
+    want_num, want_xf, _ = _oracle.sched_batch(oracle, sizes, 4, 131072, 64, (0, 0))
+    d_sizes = _gpu.to_dev(sizes)
+    d_num = torch.zeros(n, dtype=torch.int32, device="cuda")
+    d_xf = torch.zeros(n * 12, dtype=torch.int64, device="cuda")
+
+    def once(stream):
+        d_state = dev_state(4, 131072, 64, (0, 0))
+        assert lib.ofi_amd_sched_batch(d_state.data_ptr(), d_sizes.data_ptr(), n, 128, d_num.data_ptr(),
+                                       d_xf.data_ptr(), ctypes.c_void_p(stream.cuda_stream)) == 0
+
+    s = torch.cuda.Stream()
+    once(s)
+    assert lib.ofi_amd_sched_stream_release(ctypes.c_void_p(s.cuda_stream)) == 0     # waits for the launches
+    assert np.array_equal(_gpu.to_host(d_num, np.uint32), want_num)
+    assert lib.ofi_amd_sched_stream_release(ctypes.c_void_p(s.cuda_stream)) == 0     # nothing left: fine
+    d_num.zero_()
+    once(s)                                                                          # allocated afresh
+    torch.cuda.synchronize()
+    assert np.array_equal(_gpu.to_host(d_num, np.uint32), want_num)
+    assert np.array_equal(_gpu.to_host(d_xf, np.uint64).reshape(n, 4, 3), want_xf)
+    assert lib.ofi_amd_sched_stream_release(ctypes.c_void_p(s.cuda_stream)) == 0
+    # torch hands out streams from a pool of 32: a first round makes them all (a stream's queue takes
+    # device memory of its own), the second round must then leave the count of free memory alone
+    free_before = None
+    for rnd in range(2):
+        for _ in range(64):
+            t = torch.cuda.Stream()
+            once(t)
+            assert lib.ofi_amd_sched_stream_release(ctypes.c_void_p(t.cuda_stream)) == 0
+        torch.cuda.synchronize()
+        if rnd == 0:
+            free_before, _ = torch.cuda.mem_get_info()
+    assert torch.cuda.mem_get_info()[0] == free_before

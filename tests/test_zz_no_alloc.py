@@ -1,6 +1,8 @@
 """GPU parity of the striping entry point that allocates nothing (ofi_amd_sched_batch_noalloc)
 against ofi_amd_sched_batch and the CPU oracle: two calls in a row on the same scratch, the
 second with a smaller input, then a batch large enough for the separate scan launch."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -71,6 +73,38 @@ def test_noalloc_at_its_largest_batch(lib, gpu):
     assert torch.equal(rows[:, :, 2].sum(dim=1), d_sizes)
     assert int(outs[0][0].min()) == 1 and int(outs[0][0].max()) == 4
     assert _gpu.fetch_async_errors(lib) == 0
+
+
+def test_noalloc_calls_leave_free_device_memory_where_it_was(lib, gpu):
+    """What the entry point is for: after ofi_amd_gpu_init() (which records the scratch array's
+    address on every GPU) a call takes no device memory -- the runtime's count of free bytes
+    (hipMemGetInfo) is the same before and after calls of several sizes, the larger ones through
+    the separate scan launch, on a stream that has never been used with the allocating entry
+    point (that one would allocate its per-stream scratch on such a stream)."""
+    assert lib.ofi_amd_gpu_init() == 0
+    side = torch.cuda.Stream()
+    stream = ctypes.c_void_p(side.cuda_stream)
+    big = (1 << 22) + 777
+    d_sizes = _gpu.to_dev(synthetic.stripe_sizes(21, big))
+    d_state = dev_state(4, 131072, 64, (0, 0))
+    d_num = torch.zeros(big, dtype=torch.int32, device="cuda")
+    d_xf = torch.zeros(big * 12, dtype=torch.int64, device="cuda")
+    call = lambda n: lib.ofi_amd_sched_batch_noalloc(d_state.data_ptr(), d_sizes.data_ptr(), n, 128, d_num.data_ptr(),
+                                                     d_xf.data_ptr(), stream)
+    assert call(1000) == 0 and call(big) == 0              # code objects of every kernel are on the device now
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for n in (1, 513, 300007, big, 1234, 3_000_000):
+        assert call(n) == 0
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, (free_before, free_after)
+    assert _gpu.fetch_async_errors(lib) == 0
+    # the count does move when device memory is taken: the comparison above can tell
+    p = ctypes.c_void_p()
+    assert lib.ofi_amd_gpu_mem_alloc(ctypes.byref(p), 64 << 20) == 0
+    assert torch.cuda.mem_get_info()[0] <= free_before - (64 << 20)
+    assert lib.ofi_amd_gpu_mem_free(p) == 0
 
 
 def test_noalloc_rejects_oversized_batch(lib, gpu):
