@@ -57,26 +57,6 @@
 #include "common.hpp"
 #include "ofi_amd_hotpath.h"
 
-/* Swept on the configured batch over thousands of launches in a row (1, 2, 4, 8 or 16
- * wavefronts per workgroup, XCD runs of 8 to 128 buffers): 8 wavefronts per workgroup with runs
- * of 32 buffers per XCD was the fastest (91.1 us per launch; 1 x 32: 92.7, 4 x 8: 91.8,
- * 16 x 2: 92.6). */
-#ifndef OFI_BOUNCE_WAVES
-#define OFI_BOUNCE_WAVES 8 /* buffers (= wavefronts) per workgroup */
-#endif
-#ifndef OFI_EAGER_WAVES
-#define OFI_EAGER_WAVES 1
-#endif
-#ifndef OFI_EAGER_GROUP
-#define OFI_EAGER_GROUP 32
-#endif
-#ifndef OFI_TABLE_WAVES
-#define OFI_TABLE_WAVES 1
-#endif
-#ifndef OFI_BOUNCE_GROUP
-#define OFI_BOUNCE_GROUP 4 /* consecutive workgroups that share an XCD */
-#endif
-
 namespace {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -85,13 +65,19 @@ struct __attribute__((packed, aligned(4))) dword_aligned_u32x4 {
 	u32x4 v;
 };
 
-constexpr int kWavesPerBlock = OFI_BOUNCE_WAVES;
+/* Buffers (= wavefronts) per workgroup and consecutive workgroups that share an XCD, swept over
+ * thousands of launches in a row on 65,536 buffers.  Bounce copy: 8 wavefronts per workgroup with
+ * runs of 4 workgroups (32 buffers) per XCD was the fastest (91.1 us per launch; 4 x 8: 91.8,
+ * 2 x 16: 92.5, 16 x 2: 92.6, 8 x 8: 91.7).  The eager copy, whose sources are rx buffers in
+ * arrival order, prefers single-wavefront workgroups (1 x 32: 97.8 us, 4 x 8: 98.4, 8 x 4: 101.6,
+ * 16 x 2: 108.6), and so does the table copy (1: 419.9 us per GiB, 4: 439.5, 8: 430.3). */
+constexpr int kWavesPerBlock = 8;
 constexpr int kBlock = 64 * kWavesPerBlock;
-constexpr int kEagerWaves = OFI_EAGER_WAVES;
-constexpr uint32_t kEagerGroup = OFI_EAGER_GROUP;
-constexpr int kTableWaves = OFI_TABLE_WAVES;
+constexpr uint32_t kGroup = 4;
+constexpr int kEagerWaves = 1;
+constexpr uint32_t kEagerGroup = 32;
+constexpr int kTableWaves = 1;
 constexpr uint32_t kXcds = 8;
-constexpr uint32_t kGroup = OFI_BOUNCE_GROUP;
 constexpr uint32_t kRows = 8;              /* rows of 64 x 16 bytes per trip: 8 KiB per wave */
 constexpr uint32_t kTripVec = kRows * 64u; /* 16-byte words per trip */
 
