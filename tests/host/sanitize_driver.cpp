@@ -11,6 +11,7 @@
 #include <deque>
 #include <vector>
 
+#include "ofi_amd_rma_abi.h"
 #include "ofi_amd_sendrecv.h"
 #include "oracle.h"
 
@@ -695,6 +696,186 @@ void run_gin_engine(uint64_t seed, uint32_t n_ops)
 	ofi_amd_gin_tx_destroy(b);
 }
 
+/* ------------------------- the ncclRma_v15_t data-path entry points over derivation + engine */
+
+/* what nccl_net_ofi_retval_translate (include/nccl_ofi_api.h:30-75) makes of the codes met here */
+uint64_t g_rma_accepted, g_rma_refused, g_rma_done;
+
+int nccl_code_of(int rc)
+{
+	return rc == 0 ? ncclSuccess : rc == -22 ? ncclInternalError : rc == -90 ? ncclInvalidUsage : ncclSystemError;
+}
+
+void run_rma_abi(uint64_t seed, uint32_t n_ops)
+{
+	rng_t rng{ seed };
+	const uint32_t nranks = 1 + rng.below(6), rails = 1 + rng.below(4), pool = 32 + rng.below(64);
+	const uint64_t min_stripe = rng.chance(50) ? 131072 : 4096, max_small = 64;
+	sim_fabric_t fa, fb;
+	fa.depth = fb.depth = 2 + rng.below(6);
+	fa.fail_every = fb.fail_every = rng.chance(60) ? 0 : 150 + rng.below(300);
+	oracle_gin_fabric_ops_t oa = { oracle_post_cb, oracle_cq_cb, &fa };
+	ofi_amd_gin_fabric_ops_t ob = { product_post_cb, product_cq_cb, &fb };
+	/* oracle side: one initiator state per rank, the scheduler / pin / rail cursor lent from one
+	 * shared state round each derivation, one engine with the reference's 4 x 4 CQ defaults */
+	std::vector<oracle_gin_comm_t> pa(nranks);
+	for (uint32_t r = 0; r < nranks; r++) {
+		oracle_gin_comm_init(&pa[r], r, rails, min_stripe, max_small, 0);
+	}
+	oracle_gin_comm_t sa;
+	oracle_gin_comm_init(&sa, 0, rails, min_stripe, max_small, 0);
+	oracle_gin_tx_t *a = oracle_gin_tx_create(rails, 4, 4, pool, &oa);
+	ofi_amd_rma_ctx_t *ctx = nullptr;
+	SAME("rma ctx create", ofi_amd_rma_ctx_create(nranks, rails, min_stripe, max_small, &ob, pool, 1, &ctx), 0);
+	if (!a) {
+		fail("oracle engine");
+	}
+	/* three registrations: source, destination, signal */
+	oracle_gin_mr_t mra[3][6];
+	ofi_amd_rma_mr_t *mrb[3];
+	for (int h = 0; h < 3; h++) {
+		uint64_t base = 0x10000000ull * (uint64_t)(h + 1), addr[6], off[6], keys[6 * 4];
+		for (uint32_t r = 0; r < nranks; r++) {
+			addr[r] = rng.next() >> 16;
+			off[r] = rng.chance(50) ? 0 : addr[r];
+			mra[h][r].local_base = base;
+			mra[h][r].remote_address = addr[r];
+			mra[h][r].remote_address_offset = off[r];
+			for (int k = 0; k < 4; k++) {
+				keys[r * 4 + k] = mra[h][r].key[k] = rng.next();
+			}
+		}
+		SAME("rma mr create", ofi_amd_rma_mr_create(ctx, base, addr, off, keys, &mrb[h]), 0);
+	}
+	static uint64_t slots[32];
+	SAME("flush buffers", ofi_amd_rma_set_flush_buffers(ctx, slots, 0x5000, 0xdeadbeefdeadbeefull), 0);
+
+	struct open_t {
+		int32_t q;
+		void *req;
+	};
+	std::vector<open_t> open;
+	for (uint32_t i = 0; i < n_ops; i++) {
+		const uint32_t what = rng.below(100);
+		if (what < 38) {
+			const uint32_t rank = rng.below(nranks);
+			/* keep the peer's sequence window open: an ACK for everything sent so far */
+			if (((pa[rank].tx_head - pa[rank].tx_tail) & 0x3FFFu) >= 200 || rng.chance(5)) {
+				const uint32_t consumed = pa[rank].tx_head & 0x3FFFu;
+				oracle_gin_apply_ack(&pa[rank], consumed);
+				SAME("ack rc", ofi_amd_rma_ack_received(ctx, rank, oracle_gin_ack_msg(rank, consumed)), 0);
+			}
+			const uint32_t kind = rng.below(10); /* 0-1 get, 2-4 put, 5-9 put with signal */
+			const bool get = kind < 2, sig = kind >= 5;
+			oracle_gin_desc_t d;
+			std::memset(&d, 0, sizeof(d));
+			d.src_off = rng.below(1u << 24);
+			d.dst_off = rng.below(1u << 24);
+			d.size = rng.chance(10) ? 0 : rng.chance(50) ? rng.below(4096) : rng.below(1u << 22);
+			d.rank = rank;
+			d.opt_flags = rng.below(2);
+			d.src_mr = 0;
+			d.dst_mr = 1;
+			d.sig_mr = 0xffff;
+			d.kind = get ? 3 : 1;
+			if (sig) {
+				d.signal_off = 8 * rng.below(1024);
+				d.signal_value = rng.next();
+				d.signal_op = 1 + rng.below(3); /* 3 is rejected by both */
+				d.sig_mr = 2;
+				d.kind = 2;
+			}
+			if (get && d.size == 0) {
+				d.size = 1;
+			}
+			const oracle_gin_mr_t table[3] = { mra[0][rank], mra[1][rank], mra[2][rank] };
+			oracle_gin_comm_t *peer = &pa[rank];
+			peer->sched = sa.sched;
+			peer->pinned_rail_id = sa.pinned_rail_id;
+			peer->pinned_rail_run = sa.pinned_rail_run;
+			peer->next_rail_id = sa.next_rail_id;
+			oracle_gin_wire_t wa;
+			std::memset(&wa, 0, sizeof(wa));
+			int ra = get ? oracle_gin_iget(peer, table, &d, &wa) : oracle_gin_iput_signal(peer, table, &d, &wa);
+			sa.sched = peer->sched;
+			sa.pinned_rail_id = peer->pinned_rail_id;
+			sa.pinned_rail_run = peer->pinned_rail_run;
+			sa.next_rail_id = peer->next_rail_id;
+			int32_t qa = -1;
+			if (ra == 0) {
+				ra = get ? oracle_gin_tx_iget(a, rank, &wa, &qa) : oracle_gin_tx_iput_signal(a, rank, &wa, &qa);
+			}
+			void *req = &req; /* must be overwritten */
+			int rb;
+			if (get) {
+				rb = ofi_amd_rma_iget(ctx, 0, d.src_off, mrb[0], d.size, d.dst_off, mrb[1], rank, d.opt_flags, &req);
+			} else if (sig) {
+				rb = ofi_amd_rma_iputSignal(ctx, 0, d.src_off, mrb[0], d.size, d.dst_off, mrb[1], rank, d.signal_off,
+							    mrb[2], d.signal_value, d.signal_op, true, d.opt_flags, &req);
+			} else {
+				rb = ofi_amd_rma_iput(ctx, 0, d.src_off, mrb[0], d.size, d.dst_off, mrb[1], rank, d.opt_flags, &req);
+			}
+			SAME("rma op code", nccl_code_of(ra), rb);
+			if (ra == 0) {
+				SAME("rma request", qa, *static_cast<int32_t *>(req));
+				open.push_back({ qa, req });
+				g_rma_accepted++;
+			} else {
+				g_rma_refused++;
+				SAME("rma request cleared", req == nullptr, 1);
+			}
+			SAME("rma peer state", std::memcmp(peer, ofi_amd_rma_peer_state(ctx, rank), sizeof(*peer)), 0);
+			SAME("rma shared state", std::memcmp(&sa, ofi_amd_rma_peer_state(ctx, UINT32_MAX), sizeof(sa)), 0);
+		} else if (what < 41) {
+			int32_t qa = -1;
+			void *req = nullptr;
+			const int ra = oracle_gin_tx_iflush(a, slots, 0x5000, 0xdeadbeefdeadbeefull, &qa);
+			SAME("rma iflush code", nccl_code_of(ra), ofi_amd_rma_iflush(ctx, 0, mrb[1], 0, &req));
+			if (ra == 0) {
+				SAME("rma flush request", qa, *static_cast<int32_t *>(req));
+				for (int r = 0; r < 4; r++) {
+					slots[8 * r] = 0xdeadbeefdeadbeefull; /* the reads land */
+				}
+				open.push_back({ qa, req });
+			}
+		} else if (what < 62) {
+			rng_t r1{ rng.s }, r2{ rng.s };
+			fa.complete_some(r1);
+			fb.complete_some(r2);
+			rng.s = r1.s;
+			SAME("rma progress code", nccl_code_of(oracle_gin_tx_progress(a)), ofi_amd_rma_rmaProgress(ctx));
+		} else if (!open.empty()) {
+			const size_t k = rng.below((uint32_t)open.size());
+			int da = -1, db = -1;
+			SAME("rma test code", nccl_code_of(oracle_gin_tx_test(a, open[k].q, &da)),
+			     ofi_amd_rma_test(ctx, open[k].req, &db));
+			SAME("rma test done", da, db);
+			if (da == 1) {
+				g_rma_done++;
+				/* the request is back in the pool: a second test is refused, nothing posted */
+				SAME("rma test twice", ofi_amd_rma_test(ctx, open[k].req, &db), ncclInternalError);
+				open[k] = open.back();
+				open.pop_back();
+			}
+		}
+		if (fa.log != fb.log) {
+			fail("rma fabric logs differ", i);
+		}
+		fa.log.clear();
+		fb.log.clear();
+		oracle_gin_tx_stats_t sta;
+		ofi_amd_gin_tx_stats_t stb;
+		oracle_gin_tx_stats(a, &sta);
+		SAME("rma stats rc", ofi_amd_rma_tx_stats(ctx, &stb), 0);
+		SAME("rma engine stats", std::memcmp(&sta, &stb, sizeof(sta)), 0);
+	}
+	for (int h = 0; h < 3; h++) {
+		SAME("rma mr destroy", ofi_amd_rma_mr_destroy(mrb[h]), 0);
+	}
+	SAME("rma ctx destroy", ofi_amd_rma_ctx_destroy(ctx), 0);
+	oracle_gin_tx_destroy(a);
+}
+
 } // namespace
 
 int main(int argc, char **argv)
@@ -713,6 +894,13 @@ int main(int argc, char **argv)
 		run_gin_tx(s + 50, 30000, 1);
 		run_gin_engine(s, 20000);
 		run_gin_engine(s + 90, 20000);
+		run_rma_abi(s, 20000);
+		run_rma_abi(s + 70, 20000);
+	}
+	std::printf("rma entry points: %llu operations accepted, %llu refused, %llu tested to completion\n",
+		    (unsigned long long)g_rma_accepted, (unsigned long long)g_rma_refused, (unsigned long long)g_rma_done);
+	if (g_rma_accepted < 1000 * seeds || g_rma_refused == 0 || g_rma_done < 500 * seeds) {
+		fail("the rma program did not exercise the entry points", g_rma_accepted, g_rma_done);
 	}
 	std::printf("host state machines: oracle and product agree over %llu seeds\n", (unsigned long long)seeds);
 	return 0;

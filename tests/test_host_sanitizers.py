@@ -1,5 +1,5 @@
 """The product's plain-C++ host code (message buffer, send/receive state machines, wire codec,
-host scheduler, GIN derivation, transmit engine and receiver) built with AddressSanitizer and UndefinedBehaviorSanitizer and
+host scheduler, GIN derivation, transmit engine and receiver, and the RMA entry points over them) built with AddressSanitizer and UndefinedBehaviorSanitizer and
 run side by side with the oracle on random programs (tests/host/sanitize_driver.cpp), and the
 descriptor rings' host push/pop and proxy threads built with ThreadSanitizer
 (tests/host/tsan_rings_driver.cpp).  CPU only; the GPU sources are not part of these builds."""
@@ -12,7 +12,8 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(ROOT, "aws_ofi_nccl_amd", "csrc")
-HOST_SOURCES = ["sendrecv_proto.cpp", "wire_codec.cpp", "sched_host.cpp", "gin_rx.cpp", "gin_wire.cpp", "gin_tx.cpp"]
+HOST_SOURCES = ["sendrecv_proto.cpp", "wire_codec.cpp", "sched_host.cpp", "gin_rx.cpp", "gin_wire.cpp", "gin_tx.cpp",
+                "rma_abi.cpp"]
 # the sanitizer runtimes are linked statically: a dynamic AddressSanitizer runtime insists on being the
 # first library loaded, which it is not in a process that has other libraries preloaded
 SAN = ["-fsanitize=address,undefined", "-fno-sanitize-recover=all", "-fno-omit-frame-pointer", "-g", "-O1"]
@@ -43,6 +44,8 @@ def test_host_state_machines_clean_under_sanitizers_and_equal_to_the_oracle(driv
                           timeout=300)
     assert proc.returncode == 0, proc.stdout[-4000:]
     assert "agree over 6 seeds" in proc.stdout
+    assert "rma entry points:" in proc.stdout
+    print(proc.stdout[-400:])
 
 
 def test_ring_push_pop_and_proxy_threads_clean_under_thread_sanitizer(tmp_path):
