@@ -771,6 +771,8 @@ def main():
                      "kernel": "bounce_scatter_kernel", "kernel_ms": bounce["ms_kernel_median"],
                      "kernel_ms_median": bounce["ms_kernel_median"], "kernel_ms_min": bounce["ms_kernel_min"],
                      "kernel_ms_back_to_back": bounce["ms_kernel"],
+                     # what a pair of events reads with nothing between them: the resolution of kernel_ms
+                     "event_pair_empty_ms": per_launch_ms(lambda: None, 200, torch)[0],
                      "sustained": bounce["sustained"],
                      "sustained_device_copy": bounce.get("sustained_device_copy"),
                      "algorithmic_bytes_per_launch": bounce["algo_bytes"],
