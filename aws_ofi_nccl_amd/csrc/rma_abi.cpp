@@ -9,6 +9,7 @@
  */
 #include <cerrno>
 #include <chrono>
+#include <cstdint>
 #include <cstring>
 #include <new>
 #include <vector>
@@ -347,14 +348,20 @@ ncclResult_t ofi_amd_rma_test(void *collComm, void *request, int *done)
 	if (!ctx || !request || !done || ctx->request_slot.empty()) {
 		return ncclInternalError;
 	}
-	const int32_t *slot = static_cast<const int32_t *>(request);
-	if (slot < ctx->request_slot.data() || slot >= ctx->request_slot.data() + ctx->request_slot.size() ||
-	    *slot != (int32_t)(slot - ctx->request_slot.data())) {
-		return ncclInternalError; /* not a request of this context, or one already completed */
+	/* a request is the address of an entry of request_slot: anything else (another context's,
+	 * a stray pointer, an address inside an entry) is refused before it is read */
+	const uintptr_t first = reinterpret_cast<uintptr_t>(ctx->request_slot.data());
+	const uintptr_t at = reinterpret_cast<uintptr_t>(request);
+	if (at < first || at - first >= ctx->request_slot.size() * sizeof(int32_t) || (at - first) % sizeof(int32_t) != 0) {
+		return ncclInternalError;
 	}
-	const int rc = ofi_amd_gin_tx_test(ctx->tx, *slot, done);
+	const size_t index = (at - first) / sizeof(int32_t);
+	if (ctx->request_slot[index] != (int32_t)index) {
+		return ncclInternalError; /* already completed */
+	}
+	const int rc = ofi_amd_gin_tx_test(ctx->tx, (int32_t)index, done);
 	if (rc == 0 && *done) {
-		ctx->request_slot[(size_t)(slot - ctx->request_slot.data())] = -1;
+		ctx->request_slot[index] = -1;
 	}
 	return translate(rc);
 }

@@ -80,7 +80,10 @@ int ofi_amd_rma_set_flush_buffers(ofi_amd_rma_ctx_t *ctx, void *host_slots, uint
 				  uint64_t sentinel);
 
 /* An ACK message from peer `rank` has arrived (handle_ack_completion,
- * src/rdma/gin/nccl_ofi_gin.cpp:1843-1869): ack_msg is the 8-byte gin_ack_msg_t. */
+ * src/rdma/gin/nccl_ofi_gin.cpp:1843-1869): ack_msg is the 8-byte gin_ack_msg_t.  In the reference
+ * that is a receive completion handled inside a progress call; here the owner of the fabric calls
+ * this when it sees one, and may do so from inside its cq_read callback -- which is how the
+ * window opens for an iput / iputSignal that is waiting in its progress loop. */
 int ofi_amd_rma_ack_received(ofi_amd_rma_ctx_t *ctx, uint32_t rank, uint64_t ack_msg);
 
 /* The initiator state towards one peer (sequence numbers, window, ACK requests: per rank as in

@@ -277,3 +277,54 @@ def test_return_codes_follow_the_reference_translation(lib):
     assert put(1) == 0
     assert lib.ofi_amd_rma_peer_state(ini.ctx, 1).contents.tx_tail == 4096
     ini.close()
+
+
+def test_a_full_window_opens_when_the_ack_arrives_inside_a_progress_call(lib):
+    """await_tx_window (src/rdma/gin/nccl_ofi_gin.cpp:518-537): a put towards a rank whose window is
+    full keeps calling progress; the ACK that makes room is a receive completion handled inside that
+    progress call (handle_ack_completion, :1843-1869).  Here the CQ callback plays it: on its third
+    call during the wait it hands the ACK to ofi_amd_rma_ack_received, and the put that was waiting
+    goes through with the next sequence number (its post queues up behind those the full send
+    queues have refused so far)."""
+    ini = Initiator.__new__(Initiator)
+    ini.lib = lib
+    ini.fab = ctypes.c_void_p()
+    assert lib.ofi_amd_loopfab_create(4, 512, ctypes.byref(ini.fab)) == 0
+    inner = m.GinFabricOps()
+    assert lib.ofi_amd_loopfab_ops(ini.fab, ctypes.byref(inner)) == 0
+    state = {"armed": False, "calls": 0, "ctx": None}
+
+    def cq_read(fabric, rail, contexts, cap):
+        if state["armed"]:
+            state["calls"] += 1
+            if state["calls"] == 3:
+                state["armed"] = False
+                assert lib.ofi_amd_rma_ack_received(state["ctx"], 1, int(lib.ofi_amd_gin_ack_msg(1, 100))) == 0
+        return inner.cq_read(fabric, rail, contexts, cap)
+
+    ini.ops = m.GinFabricOps(inner.post, m.FABRIC_CQ_READ_FN(cq_read), inner.fabric)
+    ini.ctx = ctypes.c_void_p()
+    assert lib.ofi_amd_rma_ctx_create(NRANKS, 4, 131072, 64, ctypes.byref(ini.ops), 40000, 5000,
+                                      ctypes.byref(ini.ctx)) == 0
+    state["ctx"] = ini.ctx
+    ini.mrs, ini.tables, ini.posts = [], [], (m.GinPost * 64)()
+    for i in range(3):
+        base, addr, off, keys = mr_arrays(i)
+        h = ctypes.c_void_p()
+        assert lib.ofi_amd_rma_mr_create(ini.ctx, base, addr.ctypes.data, off.ctypes.data, keys.ctypes.data,
+                                         ctypes.byref(h)) == 0
+        ini.mrs.append(h)
+    req = ctypes.c_void_p()
+    put = lambda: lib.ofi_amd_rma_iput(ini.ctx, 0, 0, ini.mrs[0], 8, 0, ini.mrs[1], 1, 0, ctypes.byref(req))
+    for i in range(8192):
+        assert put() == 0
+        if i % 256 == 0:
+            ini.wire()
+            assert lib.ofi_amd_rma_rmaProgress(ini.ctx) == 0
+    ini.wire()
+    state["armed"] = True
+    assert put() == ncclSuccess and req.value         # waited through two progress calls, then went
+    assert state["calls"] >= 3 and not state["armed"]
+    peer = lib.ofi_amd_rma_peer_state(ini.ctx, 1).contents
+    assert peer.tx_tail == 100 and peer.tx_head == 8193
+    ini.close()
