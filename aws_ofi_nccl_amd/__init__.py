@@ -372,6 +372,21 @@ PROTOTYPES = {
     "ofi_amd_rma_iget": (ctypes.c_int, [c_vp, ctypes.c_int, c_u64, c_vp, ctypes.c_size_t, c_u64, c_vp, c_u32, c_u32,
                                         ctypes.POINTER(c_vp)]),
     "ofi_amd_rma_iflush": (ctypes.c_int, [c_vp, ctypes.c_int, c_vp, c_u32, ctypes.POINTER(c_vp)]),
+    # the same operations as the older op-tables spell them (no optFlags; v13 / v11 no isStrongSignal;
+    # v11 no context number)
+    "ofi_amd_rma_iput_v14": (ctypes.c_int, [c_vp, ctypes.c_int, c_u64, c_vp, ctypes.c_size_t, c_u64, c_vp, c_u32,
+                                            ctypes.POINTER(c_vp)]),
+    "ofi_amd_rma_iputSignal_v14": (ctypes.c_int, [c_vp, ctypes.c_int, c_u64, c_vp, ctypes.c_size_t, c_u64, c_vp,
+                                                  c_u32, c_u64, c_vp, c_u64, c_u32, ctypes.c_bool,
+                                                  ctypes.POINTER(c_vp)]),
+    "ofi_amd_rma_iget_v14": (ctypes.c_int, [c_vp, ctypes.c_int, c_u64, c_vp, ctypes.c_size_t, c_u64, c_vp, c_u32,
+                                            ctypes.POINTER(c_vp)]),
+    "ofi_amd_gin_iputSignal_v13": (ctypes.c_int, [c_vp, ctypes.c_int, c_u64, c_vp, ctypes.c_size_t, c_u64, c_vp,
+                                                  c_u32, c_u64, c_vp, c_u64, c_u32, ctypes.POINTER(c_vp)]),
+    "ofi_amd_gin_iput_v11": (ctypes.c_int, [c_vp, c_u64, c_vp, ctypes.c_size_t, c_u64, c_vp, c_u32,
+                                            ctypes.POINTER(c_vp)]),
+    "ofi_amd_gin_iputSignal_v11": (ctypes.c_int, [c_vp, c_u64, c_vp, ctypes.c_size_t, c_u64, c_vp, c_u32, c_u64, c_vp,
+                                                  c_u64, c_u32, ctypes.POINTER(c_vp)]),
     "ofi_amd_rma_test": (ctypes.c_int, [c_vp, c_vp, ctypes.POINTER(ctypes.c_int)]),
     "ofi_amd_rma_rmaProgress": (ctypes.c_int, [c_vp]),
     "ofi_amd_loopfab_create": (ctypes.c_int, [c_u32, c_u32, ctypes.POINTER(c_vp)]),

@@ -1,5 +1,6 @@
 /*
- * The data-path members of ncclRma_v15_t (3rd-party/nccl/cuda/include/nccl/rma_v15.h:43-56)
+ * The data-path members of ncclRma_v15_t (3rd-party/nccl/cuda/include/nccl/rma_v15.h:43-56),
+ * and of the older ncclRma_v14_t / ncclGin_v13_t / ncclGin_v11_t the reference also exports,
  * as free functions over this library's derivation (gin_wire.cpp) and transmit engine
  * (gin_tx.cpp).  Each packs its arguments into the 64-byte descriptor the device-side put
  * would have written, resolves the caller's registration handles for the target rank,
@@ -370,6 +371,51 @@ ncclResult_t ofi_amd_rma_rmaProgress(void *rmaCtx)
 {
 	ofi_amd_rma_ctx_t *ctx = static_cast<ofi_amd_rma_ctx_t *>(rmaCtx);
 	return ctx ? translate(ofi_amd_gin_tx_progress(ctx->tx)) : ncclInternalError;
+}
+
+/* The older op-tables: no optFlags (0, as the reference's wrappers forward,
+ * src/rdma/gin/nccl_ofi_gin_api.cpp:505-564, 651-663). */
+ncclResult_t ofi_amd_rma_iput_v14(void *rmaCtx, int context, uint64_t srcOff, void *srcMhandle, size_t size,
+				  uint64_t dstOff, void *dstMhandle, uint32_t rank, void **request)
+{
+	return ofi_amd_rma_iput(rmaCtx, context, srcOff, srcMhandle, size, dstOff, dstMhandle, rank, 0, request);
+}
+
+ncclResult_t ofi_amd_rma_iputSignal_v14(void *rmaCtx, int context, uint64_t srcOff, void *srcMhandle, size_t size,
+					uint64_t dstOff, void *dstMhandle, uint32_t rank, uint64_t signalOff,
+					void *signalMhandle, uint64_t signalValue, uint32_t signalOp,
+					bool isStrongSignal, void **request)
+{
+	return ofi_amd_rma_iputSignal(rmaCtx, context, srcOff, srcMhandle, size, dstOff, dstMhandle, rank, signalOff,
+				      signalMhandle, signalValue, signalOp, isStrongSignal, 0, request);
+}
+
+ncclResult_t ofi_amd_rma_iget_v14(void *rmaCtx, int context, uint64_t remoteOff, void *remoteMhandle, size_t size,
+				  uint64_t localOff, void *localMhandle, uint32_t rank, void **request)
+{
+	return ofi_amd_rma_iget(rmaCtx, context, remoteOff, remoteMhandle, size, localOff, localMhandle, rank, 0, request);
+}
+
+ncclResult_t ofi_amd_gin_iputSignal_v13(void *ginCtx, int context, uint64_t srcOff, void *srcMhandle, size_t size,
+					uint64_t dstOff, void *dstMhandle, uint32_t rank, uint64_t signalOff,
+					void *signalMhandle, uint64_t signalValue, uint32_t signalOp, void **request)
+{
+	return ofi_amd_rma_iputSignal(ginCtx, context, srcOff, srcMhandle, size, dstOff, dstMhandle, rank, signalOff,
+				      signalMhandle, signalValue, signalOp, true, 0, request);
+}
+
+ncclResult_t ofi_amd_gin_iput_v11(void *collComm, uint64_t srcOff, void *srcMhandle, size_t size, uint64_t dstOff,
+				  void *dstMhandle, uint32_t rank, void **request)
+{
+	return ofi_amd_rma_iput(collComm, 0, srcOff, srcMhandle, size, dstOff, dstMhandle, rank, 0, request);
+}
+
+ncclResult_t ofi_amd_gin_iputSignal_v11(void *collComm, uint64_t srcOff, void *srcMhandle, size_t size,
+					uint64_t dstOff, void *dstMhandle, uint32_t rank, uint64_t signalOff,
+					void *signalMhandle, uint64_t signalValue, uint32_t signalOp, void **request)
+{
+	return ofi_amd_rma_iputSignal(collComm, 0, srcOff, srcMhandle, size, dstOff, dstMhandle, rank, signalOff,
+				      signalMhandle, signalValue, signalOp, true, 0, request);
 }
 
 } /* extern "C" */

@@ -121,6 +121,35 @@ ncclResult_t ofi_amd_rma_test(void *collComm, void *request, int *done);
 /* nccl_ofi_gin_ginProgress, :284-296: bounded CQ drain on every rail, then the pending posts */
 ncclResult_t ofi_amd_rma_rmaProgress(void *rmaCtx);
 
+/* ---- the same data path behind the older op-tables the reference also exports ----
+ *
+ * ncclRma_v14_t (rma_v14.h:49-57), ncclGin_v13_t (gin_v13.h:48-57) and ncclGin_v11_t
+ * (net_v11.h:222-227) carry the same operations without optFlags (the reference's wrappers
+ * forward 0, src/rdma/gin/nccl_ofi_gin_api.cpp:505-564, 651-663), v13 and v11 without
+ * isStrongSignal, v11 without the context number and without iget / iflush.  iflush, test and
+ * the progress call have one signature in all of them: ofi_amd_rma_iflush, ofi_amd_rma_test and
+ * ofi_amd_rma_rmaProgress serve every table (ginProgress in the GIN ones). */
+ncclResult_t ofi_amd_rma_iput_v14(void *rmaCtx, int context, uint64_t srcOff, void *srcMhandle, size_t size,
+				  uint64_t dstOff, void *dstMhandle, uint32_t rank, void **request);
+ncclResult_t ofi_amd_rma_iputSignal_v14(void *rmaCtx, int context, uint64_t srcOff, void *srcMhandle, size_t size,
+					uint64_t dstOff, void *dstMhandle, uint32_t rank, uint64_t signalOff,
+					void *signalMhandle, uint64_t signalValue, uint32_t signalOp,
+					bool isStrongSignal, void **request);
+ncclResult_t ofi_amd_rma_iget_v14(void *rmaCtx, int context, uint64_t remoteOff, void *remoteMhandle, size_t size,
+				  uint64_t localOff, void *localMhandle, uint32_t rank, void **request);
+/* ncclGin_v13_t: iput and iget as in ncclRma_v14_t (the reference uses one pair of wrappers for
+ * both tables, :680-682); iputSignal without isStrongSignal */
+ncclResult_t ofi_amd_gin_iputSignal_v13(void *ginCtx, int context, uint64_t srcOff, void *srcMhandle, size_t size,
+					uint64_t dstOff, void *dstMhandle, uint32_t rank, uint64_t signalOff,
+					void *signalMhandle, uint64_t signalValue, uint32_t signalOp, void **request);
+/* ncclGin_v11_t: the first argument is the collective comm, which is also the context there
+ * (createContext returns ginCtx = collComm, :481-498) */
+ncclResult_t ofi_amd_gin_iput_v11(void *collComm, uint64_t srcOff, void *srcMhandle, size_t size, uint64_t dstOff,
+				  void *dstMhandle, uint32_t rank, void **request);
+ncclResult_t ofi_amd_gin_iputSignal_v11(void *collComm, uint64_t srcOff, void *srcMhandle, size_t size,
+					uint64_t dstOff, void *dstMhandle, uint32_t rank, uint64_t signalOff,
+					void *signalMhandle, uint64_t signalValue, uint32_t signalOp, void **request);
+
 #ifdef __cplusplus
 }
 #endif

@@ -80,6 +80,45 @@ static ncclRma_v15_t rma_table_with_this_librarys_data_path()
 	return t;
 }
 
+/* ... and the older tables the reference exports beside it (ncclRmaPlugin_v14, ncclGinPlugin_v13,
+ * ncclGinPlugin_v11: src/rdma/gin/nccl_ofi_gin_api.cpp:566-617, 666-688) */
+#include "nccl/rma_v14.h"
+#include "nccl/gin_v13.h"
+
+static ncclRma_v14_t rma_v14_table_with_this_librarys_data_path()
+{
+	ncclRma_v14_t t = {};
+	t.iput = ofi_amd_rma_iput_v14;
+	t.iputSignal = ofi_amd_rma_iputSignal_v14;
+	t.iget = ofi_amd_rma_iget_v14;
+	t.iflush = ofi_amd_rma_iflush;
+	t.test = ofi_amd_rma_test;
+	t.rmaProgress = ofi_amd_rma_rmaProgress;
+	return t;
+}
+
+static ncclGin_v13_t gin_v13_table_with_this_librarys_data_path()
+{
+	ncclGin_v13_t t = {};
+	t.iput = ofi_amd_rma_iput_v14;
+	t.iputSignal = ofi_amd_gin_iputSignal_v13;
+	t.iget = ofi_amd_rma_iget_v14;
+	t.iflush = ofi_amd_rma_iflush;
+	t.test = ofi_amd_rma_test;
+	t.ginProgress = ofi_amd_rma_rmaProgress;
+	return t;
+}
+
+static ncclGin_v11_t gin_v11_table_with_this_librarys_data_path()
+{
+	ncclGin_v11_t t = {};
+	t.iput = ofi_amd_gin_iput_v11;
+	t.iputSignal = ofi_amd_gin_iputSignal_v11;
+	t.test = ofi_amd_rma_test;
+	t.ginProgress = ofi_amd_rma_rmaProgress;
+	return t;
+}
+
 #define CHECK(cond)                                                                       \
 	do {                                                                              \
 		if (!(cond)) {                                                            \
@@ -118,6 +157,28 @@ static int link_checks()
 		CHECK(table.rmaProgress(rma) == ncclSuccess);
 		CHECK(table.test(rma, request, &done) == ncclSuccess && done == 1);
 		CHECK(table.iput(rma, 0, 0, mr, 8, 0, mr, 7, 0, &request) == ncclInternalError); /* no such rank */
+		/* the older tables reach the same context: one put-signal through each, the sequence
+		 * number in the immediate data counts on (GIN_IMM_SEQ, bits 11..23) */
+		const ncclRma_v14_t t14 = rma_v14_table_with_this_librarys_data_path();
+		const ncclGin_v13_t t13 = gin_v13_table_with_this_librarys_data_path();
+		const ncclGin_v11_t t11 = gin_v11_table_with_this_librarys_data_path();
+		void *r14 = nullptr, *r13 = nullptr, *r11 = nullptr;
+		CHECK(t14.iputSignal(rma, 0, 0, mr, 5000, 0, mr, 1, 8, mr, 1, 1, true, &r14) == ncclSuccess && r14);
+		CHECK(t13.iputSignal(rma, 0, 0, mr, 5000, 0, mr, 1, 8, mr, 1, 1, &r13) == ncclSuccess && r13);
+		CHECK(t11.iputSignal(rma, 0, mr, 5000, 0, mr, 1, 8, mr, 1, 1, &r11) == ncclSuccess && r11);
+		ofi_amd_gin_post_t later[8];
+		CHECK(ofi_amd_loopfab_take_transmitted(fab, later, 8) == 6); /* a write and a metadata message each */
+		for (int k = 0; k < 3; k++) {
+			CHECK(later[2 * k].kind == OFI_AMD_GIN_POST_WRITE && later[2 * k + 1].kind == OFI_AMD_GIN_POST_META);
+			CHECK(((later[2 * k].imm >> 11) & 0x1fffu) == 1u + (uint32_t)k);
+		}
+		CHECK(t13.ginProgress(rma) == ncclSuccess);
+		CHECK(t14.test(rma, r14, &done) == ncclSuccess && done == 1);
+		CHECK(t13.test(rma, r13, &done) == ncclSuccess && done == 1);
+		CHECK(t11.test(rma, r11, &done) == ncclSuccess && done == 1);
+		void *g = nullptr;
+		CHECK(t13.iget(rma, 0, 0, mr, 64, 0, mr, 1, &g) == ncclSuccess && g);
+		CHECK(t11.iput(rma, 0, mr, 8, 0, mr, 1, &g) == ncclSuccess && g);
 		CHECK(ofi_amd_rma_mr_destroy(mr) == 0 && ofi_amd_rma_ctx_destroy(rma) == 0 && ofi_amd_loopfab_destroy(fab) == 0);
 	}
 	const int init = nccl_net_ofi_gpu_init();

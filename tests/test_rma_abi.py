@@ -328,3 +328,45 @@ def test_a_full_window_opens_when_the_ack_arrives_inside_a_progress_call(lib):
     peer = lib.ofi_amd_rma_peer_state(ini.ctx, 1).contents
     assert peer.tx_tail == 100 and peer.tx_head == 8193
     ini.close()
+
+
+def test_the_older_op_tables_spell_the_same_operations(lib):
+    """ncclRma_v14_t, ncclGin_v13_t and ncclGin_v11_t (rma_v14.h:49-57, gin_v13.h:48-57, net_v11.h:222-227)
+    carry no optFlags, v13 and v11 no isStrongSignal, v11 no context number: the reference's wrappers
+    forward optFlags 0 (src/rdma/gin/nccl_ofi_gin_api.cpp:505-564, 651-663).  Two contexts are given the
+    same operations, one through the v15 entry points with optFlags 0, one through the older spellings:
+    the posts on the wire are the same, and so is the state towards the peer."""
+    a, b = Initiator(lib), Initiator(lib)
+    req = ctypes.c_void_p()
+    sizes = [0, 8, 5000, 200000, 4 << 20]
+    for k, size in enumerate(sizes * 3):
+        which = k // len(sizes)
+        common = (0, ) if which < 2 else ()
+        if size:
+            assert lib.ofi_amd_rma_iput(a.ctx, 0, 16, a.mrs[0], size, 32, a.mrs[1], 1, 0, ctypes.byref(req)) == 0
+            fn = lib.ofi_amd_rma_iput_v14 if which < 2 else lib.ofi_amd_gin_iput_v11
+            assert fn(b.ctx, *common, 16, b.mrs[0], size, 32, b.mrs[1], 1, ctypes.byref(req)) == 0 and req.value
+            assert lib.ofi_amd_rma_iget(a.ctx, 0, 16, a.mrs[1], size, 32, a.mrs[0], 1, 0, ctypes.byref(req)) == 0
+            assert lib.ofi_amd_rma_iget_v14(b.ctx, 0, 16, b.mrs[1], size, 32, b.mrs[0], 1, ctypes.byref(req)) == 0
+        assert lib.ofi_amd_rma_iputSignal(a.ctx, 0, 16, a.mrs[0], size, 32, a.mrs[1], 1, 8 * k, a.mrs[2], 3 + k,
+                                          SIGNAL_ADD, True, 0, ctypes.byref(req)) == 0
+        if which == 0:
+            rc = lib.ofi_amd_rma_iputSignal_v14(b.ctx, 0, 16, b.mrs[0], size, 32, b.mrs[1], 1, 8 * k, b.mrs[2], 3 + k,
+                                                SIGNAL_ADD, False, ctypes.byref(req))
+        elif which == 1:
+            rc = lib.ofi_amd_gin_iputSignal_v13(b.ctx, 0, 16, b.mrs[0], size, 32, b.mrs[1], 1, 8 * k, b.mrs[2], 3 + k,
+                                                SIGNAL_ADD, ctypes.byref(req))
+        else:
+            rc = lib.ofi_amd_gin_iputSignal_v11(b.ctx, 16, b.mrs[0], size, 32, b.mrs[1], 1, 8 * k, b.mrs[2], 3 + k,
+                                                SIGNAL_ADD, ctypes.byref(req))
+        assert rc == 0 and req.value
+        assert a.wire() == b.wire()
+    pa, pb = lib.ofi_amd_rma_peer_state(a.ctx, 1).contents, lib.ofi_amd_rma_peer_state(b.ctx, 1).contents
+    assert bytes(pa) == bytes(pb) and pa.tx_head == 15 + 12
+    # the same argument checks behind every spelling
+    assert lib.ofi_amd_gin_iput_v11(b.ctx, 0, b.mrs[0], 8, 0, b.mrs[1], NRANKS, ctypes.byref(req)) == ncclInternalError
+    assert req.value is None
+    assert lib.ofi_amd_gin_iputSignal_v13(b.ctx, 0, 0, b.mrs[0], 8, 0, b.mrs[1], 1, 0, b.mrs[2], 1, 3,
+                                          ctypes.byref(req)) == ncclInternalError
+    a.close()
+    b.close()
