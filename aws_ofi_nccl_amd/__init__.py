@@ -195,6 +195,13 @@ class RecvState(ctypes.Structure):
                 ("pad2", c_u32), ("n_ctrl_sent", c_u64)]
 
 
+class NetLinkStats(ctypes.Structure):
+    """ofi_amd_net_link_stats_t"""
+    _fields_ = [(k, c_u64) for k in ("isend_calls", "isend_again", "eager_sends", "write_sends", "rdma_writes",
+                                     "payload_bytes", "irecv_calls", "flushes", "launches", "copy_entries",
+                                     "eager_copies", "progress_calls")]
+
+
 class SendrecvLoopbackStats(ctypes.Structure):
     """ofi_amd_sendrecv_loopback_stats_t"""
     _fields_ = [("messages", c_u64), ("payload_bytes", c_u64), ("eager_messages", c_u64),
@@ -389,6 +396,26 @@ PROTOTYPES = {
                                                   c_u64, c_u32, ctypes.POINTER(c_vp)]),
     "ofi_amd_rma_test": (ctypes.c_int, [c_vp, c_vp, ctypes.POINTER(ctypes.c_int)]),
     "ofi_amd_rma_rmaProgress": (ctypes.c_int, [c_vp]),
+    # include/ofi_amd_net_abi.h: an in-process link, then the data-path members of ncclNet_vN_t
+    "ofi_amd_net_link_create": (ctypes.c_int, [c_u32, ctypes.c_int64, c_u64, c_u64, c_u32, c_vp, ctypes.POINTER(c_vp)]),
+    "ofi_amd_net_link_destroy": (ctypes.c_int, [c_vp]),
+    "ofi_amd_net_link_send_comm": (c_vp, [c_vp]),
+    "ofi_amd_net_link_recv_comm": (c_vp, [c_vp]),
+    "ofi_amd_net_link_stats": (ctypes.c_int, [c_vp, ctypes.POINTER(NetLinkStats)]),
+    "ofi_amd_net_link_state": (ctypes.c_int, [c_vp, ctypes.POINTER(SendState), ctypes.POINTER(RecvState)]),
+    "ofi_amd_net_isend": (ctypes.c_int, [c_vp, c_vp, ctypes.c_size_t, ctypes.c_int, c_vp, c_vp, ctypes.POINTER(c_vp)]),
+    "ofi_amd_net_irecv": (ctypes.c_int, [c_vp, ctypes.c_int, ctypes.POINTER(c_vp), ctypes.POINTER(ctypes.c_size_t),
+                                         ctypes.POINTER(ctypes.c_int), ctypes.POINTER(c_vp), ctypes.POINTER(c_vp),
+                                         ctypes.POINTER(c_vp)]),
+    "ofi_amd_net_iflush": (ctypes.c_int, [c_vp, ctypes.c_int, ctypes.POINTER(c_vp), ctypes.POINTER(ctypes.c_int),
+                                          ctypes.POINTER(c_vp), ctypes.POINTER(c_vp)]),
+    "ofi_amd_net_test": (ctypes.c_int, [c_vp, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]),
+    "ofi_amd_net_isend_v5": (ctypes.c_int, [c_vp, c_vp, ctypes.c_int, ctypes.c_int, c_vp, ctypes.POINTER(c_vp)]),
+    "ofi_amd_net_irecv_v5": (ctypes.c_int, [c_vp, ctypes.c_int, ctypes.POINTER(c_vp), ctypes.POINTER(ctypes.c_int),
+                                            ctypes.POINTER(ctypes.c_int), ctypes.POINTER(c_vp), ctypes.POINTER(c_vp)]),
+    "ofi_amd_net_isend_v9": (ctypes.c_int, [c_vp, c_vp, ctypes.c_size_t, ctypes.c_int, c_vp, ctypes.POINTER(c_vp)]),
+    "ofi_amd_net_irecv_v9": (ctypes.c_int, [c_vp, ctypes.c_int, ctypes.POINTER(c_vp), ctypes.POINTER(ctypes.c_size_t),
+                                            ctypes.POINTER(ctypes.c_int), ctypes.POINTER(c_vp), ctypes.POINTER(c_vp)]),
     "ofi_amd_loopfab_create": (ctypes.c_int, [c_u32, c_u32, ctypes.POINTER(c_vp)]),
     "ofi_amd_loopfab_destroy": (ctypes.c_int, [c_vp]),
     "ofi_amd_loopfab_ops": (ctypes.c_int, [c_vp, ctypes.POINTER(GinFabricOps)]),

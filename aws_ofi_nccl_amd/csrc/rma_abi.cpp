@@ -15,6 +15,7 @@
 #include <new>
 #include <vector>
 
+#include "nccl_translate.hpp"
 #include "ofi_amd_rma_abi.h"
 
 struct ofi_amd_rma_mr {
@@ -44,26 +45,9 @@ struct ofi_amd_rma_ctx {
 
 namespace {
 
-/* nccl_net_ofi_retval_translate, include/nccl_ofi_api.h:30-75 */
 ncclResult_t translate(int rc)
 {
-	switch (rc) {
-	case 0:
-		return ncclSuccess;
-	case -EINVAL:
-		return ncclInternalError; /* "invalid arguments to plugin calls should return ncclInternalError" */
-	case -EMSGSIZE:
-		return ncclInvalidUsage;
-	case -ECONNABORTED:
-	case -ECONNRESET:
-	case -ECONNREFUSED:
-	case -ENOTCONN:
-	case -EHOSTDOWN:
-	case -EHOSTUNREACH:
-		return ncclRemoteError;
-	default:
-		return ncclSystemError;
-	}
+	return ofi_amd::nccl_result_of(rc);
 }
 
 const ofi_amd_gin_mr_t kNoMr = {0, 0, 0, {0, 0, 0, 0}};

@@ -24,22 +24,10 @@
 #include <stdint.h>
 
 #include "ofi_amd_hotpath.h"
+#include "ofi_amd_nccl_err.h"
 
 #ifdef __cplusplus
 extern "C" {
-#endif
-
-/* ncclResult_t as NCCL's plugin headers define it (nccl/err.h:9-16), under the same include guard,
- * so that this header and NCCL's can be included together in either order. */
-#ifndef NCCL_ERR_H_
-#define NCCL_ERR_H_
-typedef enum { ncclSuccess                 =  0,
-               ncclUnhandledCudaError      =  1,
-               ncclSystemError             =  2,
-               ncclInternalError           =  3,
-               ncclInvalidArgument         =  4,
-               ncclInvalidUsage            =  5,
-               ncclRemoteError             =  6 } ncclResult_t;
 #endif
 
 /* ---- set-up: what createContext / regMrSym hand over (no counterpart signature in the table) ---- */

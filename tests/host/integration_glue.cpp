@@ -119,6 +119,51 @@ static ncclGin_v11_t gin_v11_table_with_this_librarys_data_path()
 	return t;
 }
 
+/* The data-path members of the reference's ncclNet tables (ncclNetPlugin_v6 .. v12,
+ * src/nccl_ofi_interface_nvidia.cpp:661-825): the three spellings the reference's shims cover */
+#include "ofi_amd_net_abi.h"
+
+static ncclNet_v12_t net_v12_table_with_this_librarys_data_path()
+{
+	ncclNet_v12_t t = {};
+	t.name = "Libfabric";
+	t.isend = ofi_amd_net_isend;
+	t.irecv = ofi_amd_net_irecv;
+	t.iflush = ofi_amd_net_iflush;
+	t.test = ofi_amd_net_test;
+	return t;
+}
+
+template <typename Table> static Table net_table_v10_or_v11()
+{
+	Table t = {};
+	t.isend = ofi_amd_net_isend;
+	t.irecv = ofi_amd_net_irecv;
+	t.iflush = ofi_amd_net_iflush;
+	t.test = ofi_amd_net_test;
+	return t;
+}
+
+static ncclNet_v9_t net_v9_table_with_this_librarys_data_path()
+{
+	ncclNet_v9_t t = {};
+	t.isend = ofi_amd_net_isend_v9;
+	t.irecv = ofi_amd_net_irecv_v9;
+	t.iflush = ofi_amd_net_iflush;
+	t.test = ofi_amd_net_test;
+	return t;
+}
+
+template <typename Table> static Table net_table_v6_to_v8()
+{
+	Table t = {};
+	t.isend = ofi_amd_net_isend_v5;
+	t.irecv = ofi_amd_net_irecv_v5;
+	t.iflush = ofi_amd_net_iflush;
+	t.test = ofi_amd_net_test;
+	return t;
+}
+
 #define CHECK(cond)                                                                       \
 	do {                                                                              \
 		if (!(cond)) {                                                            \
@@ -180,6 +225,24 @@ static int link_checks()
 		CHECK(t13.iget(rma, 0, 0, mr, 64, 0, mr, 1, &g) == ncclSuccess && g);
 		CHECK(t11.iput(rma, 0, mr, 8, 0, mr, 1, &g) == ncclSuccess && g);
 		CHECK(ofi_amd_rma_mr_destroy(mr) == 0 && ofi_amd_rma_ctx_destroy(rma) == 0 && ofi_amd_loopfab_destroy(fab) == 0);
+	}
+	{ /* every net table takes the functions; without a comm they answer as the reference's checks do */
+		const ncclNet_v12_t n12 = net_v12_table_with_this_librarys_data_path();
+		const ncclNet_v11_t n11 = net_table_v10_or_v11<ncclNet_v11_t>();
+		const ncclNet_v10_t n10 = net_table_v10_or_v11<ncclNet_v10_t>();
+		const ncclNet_v9_t n9 = net_v9_table_with_this_librarys_data_path();
+		const ncclNet_v8_t n8 = net_table_v6_to_v8<ncclNet_v8_t>();
+		const ncclNet_v7_t n7 = net_table_v6_to_v8<ncclNet_v7_t>();
+		const ncclNet_v6_t n6 = net_table_v6_to_v8<ncclNet_v6_t>();
+		void *request = &request;
+		int done = 0;
+		CHECK(n12.isend(nullptr, nullptr, 8, 1, nullptr, nullptr, &request) == ncclInternalError && !request);
+		CHECK(n11.test(nullptr, &done, nullptr) == ncclInternalError);
+		CHECK(n10.iflush(nullptr, 1, nullptr, nullptr, nullptr, &request) == ncclInternalError);
+		CHECK(n9.isend(nullptr, nullptr, 8, 1, nullptr, &request) == ncclInternalError);
+		CHECK(n8.irecv(nullptr, 1, nullptr, nullptr, nullptr, nullptr, &request) == ncclInvalidArgument);
+		CHECK(n7.isend(nullptr, nullptr, 8, 1, nullptr, &request) == ncclInternalError);
+		CHECK(n6.test(nullptr, &done, nullptr) == ncclInternalError);
 	}
 	const int init = nccl_net_ofi_gpu_init();
 	if (init == -ENODEV) {
@@ -273,6 +336,52 @@ static int gpu_checks()
 			CHECK(nccl_net_ofi_gpu_get_dma_buf_fd(ptr, 1u << 20, &fd, &off) == 0 && fd >= 0 && off == 0);
 		}
 		CHECK(nccl_net_ofi_gpu_mem_free(ptr) == 0);
+	}
+	{ /* one eager and one rendezvous message through the v12 table's pointers: post_send /
+	   * post_recv / poll as in tests/functional/functional_test.cpp:242-294, 592-640 */
+		const ncclNet_v12_t net = net_v12_table_with_this_librarys_data_path();
+		ofi_amd_net_link_t *link = nullptr;
+		CHECK(ofi_amd_net_link_create(4, 8192, 0, 0, 0, nullptr, &link) == 0);
+		void *sComm = ofi_amd_net_link_send_comm(link), *rComm = ofi_amd_net_link_recv_comm(link);
+		const size_t sizes_to_try[2] = {4096, 1u << 20};
+		for (size_t bytes : sizes_to_try) {
+			void *src = nullptr, *dst = nullptr;
+			CHECK(nccl_net_ofi_gpu_mem_alloc(&src, bytes) == 0 && nccl_net_ofi_gpu_mem_alloc(&dst, bytes) == 0);
+			std::vector<uint8_t> pattern(bytes), back(bytes, 0);
+			for (size_t i = 0; i < bytes; i++) {
+				pattern[i] = (uint8_t)((i + bytes) * 2654435761u >> 24);
+			}
+			CHECK(nccl_net_ofi_gpu_mem_copy_host_to_device(src, pattern.data(), bytes) == 0);
+			CHECK(nccl_net_ofi_gpu_mem_copy_host_to_device(dst, back.data(), bytes) == 0);
+			void *sreq = nullptr, *rreq = nullptr, *mh = nullptr;
+			size_t rsize = bytes;
+			int tag = 1;
+			CHECK(net.isend(sComm, src, bytes, tag, mh, nullptr, &sreq) == ncclSuccess);
+			CHECK((sreq != nullptr) == (bytes + 8 <= 8192)); /* eager goes ahead of its receive */
+			CHECK(net.irecv(rComm, 1, &dst, &rsize, &tag, &mh, nullptr, &rreq) == ncclSuccess && rreq);
+			for (int tries = 0; !sreq && tries < 1000; tries++) {
+				CHECK(net.isend(sComm, src, bytes, tag, mh, nullptr, &sreq) == ncclSuccess);
+			}
+			CHECK(sreq);
+			int sdone = 0, rdone = 0, ssize = -1, got = -1;
+			for (long spins = 0; (!sdone || !rdone) && spins < 100000000L; spins++) {
+				if (!sdone) CHECK(net.test(sreq, &sdone, &ssize) == ncclSuccess);
+				if (!rdone) CHECK(net.test(rreq, &rdone, &got) == ncclSuccess);
+			}
+			CHECK(sdone && rdone && ssize == (int)bytes && got == (int)bytes);
+			void *freq = nullptr;
+			int isize = (int)bytes;
+			CHECK(net.iflush(rComm, 1, &dst, &isize, &mh, &freq) == ncclSuccess && freq);
+			int fdone = 0;
+			for (long spins = 0; !fdone && spins < 100000000L; spins++) {
+				CHECK(net.test(freq, &fdone, nullptr) == ncclSuccess);
+			}
+			CHECK(fdone);
+			CHECK(ofi_amd_gpu_mem_copy_device_to_host(back.data(), dst, bytes) == 0);
+			CHECK(memcmp(back.data(), pattern.data(), bytes) == 0);
+			CHECK(nccl_net_ofi_gpu_mem_free(src) == 0 && nccl_net_ofi_gpu_mem_free(dst) == 0);
+		}
+		CHECK(ofi_amd_net_link_destroy(link) == 0);
 	}
 	printf("gpu: ok\n");
 	return 0;

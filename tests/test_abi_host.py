@@ -15,7 +15,7 @@ from aws_ofi_nccl_amd import synthetic
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADERS = [os.path.join(ROOT, "include", h) for h in ("ofi_amd_hotpath.h", "ofi_amd_wire.h", "ofi_amd_sendrecv.h",
-                                                      "ofi_amd_rma_abi.h")]
+                                                      "ofi_amd_rma_abi.h", "ofi_amd_net_abi.h", "ofi_amd_nccl_err.h")]
 
 
 def declared_symbols():
@@ -63,6 +63,7 @@ def test_gpu_entry_points_fail_loudly_without_a_gpu(lib):
                                          nodes.ctypes.data, 11, ppn.ctypes.data, 4,
                                          algos.ctypes.data, 3, ctypes.byref(p)) == enodev
     assert lib.ofi_amd_devcopy_register(1, 64, ctypes.byref(p)) == enodev
+    assert lib.ofi_amd_net_link_create(4, 8192, 0, 0, 0, None, ctypes.byref(p)) == enodev and not p.value
     assert lib.ofi_amd_gpu_flush_gpudirect_rdma_writes() == -errno.EPERM   # as the ROCm reference
     assert lib.ofi_amd_gpu_have_gdr_support_attr() == 0
 
@@ -234,3 +235,27 @@ def test_device_put_header_compiles_in_a_user_kernel(tmp_path):
                      if "packed-fp32-ops" not in l and "is not a recognized feature" not in l)
     assert proc.returncode == 0, text
     assert obj.stat().st_size > 0
+
+
+def test_net_entry_points_check_their_arguments_without_a_link(lib):
+    """nccl_net_ofi_isend / _irecv / _iflush / _test (src/nccl_ofi_api.cpp:440-567): what they answer
+    before any comm is looked at."""
+    internal, invalid = 3, 4
+    vp = ctypes.c_void_p
+    req = vp(1)
+    assert lib.ofi_amd_net_isend(None, None, 8, 1, None, None, ctypes.byref(req)) == internal and req.value is None
+    data, sizes, tags, mhs = (vp * 1)(), (ctypes.c_size_t * 1)(8), (ctypes.c_int * 1)(1), (vp * 1)()
+    assert lib.ofi_amd_net_irecv(None, 1, data, sizes, tags, mhs, None, ctypes.byref(req)) == invalid
+    not_a_comm = (ctypes.c_uint64 * 4)()
+    assert lib.ofi_amd_net_irecv(not_a_comm, 1, data, sizes, tags, mhs, None, ctypes.byref(req)) == internal
+    assert lib.ofi_amd_net_irecv(not_a_comm, 9, data, sizes, tags, mhs, None, ctypes.byref(req)) == invalid
+    assert lib.ofi_amd_net_irecv_v5(not_a_comm, 1, data, None, tags, mhs, ctypes.byref(req)) == invalid
+    assert lib.ofi_amd_net_iflush(None, 1, data, (ctypes.c_int * 1)(8), mhs, ctypes.byref(req)) == internal
+    done = ctypes.c_int()
+    assert lib.ofi_amd_net_test(None, ctypes.byref(done), None) == internal
+    not_a_request = (ctypes.c_uint64 * 4)()
+    assert lib.ofi_amd_net_test(not_a_request, ctypes.byref(done), None) == internal
+    assert lib.ofi_amd_net_link_create(0, 8192, 0, 0, 0, None, ctypes.byref(req)) == -errno.EINVAL
+    assert lib.ofi_amd_net_link_create(4, 16384, 0, 0, 0, None, ctypes.byref(req)) == -errno.EINVAL
+    assert lib.ofi_amd_net_link_destroy(None) == -errno.EINVAL
+    assert lib.ofi_amd_net_link_send_comm(None) is None and lib.ofi_amd_net_link_recv_comm(None) is None

@@ -14,7 +14,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 GLUE_SRC = os.path.join(ROOT, "tests", "host", "integration_glue.cpp")
 GLUE_BIN = os.path.join(ROOT, "tests", "host", "bin", "integration_glue")
 REFERENCE = os.environ.get("REFERENCE", "/root/reference")
-HEADERS = ["ofi_amd_hotpath.h", "ofi_amd_wire.h", "ofi_amd_sendrecv.h", "ofi_amd_rma_abi.h", "ofi_amd_gin_device.h"]
+HEADERS = ["ofi_amd_hotpath.h", "ofi_amd_wire.h", "ofi_amd_sendrecv.h", "ofi_amd_rma_abi.h", "ofi_amd_net_abi.h",
+           "ofi_amd_nccl_err.h", "ofi_amd_gin_device.h"]
 
 
 def fenced_cpp_blocks(section_title):
