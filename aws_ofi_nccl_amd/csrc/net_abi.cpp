@@ -13,8 +13,8 @@
  * ends in a sentinel read-back into a pinned word.  When the sentinel of a group is seen, its
  * transfers are reported to the state machines in the order they were posted: the arrivals to
  * the receiving end, the completions to the sending end.  Every entry point makes progress
- * (polls the sentinels, launches what is waiting), the way the reference's drain the
- * completion queue.
+ * (polls the sentinels), the way the reference's drain the completion queue; test and iflush
+ * also launch the group being filled, so a run of posts followed by polling is one group.
  */
 #include <cerrno>
 #include <cstring>
@@ -250,12 +250,15 @@ struct ofi_amd_net_link {
 		return 0;
 	}
 
-	int progress()
+	/* Posting calls (isend, irecv) only look at what has completed; the calls that wait for
+	 * something (test, iflush) also launch what has been posted since the last launch, so a run
+	 * of posts followed by polling -- NCCL's pattern -- travels as one launch group. */
+	int progress(bool launch_pending)
 	{
 		st.progress_calls++;
 		int rc = reap();
 		if (rc == 0) rc = gather_eager_copies();
-		if (rc == 0) rc = launch();
+		if (rc == 0 && launch_pending) rc = launch();
 		return rc;
 	}
 };
@@ -292,7 +295,7 @@ int isend_impl(void *sendComm, void *data, size_t size, int tag, void **request)
 		return -EINVAL;
 	}
 	l->st.isend_calls++;
-	int rc = l->progress();
+	int rc = l->progress(false);
 	if (rc != 0) {
 		return rc;
 	}
@@ -390,7 +393,7 @@ int irecv_impl(void *recvComm, int n, void **data, const size_t *sizes, int *tag
 	}
 	*request = nullptr;
 	l->st.irecv_calls++;
-	int rc = l->progress();
+	int rc = l->progress(false);
 	if (rc != 0) {
 		return rc;
 	}
@@ -569,7 +572,7 @@ ncclResult_t ofi_amd_net_iflush(void *recvComm, int n, void **data, int *sizes, 
 	if (n < 1 || !sizes) {
 		return ncclInternalError;
 	}
-	int rc = l->progress();
+	int rc = l->progress(true);
 	if (rc != 0) {
 		return ofi_amd::nccl_result_of(rc);
 	}
@@ -606,7 +609,7 @@ ncclResult_t ofi_amd_net_test(void *request, int *done, int *sizes)
 	}
 	*done = 0;
 	ofi_amd_net_link *l = q->link;
-	int rc = l->progress();
+	int rc = l->progress(true);
 	if (rc != 0) {
 		return ofi_amd::nccl_result_of(rc);
 	}

@@ -691,6 +691,10 @@ def bench_sendrecv(lib, oracle, torch, np, args):
     out["parity_ok"] = all(s["parity_ok"] for s in out["sizes"])
     out["peak_payload_gbs"] = max(s["payload_gbs"] for s in out["sizes"])
     out["peak_msgs_per_s"] = max(s["msgs_per_s"] for s in out["sizes"])
+    # the same messages through the entry points NCCL calls (ofi_amd_net_isend / _irecv / _test / _iflush on
+    # the two ends of an in-process link), one call per message and poll, from this interpreter
+    out["through_net_entry_points"] = net_entry_points_leg(lib, torch, src, dst, top, inflight)
+    out["parity_ok"] = out["parity_ok"] and out["through_net_entry_points"]["parity_ok"]
     # the same harness with host buffers (pinned, read and written in place over the host link)
     if not args.skip_cpu:
         hsize, hn = 1 << 20, inflight * 4
@@ -710,6 +714,86 @@ def bench_sendrecv(lib, oracle, torch, np, args):
     del src, dst, pool
     torch.cuda.empty_cache()
     return out
+
+
+def net_entry_points_leg(lib, torch, src, dst, top, inflight):
+    """64 receives posted, 64 sends posted, every request polled with test(), a flush posted behind each
+    completed receive and polled with the rest: the calls of tests/functional/functional_test.cpp:592-731
+    with both ranks here, the flushes asynchronous as in NCCL's proxy."""
+    import _gpu
+    vp = ctypes.c_void_p
+    link = vp()
+    rc = lib.ofi_amd_net_link_create(4, 8192, 0, 0, 0, _gpu.stream(), ctypes.byref(link))
+    if rc != 0:
+        raise RuntimeError("net link rc=%d" % rc)
+    s_comm, r_comm = vp(lib.ofi_amd_net_link_send_comm(link)), vp(lib.ofi_amd_net_link_recv_comm(link))
+    done, tag, mh, sizes_out = ctypes.c_int(), (ctypes.c_int * 1)(1), (vp * 1)(0), (ctypes.c_int * 8)()
+
+    def poll(req):
+        if lib.ofi_amd_net_test(req, ctypes.byref(done), sizes_out) != 0:
+            raise RuntimeError("net test failed")
+        return done.value != 0
+
+    res = []
+    for size in (1 << 20, 64 << 20):
+        if size > top:
+            continue
+        rounds = 8 if size <= (1 << 20) else 2
+        best = None
+        for _ in range(2):                                           # first pass warms up
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(rounds):
+                rreqs, sreqs = [], []
+                for k in range(inflight):
+                    req = vp()
+                    data = (vp * 1)(dst.data_ptr() + k * top)
+                    if lib.ofi_amd_net_irecv(r_comm, 1, data, (ctypes.c_size_t * 1)(size), tag, mh, None,
+                                             ctypes.byref(req)) != 0 or not req.value:
+                        raise RuntimeError("net irecv failed")
+                    rreqs.append((req, data))
+                for k in range(inflight):
+                    req = vp()
+                    while not req.value:
+                        if lib.ofi_amd_net_isend(s_comm, vp(src.data_ptr() + k * top), size, 1, None, None,
+                                                 ctypes.byref(req)) != 0:
+                            raise RuntimeError("net isend failed")
+                    sreqs.append(req)
+                freqs = []
+                while rreqs or sreqs or freqs:
+                    sreqs = [q for q in sreqs if not poll(q)]
+                    freqs = [q for q in freqs if not poll(q)]
+                    still = []
+                    for q, data in rreqs:
+                        if not poll(q):
+                            still.append((q, data))
+                            continue
+                        # NCCL's proxy posts the flush behind a completed receive and polls it with the rest
+                        freq = vp()
+                        if lib.ofi_amd_net_iflush(r_comm, 1, data, (ctypes.c_int * 1)(min(size, 1 << 30)), mh,
+                                                  ctypes.byref(freq)) != 0 or not freq.value:
+                            raise RuntimeError("net iflush failed")
+                        freqs.append(freq)
+                    rreqs = still
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        n = inflight * rounds
+        ok = all(bool(torch.equal(dst[k * top:k * top + size], src.view(torch.uint8)[k * top:k * top + size]))
+                 for k in (0, inflight // 2, inflight - 1))
+        res.append({"bytes": size, "messages": n, "payload_gbs": n * size / best / 1e9,
+                    "us_per_message": best / n * 1e6, "parity_ok": ok})
+    st = m_stats(lib, link)
+    if lib.ofi_amd_net_link_destroy(link) != 0:
+        raise RuntimeError("net link destroy failed")
+    return {"sizes": res, "launches": st.launches, "progress_calls": st.progress_calls,
+            "parity_ok": all(r["parity_ok"] for r in res)}
+
+
+def m_stats(lib, link):
+    import aws_ofi_nccl_amd as m
+    st = m.NetLinkStats()
+    lib.ofi_amd_net_link_stats(link, ctypes.byref(st))
+    return st
 
 
 def main():
