@@ -71,7 +71,7 @@ def build_oracle():
                           stderr=subprocess.STDOUT, text=True)
     if proc.returncode != 0:
         raise RuntimeError("oracle build failed:\n%s" % proc.stdout)
-    # the reference-side glue of INTEGRATION.md against the reference's headers (a test binary; only
+    # the reference-side glue of the integration guide against the reference's headers (a test binary; only
     # where the reference tree is present)
     proc = subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "host")], stdout=subprocess.PIPE,
                           stderr=subprocess.STDOUT, text=True)

@@ -1,8 +1,9 @@
 /*
  * The glue a maintainer of the reference would add on top of the C ABI, compiled for real:
  * the replacement of src/nccl_ofi_rocm.cpp and an nccl_ofi_device_copy implementation, both
- * as they are printed in INTEGRATION.md (sections 1 and 2; tests/test_integration_glue.py
- * checks that the text between the markers below is the text printed there), built against
+ * as they are printed in sections 1 and 2 of the integration guide at the repository root
+ * (tests/test_integration_glue.py checks that the text between the markers below is the text
+ * printed there), built against
  * the reference's own headers where they lie (include/nccl_ofi_rocm.h,
  * include/nccl_ofi_device_copy.h) and linked against libofi_amd_hotpath.so.
  *
