@@ -195,6 +195,15 @@ class RecvState(ctypes.Structure):
                 ("pad2", c_u32), ("n_ctrl_sent", c_u64)]
 
 
+DEVFAB_ACK_FN = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, c_u32, c_u64)
+
+
+class DevfabStats(ctypes.Structure):
+    """ofi_amd_devfab_stats_t"""
+    _fields_ = [(k, c_u64) for k in ("groups", "launches", "copy_entries", "bytes", "writes", "reads", "flush_reads",
+                                     "metas", "acks", "work_items")]
+
+
 class NetLinkStats(ctypes.Structure):
     """ofi_amd_net_link_stats_t"""
     _fields_ = [(k, c_u64) for k in ("isend_calls", "isend_again", "eager_sends", "write_sends", "rdma_writes",
@@ -416,6 +425,14 @@ PROTOTYPES = {
     "ofi_amd_net_isend_v9": (ctypes.c_int, [c_vp, c_vp, ctypes.c_size_t, ctypes.c_int, c_vp, ctypes.POINTER(c_vp)]),
     "ofi_amd_net_irecv_v9": (ctypes.c_int, [c_vp, ctypes.c_int, ctypes.POINTER(c_vp), ctypes.POINTER(ctypes.c_size_t),
                                             ctypes.POINTER(ctypes.c_int), ctypes.POINTER(c_vp), ctypes.POINTER(c_vp)]),
+    "ofi_amd_devfab_create": (ctypes.c_int, [c_u32, c_u32, c_u32, ctypes.POINTER(c_u32), ctypes.POINTER(GinSignalRegion),
+                                             c_u32, c_vp, ctypes.POINTER(c_vp)]),
+    "ofi_amd_devfab_destroy": (ctypes.c_int, [c_vp]),
+    "ofi_amd_devfab_ops": (ctypes.c_int, [c_vp, ctypes.POINTER(GinFabricOps)]),
+    "ofi_amd_devfab_on_ack": (ctypes.c_int, [c_vp, DEVFAB_ACK_FN, c_vp]),
+    "ofi_amd_devfab_ring_all": (ctypes.c_int, [c_vp]),
+    "ofi_amd_devfab_quiesce": (ctypes.c_int, [c_vp, c_u32]),
+    "ofi_amd_devfab_stats": (ctypes.c_int, [c_vp, ctypes.POINTER(DevfabStats)]),
     "ofi_amd_loopfab_create": (ctypes.c_int, [c_u32, c_u32, ctypes.POINTER(c_vp)]),
     "ofi_amd_loopfab_destroy": (ctypes.c_int, [c_vp]),
     "ofi_amd_loopfab_ops": (ctypes.c_int, [c_vp, ctypes.POINTER(GinFabricOps)]),

@@ -677,6 +677,49 @@ int ofi_amd_gin_signal_apply(const ofi_amd_gin_signal_work_t *d_work, uint32_t n
 			     uint32_t *d_rejected, void *stream);
 
 /*
+ * A fabric for the transmit engine (and for ofi_amd_rma_ctx_create) that moves the bytes: the
+ * initiator and its targets are this process, the wire is device copies on `stream`.  It stands
+ * where the reference has libfabric endpoints, the target's progress thread and GDRCopy
+ * (what tests/functional/rma.cpp sets up with two ranks).  Send queues and doorbells as
+ * ofi_amd_loopfab_*.  Transmitted posts travel in launch groups: a write or a read is one entry
+ * of ofi_amd_copy_table_pieces (a read of peer OFI_AMD_GIN_PEER_SELF lands in pinned host
+ * memory from ofi_amd_gpu_host_alloc), a group ends in a sentinel read-back, and when that is
+ * seen -- inside cq_read, i.e. inside the engine's progress call -- the group's posts complete
+ * and the target hears of them in transmission order: write completions and metadata
+ * messages go to a receiver (ofi_amd_gin_rx_* with n_peers peers: the state of target rank
+ * `peer` towards this initiator), the signal work it releases is applied to `regions` by
+ * ofi_amd_gin_signal_apply in the next group's launch, and its ACKs go to on_ack (an ACK post
+ * of the engine itself is delivered there too).  Signals therefore land one progress call after
+ * the completion that released them: keep calling progress (NCCL's proxy does), or call
+ * ofi_amd_devfab_quiesce, which runs the fabric until nothing is in flight or waiting and then
+ * waits for the stream (-ETIMEDOUT after timeout_ms, 0 = 10,000).  One thread.  -ENODEV without a
+ * GPU.
+ */
+typedef struct ofi_amd_devfab ofi_amd_devfab_t;
+typedef struct {
+	uint64_t groups;       /* launch groups */
+	uint64_t launches;     /* kernel launches: copies, signal applies, sentinels */
+	uint64_t copy_entries;
+	uint64_t bytes;        /* payload of writes and reads */
+	uint64_t writes;
+	uint64_t reads;
+	uint64_t flush_reads;
+	uint64_t metas;
+	uint64_t acks;         /* handed to on_ack */
+	uint64_t work_items;   /* folded signal updates applied */
+} ofi_amd_devfab_stats_t;
+int ofi_amd_devfab_create(uint32_t num_rails, uint32_t sq_depth, uint32_t n_peers, const uint32_t *peer_comm_ids,
+			  const ofi_amd_gin_signal_region_t *regions, uint32_t n_regions, void *stream,
+			  ofi_amd_devfab_t **out);
+int ofi_amd_devfab_destroy(ofi_amd_devfab_t *f);
+int ofi_amd_devfab_ops(ofi_amd_devfab_t *f, ofi_amd_gin_fabric_ops_t *ops);
+int ofi_amd_devfab_on_ack(ofi_amd_devfab_t *f, int (*on_ack)(void *arg, uint32_t peer, uint64_t ack_msg), void *arg);
+/* Rings every rail's doorbell: posts still waiting behind FI_MORE are transmitted. */
+int ofi_amd_devfab_ring_all(ofi_amd_devfab_t *f);
+int ofi_amd_devfab_quiesce(ofi_amd_devfab_t *f, uint32_t timeout_ms);
+int ofi_amd_devfab_stats(const ofi_amd_devfab_t *f, ofi_amd_devfab_stats_t *out);
+
+/*
  * In-process loop-back of the whole GIN path on one GPU: initiator and target are the same
  * device, the "network" is this call.  For every descriptor drained from the rings it
  *   1. derives the wire record (ofi_amd_gin_derive on comms[context], ack_model 0),

@@ -384,6 +384,58 @@ static int gpu_checks()
 		}
 		CHECK(ofi_amd_net_link_destroy(link) == 0);
 	}
+	{ /* a put-signal through the RMA v15 table over the fabric that moves the bytes: the data is at the
+	   * peer, the request completes, and the peer's signal counts one once progress has run on */
+		const ncclRma_v15_t table = rma_table_with_this_librarys_data_path();
+		constexpr size_t bytes = 300000;
+		void *src = nullptr, *dst = nullptr, *counters = nullptr;
+		CHECK(nccl_net_ofi_gpu_mem_alloc(&src, bytes) == 0 && nccl_net_ofi_gpu_mem_alloc(&dst, bytes) == 0 &&
+		      nccl_net_ofi_gpu_mem_alloc(&counters, 4096) == 0);
+		std::vector<uint8_t> pattern(bytes), back(bytes, 0), zero(4096, 0);
+		for (size_t i = 0; i < bytes; i++) {
+			pattern[i] = (uint8_t)((i * 7 + 3) * 2654435761u >> 24);
+		}
+		CHECK(nccl_net_ofi_gpu_mem_copy_host_to_device(src, pattern.data(), bytes) == 0);
+		CHECK(nccl_net_ofi_gpu_mem_copy_host_to_device(dst, back.data(), bytes) == 0);
+		CHECK(nccl_net_ofi_gpu_mem_copy_host_to_device(counters, zero.data(), 4096) == 0);
+		const uint64_t signal_base = 0x7f5500000000ull;
+		const ofi_amd_gin_signal_region_t region = {signal_base, 4096, counters};
+		const uint32_t ids[2] = {0, 1};
+		ofi_amd_devfab_t *fab = nullptr;
+		ofi_amd_gin_fabric_ops_t ops;
+		CHECK(ofi_amd_devfab_create(4, 64, 2, ids, &region, 1, nullptr, &fab) == 0 && ofi_amd_devfab_ops(fab, &ops) == 0);
+		ofi_amd_rma_ctx_t *rma = nullptr;
+		CHECK(ofi_amd_rma_ctx_create(2, 4, 131072, 64, &ops, 256, 0, &rma) == 0);
+		CHECK(ofi_amd_devfab_on_ack(fab, [](void *ctx, uint32_t peer, uint64_t msg) {
+			      return ofi_amd_rma_ack_received(static_cast<ofi_amd_rma_ctx_t *>(ctx), peer, msg);
+		      }, rma) == 0);
+		const uint64_t keys[8] = {1, 2, 3, 4, 5, 6, 7, 8};
+		const uint64_t src_addr[2] = {(uint64_t)(uintptr_t)src, (uint64_t)(uintptr_t)src};
+		const uint64_t dst_addr[2] = {(uint64_t)(uintptr_t)dst, (uint64_t)(uintptr_t)dst};
+		const uint64_t sig_addr[2] = {signal_base, signal_base};
+		ofi_amd_rma_mr_t *mr_src = nullptr, *mr_dst = nullptr, *mr_sig = nullptr;
+		CHECK(ofi_amd_rma_mr_create(rma, src_addr[0], src_addr, src_addr, keys, &mr_src) == 0);
+		CHECK(ofi_amd_rma_mr_create(rma, dst_addr[0], dst_addr, dst_addr, keys, &mr_dst) == 0);
+		CHECK(ofi_amd_rma_mr_create(rma, signal_base, sig_addr, sig_addr, keys, &mr_sig) == 0);
+		void *request = nullptr;
+		CHECK(table.iputSignal(rma, 0, 0, mr_src, bytes, 0, mr_dst, 1, 16, mr_sig, 1, 1 /* increment */, true,
+				       ncclRmaOptFlagsDefault, &request) == ncclSuccess && request);
+		int done = 0;
+		for (long spins = 0; !done && spins < 100000000L; spins++) {
+			CHECK(table.test(rma, request, &done) == ncclSuccess);
+			if (!done) CHECK(table.rmaProgress(rma) == ncclSuccess);
+		}
+		CHECK(done);
+		CHECK(ofi_amd_devfab_quiesce(fab, 0) == 0);
+		CHECK(ofi_amd_gpu_mem_copy_device_to_host(back.data(), dst, bytes) == 0);
+		CHECK(memcmp(back.data(), pattern.data(), bytes) == 0);
+		uint64_t slots[4] = {9, 9, 9, 9};
+		CHECK(ofi_amd_gpu_mem_copy_device_to_host(slots, counters, sizeof(slots)) == 0);
+		CHECK(slots[0] == 0 && slots[1] == 0 && slots[2] == 1 && slots[3] == 0);
+		CHECK(ofi_amd_rma_mr_destroy(mr_src) == 0 && ofi_amd_rma_mr_destroy(mr_dst) == 0 && ofi_amd_rma_mr_destroy(mr_sig) == 0);
+		CHECK(ofi_amd_rma_ctx_destroy(rma) == 0 && ofi_amd_devfab_destroy(fab) == 0);
+		CHECK(nccl_net_ofi_gpu_mem_free(src) == 0 && nccl_net_ofi_gpu_mem_free(dst) == 0 && nccl_net_ofi_gpu_mem_free(counters) == 0);
+	}
 	printf("gpu: ok\n");
 	return 0;
 }

@@ -64,6 +64,8 @@ def test_gpu_entry_points_fail_loudly_without_a_gpu(lib):
                                          algos.ctypes.data, 3, ctypes.byref(p)) == enodev
     assert lib.ofi_amd_devcopy_register(1, 64, ctypes.byref(p)) == enodev
     assert lib.ofi_amd_net_link_create(4, 8192, 0, 0, 0, None, ctypes.byref(p)) == enodev and not p.value
+    ids = (ctypes.c_uint32 * 2)(0, 1)
+    assert lib.ofi_amd_devfab_create(4, 64, 2, ids, None, 0, None, ctypes.byref(p)) == enodev and not p.value
     assert lib.ofi_amd_gpu_flush_gpudirect_rdma_writes() == -errno.EPERM   # as the ROCm reference
     assert lib.ofi_amd_gpu_have_gdr_support_attr() == 0
 
