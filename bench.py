@@ -570,10 +570,11 @@ def bench_gin(lib, oracle, torch, np, args):
     side = torch.cuda.Stream()
     # a progress call after every operation (the strictest caller), and after every 64th: the
     # reference's own test posts 64 puts and 64 put-signals before its first progress call
-    # (tests/functional/rma.cpp:213-246).  Two passes each; the first warms the pinned tables up.
+    # (tests/functional/rma.cpp:213-246).  Four passes each of some 60 ms: the first warms the pinned tables up,
+    # and the host thread's rate moves by 10 % from pass to pass; the best pass is reported, all are listed.
     for key, interval in (("loopback", 1), ("loopback_progress_every_64", 64)):
-        best = None
-        for _ in range(2):
+        best, rates = None, []
+        for _ in range(4):
             for c in range(l_ctx):
                 lib.ofi_amd_gin_comm_init(ctypes.byref(comms[c]), c, 4, 131072, 64, 0)
             d_cnt.zero_()
@@ -602,8 +603,10 @@ def bench_gin(lib, oracle, torch, np, args):
                    "ns_per_put": secs / lstats.descriptors * 1e9,
                    "ns_per_put_by_stage": {k: getattr(lstats, "ns_" + k) / lstats.descriptors for k in (
                        "pop_derive", "tx_post", "wire", "progress", "rx", "launch_wait")}}
+            rates.append(res["puts_per_s"])
             if best is None or res["puts_per_s"] > best["puts_per_s"]:
                 best = res
+        best["puts_per_s_of_each_pass"] = rates
         out[key] = best
     del d_srcbuf, d_dstbuf
     torch.cuda.empty_cache()
