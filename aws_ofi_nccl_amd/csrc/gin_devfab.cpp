@@ -22,37 +22,18 @@
 #include <new>
 #include <vector>
 
+#include "host_util.hpp"
 #include "ofi_amd_hotpath.h"
 
 namespace {
+
+using ofi_amd::pinned_t;
+using ofi_amd::ring_t;
 
 constexpr uint32_t kGroups = 4;
 constexpr uint32_t kGroupEntries = 4096;
 constexpr uint32_t kGroupWork = 4096;
 constexpr uint64_t kSentinel = 0xdeadbeefdeadbeefull; /* NCCL_OFI_GIN_FLUSH_SENTINEL_VAL */
-
-struct pinned_t {
-	void *host = nullptr;
-	void *dev = nullptr;
-	int alloc(size_t bytes)
-	{
-		int rc = ofi_amd_gpu_host_alloc(&host, bytes);
-		if (rc == 0) {
-			std::memset(host, 0, bytes);
-			rc = ofi_amd_gpu_host_get_device_pointer(&dev, host);
-		}
-		return rc;
-	}
-	void release()
-	{
-		if (host) {
-			(void)ofi_amd_gpu_host_free(host);
-		}
-		host = dev = nullptr;
-	}
-	template <typename T> T *as() { return static_cast<T *>(host); }
-	template <typename T> const T *dev_as() const { return static_cast<const T *>(dev); }
-};
 
 /* What the target (or, for an ACK, the initiator) hears when a group has landed. */
 struct event_t {
@@ -99,27 +80,6 @@ struct group_t {
 		events.clear();
 		launched = false;
 	}
-};
-
-template <typename T>
-struct ring_t {
-	std::vector<T> slot;
-	uint32_t mask = 0, head = 0, tail = 0;
-	void reset(uint32_t capacity)
-	{
-		uint32_t n = 1;
-		while (n < capacity) {
-			n <<= 1;
-		}
-		slot.assign(n, T());
-		mask = n - 1;
-		head = tail = 0;
-	}
-	uint32_t size() const { return tail - head; }
-	bool empty() const { return tail == head; }
-	T &at(uint32_t k) { return slot[(head + k) & mask]; }
-	void push(const T &v) { slot[tail++ & mask] = v; }
-	void pop() { head++; }
 };
 
 } // namespace
@@ -349,20 +309,9 @@ struct ofi_amd_devfab {
 		return (int)n;
 	}
 
-	bool idle()
-	{
-		if (head != cur || !rung.empty() || !filling().empty()) {
-			return false;
-		}
-		ofi_amd_gin_signal_work_t probe;
-		const uint32_t n = ofi_amd_gin_rx_take_work(rx, &probe, 1);
-		if (n) {
-			group_t &g = filling();
-			g.work.as<ofi_amd_gin_signal_work_t>()[g.n_work++] = probe;
-			return false;
-		}
-		return true;
-	}
+	/* nothing in flight and nothing waiting: advance() has just run, so whatever the last landing
+	 * released is either launched (head != cur) or still in the group being filled */
+	bool idle() { return head == cur && rung.empty() && filling().empty(); }
 };
 
 extern "C" {

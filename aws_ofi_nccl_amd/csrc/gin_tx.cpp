@@ -15,6 +15,7 @@
 #include <new>
 #include <vector>
 
+#include "host_util.hpp"
 #include "ofi_amd_hotpath.h"
 
 namespace {
@@ -440,28 +441,7 @@ int ofi_amd_gin_tx_stats(const ofi_amd_gin_tx_t *tx, ofi_amd_gin_tx_stats_t *out
 
 /* ---------------------------------------------------------------- the in-process fabric ---- */
 
-/* Fixed-size queue over a power-of-two array: positions only grow, the index is the position
- * masked. */
-template <typename T>
-struct ring_t {
-	std::vector<T> slot;
-	uint32_t mask = 0, head = 0, tail = 0; /* head: oldest entry, tail: next free position */
-	void reset(uint32_t capacity)
-	{
-		uint32_t n = 1;
-		while (n < capacity) {
-			n <<= 1;
-		}
-		slot.assign(n, T());
-		mask = n - 1;
-		head = tail = 0;
-	}
-	uint32_t size() const { return tail - head; }
-	bool empty() const { return tail == head; }
-	T &at(uint32_t k) { return slot[(head + k) & mask]; } /* k-th oldest */
-	void push(const T &v) { slot[tail++ & mask] = v; }
-	void pop() { head++; }
-};
+using ofi_amd::ring_t;
 
 struct ofi_amd_loopfab {
 	struct rail_t {

@@ -21,6 +21,7 @@
 #include <new>
 #include <vector>
 
+#include "host_util.hpp"
 #include "nccl_translate.hpp"
 #include "ofi_amd_hotpath.h"
 #include "ofi_amd_net_abi.h"
@@ -34,28 +35,7 @@ constexpr uint32_t kGroupEager = 256;   /* eager copies of a group */
 constexpr uint32_t kMagic = 0x4e455451; /* marks a live request */
 constexpr uint32_t kMaxRxBuffers = 4096;
 
-struct pinned_t {
-	void *host = nullptr;
-	void *dev = nullptr;
-	int alloc(size_t bytes)
-	{
-		int rc = ofi_amd_gpu_host_alloc(&host, bytes ? bytes : 8);
-		if (rc == 0) {
-			std::memset(host, 0, bytes ? bytes : 8);
-			rc = ofi_amd_gpu_host_get_device_pointer(&dev, host);
-		}
-		return rc;
-	}
-	void release()
-	{
-		if (host) {
-			(void)ofi_amd_gpu_host_free(host);
-		}
-		host = dev = nullptr;
-	}
-	template <typename T> T *as() { return static_cast<T *>(host); }
-	template <typename T> const T *dev_as() const { return static_cast<const T *>(dev); }
-};
+using ofi_amd::pinned_t;
 
 enum req_kind_t : uint8_t { kSend = 1, kRecv = 2, kFlush = 3 };
 

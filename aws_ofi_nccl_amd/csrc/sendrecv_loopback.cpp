@@ -13,32 +13,16 @@
 #include <cstring>
 #include <vector>
 
+#include "host_util.hpp"
 #include "ofi_amd_sendrecv.h"
 
 namespace {
 
+using ofi_amd::pinned_t;
+
 constexpr uint32_t kPiece = 1u << 30;    /* a table entry's length is 32 bits: longer writes are cut */
 constexpr uint32_t kRxStride = 8320;     /* 8192 + header room, rounded to the 128-byte rx alignment */
 constexpr int64_t kEagerSendSize = 8192; /* OFI_NCCL_EAGER_MAX_SIZE default, src/nccl_ofi_rdma.cpp:6808 */
-
-struct pinned_t {
-	void *host = nullptr;
-	void *dev = nullptr;
-	int alloc(size_t bytes)
-	{
-		int rc = ofi_amd_gpu_host_alloc(&host, bytes ? bytes : 8);
-		return rc ? rc : ofi_amd_gpu_host_get_device_pointer(&dev, host);
-	}
-	void release()
-	{
-		if (host) {
-			(void)ofi_amd_gpu_host_free(host);
-		}
-		host = dev = nullptr;
-	}
-	template <typename T> T *as() { return static_cast<T *>(host); }
-	template <typename T> const T *dev_as() const { return static_cast<const T *>(dev); }
-};
 
 struct open_msg_t {
 	uint64_t index = 0;
