@@ -641,6 +641,9 @@ def bench_gin(lib, oracle, torch, np, args):
         out["parity_ok"] = (out["drain"]["checksum"] == "%016x" % ck and
                             out["drain_and_derive_wire"]["checksum"] == "%016x" % ck and
                             out["drain_derive_and_check_wire"]["checksum"] == "%016x" % ck_wire)
+    out["rma_entry_points_over_device_fabric"] = rma_entry_points_leg(lib, torch, np)
+    if "parity_ok" in out:
+        out["parity_ok"] = out["parity_ok"] and out["rma_entry_points_over_device_fabric"]["parity_ok"]
     out["derive_checksums_agree_across_thread_counts"] = (
         out["drain_derive_and_check_wire"]["checksum"] ==
         out["drain_derive_and_check_wire_4_proxy_threads"]["checksum"] and
@@ -717,6 +720,68 @@ def bench_sendrecv(lib, oracle, torch, np, args):
     del src, dst, pool
     torch.cuda.empty_cache()
     return out
+
+
+def rma_entry_points_leg(lib, torch, np):
+    """Put-signals through ofi_amd_rma_iputSignal / _test / _rmaProgress, one call each from this
+    interpreter, over the fabric that moves the bytes on the device (ofi_amd_devfab_*): 64 operations in
+    flight, "test the oldest, progress if it is not done" (tests/functional/rma.cpp:316-330)."""
+    import _gpu
+    import aws_ofi_nccl_amd as m
+    vp = ctypes.c_void_p
+    n_ops, inflight, res = 8192, 64, []
+    base = 0x7F5500000000
+    counters = torch.zeros(512, dtype=torch.int64, device="cuda")
+    region = (m.GinSignalRegion * 1)(m.GinSignalRegion(base, 4096, counters.data_ptr()))
+    ids = (ctypes.c_uint32 * 2)(0, 1)
+    for size in (4096, 1 << 20):
+        window = size * inflight
+        src = torch.randint(0, 256, (window,), dtype=torch.uint8, device="cuda")
+        dst = torch.zeros(window, dtype=torch.uint8, device="cuda")
+        counters.zero_()
+        torch.cuda.synchronize()
+        fab, ctx, ops = vp(), vp(), m.GinFabricOps()
+        m.check(lib.ofi_amd_devfab_create(4, 256, 2, ids, region, 1, _gpu.stream(), ctypes.byref(fab)), "devfab")
+        m.check(lib.ofi_amd_devfab_ops(fab, ctypes.byref(ops)), "devfab ops")
+        m.check(lib.ofi_amd_rma_ctx_create(2, 4, 131072, 64, ctypes.byref(ops), 4096, 0, ctypes.byref(ctx)), "rma ctx")
+        ack = m.DEVFAB_ACK_FN(ctypes.cast(lib.ofi_amd_rma_ack_received, vp).value)
+        m.check(lib.ofi_amd_devfab_on_ack(fab, ack, ctx), "on_ack")
+        keys = np.arange(8, dtype=np.uint64)
+        handles = []
+        for local, remote in ((src.data_ptr(), src.data_ptr()), (dst.data_ptr(), dst.data_ptr()), (base, base)):
+            addr, h = np.array([remote, remote], dtype=np.uint64), vp()
+            m.check(lib.ofi_amd_rma_mr_create(ctx, local, addr.ctypes.data, addr.ctypes.data, keys.ctypes.data,
+                                              ctypes.byref(h)), "mr")
+            handles.append(h)
+        mr_src, mr_dst, mr_sig = handles
+        open_reqs, done = [], ctypes.c_int()
+        t0 = time.perf_counter()
+        for i in range(n_ops):
+            req, off = vp(), (i % inflight) * size
+            if lib.ofi_amd_rma_iputSignal(ctx, 0, off, mr_src, size, off, mr_dst, 1, 8 * (i % 4), mr_sig, 1, 1, True, 0,
+                                          ctypes.byref(req)) != 0:
+                raise RuntimeError("rma iputSignal failed")
+            open_reqs.append(req)
+            while len(open_reqs) >= inflight or (i == n_ops - 1 and open_reqs):
+                if lib.ofi_amd_rma_test(ctx, open_reqs[0], ctypes.byref(done)) != 0:
+                    raise RuntimeError("rma test failed")
+                if done.value:
+                    open_reqs.pop(0)
+                elif lib.ofi_amd_rma_rmaProgress(ctx) != 0:
+                    raise RuntimeError("rma progress failed")
+        m.check(lib.ofi_amd_devfab_quiesce(fab, 0), "quiesce")
+        secs = time.perf_counter() - t0
+        st = m.DevfabStats()
+        lib.ofi_amd_devfab_stats(fab, ctypes.byref(st))
+        ok = bool(torch.equal(src, dst)) and counters[:4].tolist() == [n_ops // 4] * 4
+        res.append({"bytes": size, "operations": n_ops, "puts_per_s": n_ops / secs, "payload_gbs": n_ops * size / secs / 1e9,
+                    "launch_groups": st.groups, "acks": st.acks, "parity_ok": ok})
+        for h in handles:
+            lib.ofi_amd_rma_mr_destroy(h)
+        lib.ofi_amd_rma_ctx_destroy(ctx)
+        lib.ofi_amd_devfab_destroy(fab)
+        del src, dst
+    return {"in_flight": inflight, "sizes": res, "parity_ok": all(r["parity_ok"] for r in res)}
 
 
 def net_entry_points_leg(lib, torch, src, dst, top, inflight):
