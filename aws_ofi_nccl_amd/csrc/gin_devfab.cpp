@@ -31,6 +31,7 @@ using ofi_amd::pinned_t;
 using ofi_amd::ring_t;
 
 constexpr uint32_t kGroups = 4;
+constexpr uint32_t kGroupsKeptBusy = 2; /* in flight before posts start gathering instead of leaving at once */
 constexpr uint32_t kGroupEntries = 4096;
 constexpr uint32_t kGroupWork = 4096;
 constexpr uint64_t kSentinel = 0xdeadbeefdeadbeefull; /* NCCL_OFI_GIN_FLUSH_SENTINEL_VAL */
@@ -191,10 +192,14 @@ struct ofi_amd_devfab {
 		return 0;
 	}
 
+	/* While two groups are in flight, what is transmitted keeps gathering in the group being
+	 * filled instead of leaving as a group of its own: the pipeline stays busy, and the size of a
+	 * group follows the time a launch takes.  A full table leaves regardless. */
 	int launch()
 	{
 		group_t &g = filling();
-		if (g.empty() || !can_launch()) {
+		const bool full = g.n_copy >= kGroupEntries || g.n_work >= kGroupWork;
+		if (g.empty() || !can_launch() || (!full && cur - head >= kGroupsKeptBusy)) {
 			return 0;
 		}
 		int rc = 0;

@@ -10,7 +10,8 @@
  * device copies of what the sending end handed out since the last launch (an eager send:
  * header and payload into an rx buffer; a rendezvous write: one table entry per rail stripe)
  * and the eager copies of what the receiving end has matched (rx buffer -> user buffer), and
- * ends in a sentinel read-back into a pinned word.  When the sentinel of a group is seen, its
+ * ends in a sentinel read-back into a pinned word; the flushes asked for since the last launch
+ * ride on that read-back.  When the sentinel of a group is seen, its
  * transfers are reported to the state machines in the order they were posted: the arrivals to
  * the receiving end, the completions to the sending end.  Every entry point makes progress
  * (polls the sentinels), the way the reference's drain the completion queue; test and iflush
@@ -29,7 +30,8 @@
 namespace {
 
 constexpr uint32_t kRxStride = 8320;    /* 8192 + header room, rounded to the 128-byte rx alignment */
-constexpr uint32_t kGroups = 8;         /* launch groups in flight */
+constexpr uint32_t kGroups = 8;         /* launch groups in flight, at most */
+constexpr uint32_t kGroupsKeptBusy = 2; /* in flight before posts start gathering instead of leaving at once */
 constexpr uint32_t kGroupEntries = 512; /* table entries of a group's wire copies */
 constexpr uint32_t kGroupEager = 256;   /* eager copies of a group */
 constexpr uint32_t kMagic = 0x4e455451; /* marks a live request */
@@ -67,6 +69,7 @@ struct group_t {
 	uint32_t n_copy = 0, n_hdr = 0, n_eager = 0, max_len = 0;
 	std::vector<landing_t> landings;
 	std::vector<ofi_amd_eager_copy_item_t> items;
+	std::vector<int32_t> flushes; /* flush requests that ride on this group's sentinel read-back */
 	bool launched = false;
 	int alloc()
 	{
@@ -89,12 +92,13 @@ struct group_t {
 		}
 	}
 	/* a transfer without bytes (a zero-length write) still waits for its group's sentinel */
-	bool empty() const { return n_copy == 0 && n_eager == 0 && landings.empty(); }
+	bool empty() const { return n_copy == 0 && n_eager == 0 && landings.empty() && flushes.empty(); }
 	void reset()
 	{
 		n_copy = n_hdr = n_eager = max_len = 0;
 		landings.clear();
 		items.clear();
+		flushes.clear();
 		launched = false;
 	}
 };
@@ -110,7 +114,7 @@ struct ofi_amd_net_link {
 	void *rx_pool = nullptr;
 	std::vector<uint32_t> rx_free;
 	void *d_flush_buf = nullptr;
-	pinned_t flush_slots; /* per flush request: one 64-byte slot per rail */
+	std::vector<uint64_t> flush_slots; /* per flush request: one 64-byte slot per rail */
 	group_t groups[kGroups];
 	uint32_t head = 0, cur = 0; /* positions: head = oldest launched group, cur = the one being filled */
 	std::vector<net_req_t> send_reqs, recv_reqs, flush_reqs;
@@ -160,6 +164,15 @@ struct ofi_amd_net_link {
 				rx_free.push_back((uint32_t)it.rx_cookie);
 				st.eager_copies++;
 			}
+			/* the group's sentinel read-back was queued behind everything launched before these
+			 * flushes were asked for: it is their read-back too (one operation flushes all requests
+			 * at once, as the reference's flush does for the buffers of one call) */
+			for (int32_t id : g.flushes) {
+				for (uint32_t rail = 0; rail < num_rails; rail++) {
+					__atomic_store_n(&flush_slots[((size_t)id * OFI_AMD_WIRE_MAX_RAILS + rail) * 8],
+							 (uint64_t)OFI_AMD_RDMA_FLUSH_SENTINEL, __ATOMIC_RELEASE);
+				}
+			}
 			g.reset();
 			head++;
 		}
@@ -191,10 +204,14 @@ struct ofi_amd_net_link {
 		}
 	}
 
-	int launch()
+	/* While two groups are in flight, what is posted keeps gathering in the group being filled
+	 * instead of leaving as a group of its own: the pipeline stays busy, and the size of a group
+	 * follows the time a launch takes (small messages, many to a group; large ones, few).
+	 * `now`: launch regardless, as long as a group slot is free (the caller is out of room). */
+	int launch(bool now = false)
 	{
 		group_t &g = filling();
-		if (g.empty() || !can_launch()) {
+		if (g.empty() || !can_launch() || (!now && cur - head >= kGroupsKeptBusy)) {
 			return 0;
 		}
 		int rc = 0;
@@ -284,7 +301,7 @@ int isend_impl(void *sendComm, void *data, size_t size, int tag, void **request)
 	group_t *g = &l->filling();
 	const bool may_go_eager = ofi_amd_eager_fits(size, l->eager_max_size) != 0;
 	if (g->n_copy + OFI_AMD_WIRE_MAX_RAILS + 2 > kGroupEntries || (may_go_eager && l->rx_free.empty())) {
-		rc = l->launch();
+		rc = l->launch(true);
 		g = &l->filling();
 		if (rc != 0) {
 			return rc;
@@ -432,6 +449,10 @@ int ofi_amd_net_link_create(uint32_t num_rails, int64_t eager_max_size, uint64_t
 		l->send_reqs.resize(OFI_AMD_MAX_SEND_REQUESTS);
 		l->recv_reqs.resize(OFI_AMD_MAX_REQUESTS);
 		l->flush_reqs.resize(OFI_AMD_MAX_REQUESTS);
+		l->flush_slots.assign((size_t)OFI_AMD_MAX_REQUESTS * OFI_AMD_WIRE_MAX_RAILS * 8, 0);
+		for (group_t &g : l->groups) {
+			g.flushes.reserve(OFI_AMD_MAX_REQUESTS);
+		}
 		for (uint32_t k = n_rx; k > 0; k--) {
 			l->rx_free.push_back(k - 1);
 		}
@@ -452,7 +473,6 @@ int ofi_amd_net_link_create(uint32_t num_rails, int64_t eager_max_size, uint64_t
 	if (rc == 0) rc = ofi_amd_gpu_mem_alloc(&l->rx_pool, (size_t)n_rx * kRxStride);
 	if (rc == 0) rc = ofi_amd_gpu_mem_alloc(&l->d_flush_buf, 64);
 	if (rc == 0) rc = ofi_amd_flush_buffer_fill(l->d_flush_buf, OFI_AMD_RDMA_FLUSH_SENTINEL, stream);
-	if (rc == 0) rc = l->flush_slots.alloc((size_t)OFI_AMD_MAX_REQUESTS * OFI_AMD_WIRE_MAX_RAILS * 64);
 	for (uint32_t k = 0; k < kGroups && rc == 0; k++) {
 		rc = l->groups[k].alloc();
 	}
@@ -474,7 +494,6 @@ int ofi_amd_net_link_destroy(ofi_amd_net_link_t *l)
 	for (group_t &g : l->groups) {
 		g.release();
 	}
-	l->flush_slots.release();
 	if (l->rx_pool) (void)ofi_amd_gpu_mem_free(l->rx_pool);
 	if (l->d_flush_buf) (void)ofi_amd_gpu_mem_free(l->d_flush_buf);
 	if (l->sc) (void)ofi_amd_send_comm_destroy(l->sc);
@@ -565,18 +584,12 @@ ncclResult_t ofi_amd_net_iflush(void *recvComm, int n, void **data, int *sizes, 
 	if (!q) {
 		return ncclSystemError;
 	}
-	/* the read-back goes behind everything launched so far; what the receives it covers wrote
-	 * has been launched, or their requests would not have completed */
-	uint8_t *slots = l->flush_slots.as<uint8_t>() + (size_t)id * OFI_AMD_WIRE_MAX_RAILS * 64;
-	std::memset(slots, 0, OFI_AMD_WIRE_MAX_RAILS * 64);
-	rc = ofi_amd_flush_post(l->d_flush_buf,
-				static_cast<uint8_t *>(l->flush_slots.dev) + (size_t)id * OFI_AMD_WIRE_MAX_RAILS * 64,
-				l->num_rails, l->stream);
-	if (rc != 0) {
-		return ofi_amd::nccl_result_of(rc);
-	}
+	/* the flush rides on the sentinel read-back of the next launch group, which goes behind
+	 * everything launched so far; what the receives it covers wrote has been launched, or their
+	 * requests would not have completed */
+	std::memset(&l->flush_slots[(size_t)id * OFI_AMD_WIRE_MAX_RAILS * 8], 0, OFI_AMD_WIRE_MAX_RAILS * 64);
+	l->filling().flushes.push_back(id);
 	l->st.flushes++;
-	l->st.launches++;
 	*request = q;
 	return ncclSuccess;
 }
@@ -608,7 +621,7 @@ ncclResult_t ofi_amd_net_test(void *request, int *done, int *sizes)
 			}
 		}
 	} else {
-		const uint8_t *slots = l->flush_slots.as<uint8_t>() + (size_t)q->id * OFI_AMD_WIRE_MAX_RAILS * 64;
+		const uint64_t *slots = &l->flush_slots[(size_t)q->id * OFI_AMD_WIRE_MAX_RAILS * 8];
 		rc = ofi_amd_recv_comm_flush_test(l->rcv, q->id, slots, l->num_rails, OFI_AMD_RDMA_FLUSH_SENTINEL, done);
 	}
 	if (rc == 0 && *done) {

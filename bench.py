@@ -864,6 +864,21 @@ def m_stats(lib, link):
     return st
 
 
+def entry_points_from_compiled_code():
+    """The net and RMA entry points driven at 64 requests in flight by compiled code through the reference's
+    own ncclNet_v12_t / ncclRma_v15_t structs (tests/host/integration_glue.cpp, mode `rate`; the binary is
+    built where the reference's headers are and travels with the tree).  A child process; None if the
+    binary is not there."""
+    import subprocess
+    exe = os.path.join(ROOT, "tests", "host", "bin", "integration_glue")
+    if not os.path.exists(exe):
+        return None
+    proc = subprocess.run([exe, "rate"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    if proc.returncode != 0:
+        raise RuntimeError("integration_glue rate failed: %s" % proc.stderr[-500:])
+    return json.loads(proc.stdout.strip().splitlines()[-1])
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -904,6 +919,11 @@ def main():
                 continue
             log(name)
             extra[name] = fn(lib, oracle, torch, np, args)
+
+    if not args.skip_extra and {"gin", "sendrecv"} & set(args.extra.split(",")):
+        compiled = entry_points_from_compiled_code()
+        if compiled is not None:
+            extra["entry_points_from_compiled_code"] = compiled
 
     baselines = {k: bounce[k] for k in ("cpu_all_cores", "per_buffer_copy_calls") if k in bounce}
     if baselines:

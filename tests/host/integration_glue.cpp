@@ -11,13 +11,17 @@
  *   integration_glue gpu    the patterns of the reference's tests/unit/gdrcopy.cpp:15-133 (a
  *                           2 MiB buffer written and read back whole, a 10-byte buffer written
  *                           and read back byte by byte) through the C++ class, plus offsets
- *                           and sizes around the class's CPU-store / copy-engine switch
+ *                           and sizes around the class's CPU-store / copy-engine switch; a message
+ *                           each way through the net table and a put-signal through the RMA table
+ *   integration_glue rate   messages and put-signals per second through the two tables, 64 in
+ *                           flight, as one JSON line
  */
 #include <cerrno>
 #include <cstddef>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <ctime>
 #include <vector>
 
 // [section 1]
@@ -440,6 +444,162 @@ static int gpu_checks()
 	return 0;
 }
 
+/* The two entry-point families driven from compiled code at NCCL's depth of 64 requests, through
+ * the reference's own structs: messages per second and payload rate of the in-process link and of
+ * the device fabric, without an interpreter between the calls.  One JSON line. */
+static double now_s()
+{
+	struct timespec t;
+	clock_gettime(CLOCK_MONOTONIC, &t);
+	return (double)t.tv_sec + 1e-9 * (double)t.tv_nsec;
+}
+
+static int rate_checks()
+{
+	CHECK(nccl_net_ofi_gpu_init() == 0);
+	const ncclNet_v12_t net = net_v12_table_with_this_librarys_data_path();
+	const ncclRma_v15_t rma_table = rma_table_with_this_librarys_data_path();
+	constexpr int kInFlight = 64;
+	printf("{");
+	{
+		ofi_amd_net_link_t *link = nullptr;
+		CHECK(ofi_amd_net_link_create(4, 8192, 0, 0, 0, nullptr, &link) == 0);
+		void *sComm = ofi_amd_net_link_send_comm(link), *rComm = ofi_amd_net_link_recv_comm(link);
+		const size_t sizes[3] = {4096, 1u << 20, 64u << 20};
+		printf("\"net_v12\": [");
+		for (int which = 0; which < 3; which++) {
+			const size_t bytes = sizes[which];
+			const int rounds = bytes <= 4096 ? 256 : (bytes <= (1u << 20) ? 32 : 2);
+			void *src = nullptr, *dst = nullptr;
+			CHECK(nccl_net_ofi_gpu_mem_alloc(&src, bytes * kInFlight) == 0);
+			CHECK(nccl_net_ofi_gpu_mem_alloc(&dst, bytes * kInFlight) == 0);
+			double best = 1e30;
+			for (int pass = 0; pass < 3; pass++) {
+				const double t0 = now_s();
+				for (int r = 0; r < rounds; r++) {
+					void *sreq[kInFlight] = {}, *rreq[kInFlight] = {}, *freq[kInFlight] = {};
+					void *mh = nullptr;
+					int tag = 1;
+					/* the sender is ahead, as in NCCL's pipelines: small messages go eager */
+					for (int k = 0; k < kInFlight; k++) {
+						CHECK(net.isend(sComm, (char *)src + k * bytes, bytes, tag, mh, nullptr, &sreq[k]) == ncclSuccess);
+					}
+					for (int k = 0; k < kInFlight; k++) {
+						void *d = (char *)dst + k * bytes;
+						size_t sz = bytes;
+						CHECK(net.irecv(rComm, 1, &d, &sz, &tag, &mh, nullptr, &rreq[k]) == ncclSuccess && rreq[k]);
+					}
+					for (int k = 0; k < kInFlight; k++) {
+						for (long spins = 0; !sreq[k] && spins < 100000000L; spins++) {
+							CHECK(net.isend(sComm, (char *)src + k * bytes, bytes, tag, mh, nullptr, &sreq[k]) == ncclSuccess);
+						}
+						CHECK(sreq[k]);
+					}
+					int open = 3 * kInFlight; /* a send, a receive and a flush per message */
+					for (long spins = 0; open > 0 && spins < 100000000L; spins++) {
+						for (int k = 0; k < kInFlight; k++) {
+							int done = 0;
+							if (sreq[k]) {
+								CHECK(net.test(sreq[k], &done, nullptr) == ncclSuccess);
+								if (done) { sreq[k] = nullptr; open--; }
+							}
+							if (rreq[k]) {
+								CHECK(net.test(rreq[k], &done, nullptr) == ncclSuccess);
+								if (done) {
+									rreq[k] = nullptr;
+									open--;
+									void *d = (char *)dst + k * bytes;
+									int isz = (int)bytes;
+									CHECK(net.iflush(rComm, 1, &d, &isz, &mh, &freq[k]) == ncclSuccess && freq[k]);
+								}
+							}
+							if (freq[k]) {
+								CHECK(net.test(freq[k], &done, nullptr) == ncclSuccess);
+								if (done) { freq[k] = nullptr; open--; }
+							}
+						}
+					}
+					CHECK(open == 0);
+				}
+				const double dt = now_s() - t0;
+				best = dt < best ? dt : best;
+			}
+			const double n = (double)rounds * kInFlight;
+			printf("%s{\"bytes\": %zu, \"messages\": %.0f, \"msgs_per_s\": %.1f, \"payload_gbs\": %.2f}", which ? ", " : "",
+			       bytes, n, n / best, n * (double)bytes / best / 1e9);
+			CHECK(nccl_net_ofi_gpu_mem_free(src) == 0 && nccl_net_ofi_gpu_mem_free(dst) == 0);
+		}
+		printf("], ");
+		CHECK(ofi_amd_net_link_destroy(link) == 0);
+	}
+	{
+		const size_t sizes[2] = {4096, 1u << 20};
+		printf("\"rma_v15\": [");
+		for (int which = 0; which < 2; which++) {
+			const size_t bytes = sizes[which];
+			const int n_ops = bytes <= 4096 ? 65536 : 8192;
+			void *src = nullptr, *dst = nullptr, *counters = nullptr;
+			CHECK(nccl_net_ofi_gpu_mem_alloc(&src, bytes * kInFlight) == 0 && nccl_net_ofi_gpu_mem_alloc(&dst, bytes * kInFlight) == 0 &&
+			      nccl_net_ofi_gpu_mem_alloc(&counters, 4096) == 0);
+			std::vector<uint8_t> zero(4096, 0);
+			CHECK(nccl_net_ofi_gpu_mem_copy_host_to_device(counters, zero.data(), 4096) == 0);
+			const uint64_t signal_base = 0x7f5500000000ull;
+			const ofi_amd_gin_signal_region_t region = {signal_base, 4096, counters};
+			const uint32_t ids[2] = {0, 1};
+			ofi_amd_devfab_t *fab = nullptr;
+			ofi_amd_gin_fabric_ops_t ops;
+			CHECK(ofi_amd_devfab_create(4, 256, 2, ids, &region, 1, nullptr, &fab) == 0 && ofi_amd_devfab_ops(fab, &ops) == 0);
+			ofi_amd_rma_ctx_t *rma = nullptr;
+			CHECK(ofi_amd_rma_ctx_create(2, 4, 131072, 64, &ops, 4096, 0, &rma) == 0);
+			CHECK(ofi_amd_devfab_on_ack(fab, [](void *ctx, uint32_t peer, uint64_t msg) {
+				      return ofi_amd_rma_ack_received(static_cast<ofi_amd_rma_ctx_t *>(ctx), peer, msg);
+			      }, rma) == 0);
+			const uint64_t keys[8] = {1, 2, 3, 4, 5, 6, 7, 8};
+			const uint64_t a_src[2] = {(uint64_t)(uintptr_t)src, (uint64_t)(uintptr_t)src};
+			const uint64_t a_dst[2] = {(uint64_t)(uintptr_t)dst, (uint64_t)(uintptr_t)dst};
+			const uint64_t a_sig[2] = {signal_base, signal_base};
+			ofi_amd_rma_mr_t *mr_src = nullptr, *mr_dst = nullptr, *mr_sig = nullptr;
+			CHECK(ofi_amd_rma_mr_create(rma, a_src[0], a_src, a_src, keys, &mr_src) == 0);
+			CHECK(ofi_amd_rma_mr_create(rma, a_dst[0], a_dst, a_dst, keys, &mr_dst) == 0);
+			CHECK(ofi_amd_rma_mr_create(rma, signal_base, a_sig, a_sig, keys, &mr_sig) == 0);
+			void *open_reqs[kInFlight] = {};
+			int head = 0, count = 0;
+			const double t0 = now_s();
+			for (int i = 0; i < n_ops; i++) {
+				const uint64_t off = (uint64_t)(i % kInFlight) * bytes;
+				void *req = nullptr;
+				CHECK(rma_table.iputSignal(rma, 0, off, mr_src, bytes, off, mr_dst, 1, 8 * (uint64_t)(i % 4), mr_sig, 1, 1,
+							   true, ncclRmaOptFlagsDefault, &req) == ncclSuccess && req);
+				open_reqs[(head + count++) % kInFlight] = req;
+				/* "test the oldest request; if it is not done, progress" (tests/functional/rma.cpp:316-330) */
+				for (long spins = 0; (count == kInFlight || (i == n_ops - 1 && count > 0)) && spins < 100000000L; spins++) {
+					int done = 0;
+					CHECK(rma_table.test(rma, open_reqs[head], &done) == ncclSuccess);
+					if (done) {
+						head = (head + 1) % kInFlight;
+						count--;
+					} else {
+						CHECK(rma_table.rmaProgress(rma) == ncclSuccess);
+					}
+				}
+			}
+			CHECK(count == 0 && ofi_amd_devfab_quiesce(fab, 0) == 0);
+			const double dt = now_s() - t0;
+			uint64_t slots[4] = {};
+			CHECK(ofi_amd_gpu_mem_copy_device_to_host(slots, counters, sizeof(slots)) == 0);
+			CHECK(slots[0] + slots[1] + slots[2] + slots[3] == (uint64_t)n_ops);
+			printf("%s{\"bytes\": %zu, \"operations\": %d, \"puts_per_s\": %.1f, \"payload_gbs\": %.2f}", which ? ", " : "", bytes,
+			       n_ops, n_ops / dt, (double)n_ops * (double)bytes / dt / 1e9);
+			CHECK(ofi_amd_rma_mr_destroy(mr_src) == 0 && ofi_amd_rma_mr_destroy(mr_dst) == 0 && ofi_amd_rma_mr_destroy(mr_sig) == 0);
+			CHECK(ofi_amd_rma_ctx_destroy(rma) == 0 && ofi_amd_devfab_destroy(fab) == 0);
+			CHECK(nccl_net_ofi_gpu_mem_free(src) == 0 && nccl_net_ofi_gpu_mem_free(dst) == 0 && nccl_net_ofi_gpu_mem_free(counters) == 0);
+		}
+		printf("]");
+	}
+	printf("}\n");
+	return 0;
+}
+
 int main(int argc, char **argv)
 {
 	if (argc == 2 && strcmp(argv[1], "link") == 0) {
@@ -448,6 +608,9 @@ int main(int argc, char **argv)
 	if (argc == 2 && strcmp(argv[1], "gpu") == 0) {
 		return gpu_checks();
 	}
-	fprintf(stderr, "usage: %s link|gpu\n", argv[0]);
+	if (argc == 2 && strcmp(argv[1], "rate") == 0) {
+		return rate_checks();
+	}
+	fprintf(stderr, "usage: %s link|gpu|rate\n", argv[0]);
 	return 2;
 }
