@@ -35,7 +35,7 @@ constexpr uint32_t kGroupsKeptBusy = 2; /* in flight before posts start gatherin
 constexpr uint32_t kGroupEntries = 512; /* table entries of a group's wire copies */
 constexpr uint32_t kGroupEager = 256;   /* eager copies of a group */
 constexpr uint32_t kMagic = 0x4e455451; /* marks a live request */
-constexpr uint32_t kMaxRxBuffers = 4096;
+constexpr uint32_t kMaxRxBuffers = 256; /* the receiving end queues at most 256 eager arrivals (ofi_amd_recv_comm_eager_arrival) */
 
 using ofi_amd::pinned_t;
 

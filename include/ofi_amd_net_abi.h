@@ -67,7 +67,8 @@ typedef struct {
  * may go eager when its size plus the 8-byte header fits, :5758-5764; negative = no eager protocol);
  * min_stripe_size and max_small_msg_size are the scheduler's thresholds (0 = the reference's
  * defaults 131072 and 64); rx_buffers is how many eager rx buffers the receiving end keeps
- * posted (0 = 256, at most 4096; 8320 bytes of device memory each).  `stream` carries every
+ * posted (0 = 256, which is also the most: the receiving end queues at most 256 eager arrivals; 8320 bytes of
+ * device memory each).  `stream` carries every
  * launch; it must outlive the link.  The calls on one link come from one thread (NCCL calls
  * each comm from one proxy thread).  -ENODEV without a GPU.
  */

@@ -259,5 +259,6 @@ def test_net_entry_points_check_their_arguments_without_a_link(lib):
     assert lib.ofi_amd_net_test(not_a_request, ctypes.byref(done), None) == internal
     assert lib.ofi_amd_net_link_create(0, 8192, 0, 0, 0, None, ctypes.byref(req)) == -errno.EINVAL
     assert lib.ofi_amd_net_link_create(4, 16384, 0, 0, 0, None, ctypes.byref(req)) == -errno.EINVAL
+    assert lib.ofi_amd_net_link_create(4, 8192, 0, 0, 257, None, ctypes.byref(req)) == -errno.EINVAL
     assert lib.ofi_amd_net_link_destroy(None) == -errno.EINVAL
     assert lib.ofi_amd_net_link_send_comm(None) is None and lib.ofi_amd_net_link_recv_comm(None) is None
