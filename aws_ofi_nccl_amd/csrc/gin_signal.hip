@@ -33,12 +33,27 @@ __global__ __launch_bounds__(256) void gin_signal_apply_kernel(
 	}
 	const ofi_amd_gin_signal_work_t w = work[i];
 	uint64_t *slot = nullptr;
+	/* The window is found by its base; the counter by its address inside the window, which may
+	 * continue through the regions listed next while each begins where the one before it ends
+	 * (a window backed by several allocations: the reference looks the segment up by address
+	 * too, ensure_signal_seg, src/rdma/gin/nccl_ofi_gin.cpp:1038-1122, 1156-1166). */
 	for (uint32_t r = 0; r < regions.n; r++) {
-		if (w.base == regions.base[r] && w.offset <= regions.size[r] &&
-		    regions.size[r] - w.offset >= 8) {
-			slot = regions.counters[r] + (w.offset >> 3);
-			break;
+		if (w.base != regions.base[r]) {
+			continue;
 		}
+		uint64_t off = w.offset;
+		for (uint32_t k = r;; k++) {
+			if (off <= regions.size[k] && regions.size[k] - off >= 8) {
+				slot = regions.counters[k] + (off >> 3);
+				break;
+			}
+			if (off < regions.size[k] || k + 1 >= regions.n ||
+			    regions.base[k + 1] != regions.base[k] + regions.size[k]) {
+				break; /* a counter across the end of a segment, or past the window */
+			}
+			off -= regions.size[k];
+		}
+		break;
 	}
 	if (slot == nullptr || (w.offset & 7u) != 0) {
 		if (rejected) {

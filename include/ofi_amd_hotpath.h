@@ -656,7 +656,11 @@ int ofi_amd_gin_rx_cursors(const ofi_amd_gin_rx_t *rx, uint32_t peer, uint32_t *
 			   uint32_t *next_seq);
 
 /* A registered signal region: initiators address it as `base`; its counters live at
- * d_counters (device memory), `size` bytes. */
+ * d_counters (device memory), `size` bytes.  A window backed by several allocations (the
+ * reference finds the segment of a counter by its address, ensure_signal_seg,
+ * src/rdma/gin/nccl_ofi_gin.cpp:1038-1122) is listed as consecutive regions, each beginning
+ * where the one before it ends: an item addressed by the first one's base and an offset beyond
+ * its size lands in the region that holds base + offset.  A counter never straddles two. */
 typedef struct {
 	uint64_t base;
 	uint64_t size;

@@ -259,7 +259,8 @@ void oracle_gin_rx_cursors(const oracle_gin_rx_t *rx, uint32_t peer, uint32_t *r
 
 /* apply_and_complete + apply_signal_work, :1425-1479 and :1193-1256: entries of one batch
  * that hit the same (base, offset) fold into the first of them; each lead is applied with
- * one read-modify-write.  counters[r] is the 8-byte-counter array registered at bases[r].
+ * one read-modify-write.  counters[r] is the 8-byte-counter array registered at bases[r];
+ * consecutive regions that are contiguous in address are the segments of one window.
  * Returns the number of read-modify-writes, or -22 for an entry outside every region. */
 int oracle_gin_signal_apply(const oracle_gin_signal_work_t *batch, uint32_t n, const uint64_t *bases,
 			    const uint64_t *sizes, uint64_t *const *counters, uint32_t n_regions)
@@ -284,18 +285,33 @@ int oracle_gin_signal_apply(const oracle_gin_signal_work_t *batch, uint32_t n, c
 		if (lead[i] != i) {
 			continue;
 		}
-		uint32_t r;
+		/* the window by its base address (the MR lookup, :1140-1152), the segment by the counter's
+		 * address inside it (ensure_signal_seg, :1038-1122: a window may be backed by several
+		 * allocations); regions listed one after the other, each beginning where the one before
+		 * it ends, are the segments of one window */
+		uint32_t r, seg = n_regions;
+		uint64_t off = batch[i].offset;
 		for (r = 0; r < n_regions; r++) {
-			if (batch[i].base == bases[r] && batch[i].offset + 8 <= sizes[r]) {
+			if (batch[i].base == bases[r]) {
 				break;
 			}
 		}
-		if (r == n_regions || (batch[i].offset & 7) != 0) {
+		for (uint32_t k = r; k < n_regions; k++) {
+			if (off <= sizes[k] && sizes[k] - off >= 8) {
+				seg = k;
+				break;
+			}
+			if (off < sizes[k] || k + 1 >= n_regions || bases[k + 1] != bases[k] + sizes[k]) {
+				break;
+			}
+			off -= sizes[k];
+		}
+		if (seg == n_regions || (batch[i].offset & 7) != 0) {
 			free(lead);
 			free(sum);
 			return -22;
 		}
-		counters[r][batch[i].offset / 8] += sum[i];
+		counters[seg][off / 8] += sum[i];
 		rmw++;
 	}
 	free(lead);

@@ -155,6 +155,61 @@ def test_several_regions_and_rejects(lib, oracle, gpu):
         assert got[-1] == 0
 
 
+def test_windows_backed_by_several_segments(lib, oracle, gpu):
+    """Four windows of one to four contiguous segments each (16 regions, every segment an allocation of its
+    own with a canary word behind it): items addressed by a window's base and an offset anywhere in the
+    window, or by a later segment's own base, against the oracle; items past a window, straddling
+    nothing (a counter never straddles: sizes are multiples of 8) and misaligned ones are rejected."""
+    rng = np.random.default_rng(47)
+    windows, regions = [], []                      # windows: (base, [segment sizes in counters])
+    for w in range(4):
+        base = SIG_BASE + (w << 32)
+        segs = [int(rng.integers(1, 60)) for _ in range(1 + w)] + ([int(rng.integers(1, 60)) for _ in range(3 - w)] if w == 0 else [])
+        windows.append((base, len(regions), segs))
+        at = base
+        for sz in segs:
+            regions.append((at, sz))
+            at += 8 * sz
+    while len(regions) < 16:                       # unrelated single regions far away
+        regions.append((SIG_BASE + (len(regions) << 36), int(rng.integers(1, 60))))
+    host = [np.zeros(sz, dtype=np.uint64) for _b, sz in regions]
+    items, n_bad = [], 0
+    for i in range(20000):
+        base, first, segs = windows[int(rng.integers(0, len(windows)))]
+        total = sum(segs)
+        kind = rng.random()
+        if kind < 0.85:
+            slot = int(rng.integers(0, total))
+            start = int(rng.integers(0, len(segs))) if rng.random() < 0.3 else 0    # address by a later segment's base
+            skip = sum(segs[:start])
+            if slot < skip:
+                start, skip = 0, 0
+            v = int(rng.integers(0, 1 << 64, dtype=np.uint64))
+            items.append((base + 8 * skip, 8 * (slot - skip), v, 0, i & 0x1FFF, 1))
+            k, rem = 0, slot
+            while rem >= segs[k]:
+                rem -= segs[k]
+                k += 1
+            host[first + k][rem] = np.uint64((int(host[first + k][rem]) + v) % (1 << 64))
+        elif kind < 0.93:
+            items.append((base, 8 * total, 1, 0, 0, 1)); n_bad += 1                  # one past the window
+        else:
+            items.append((base, 8 * int(rng.integers(0, total)) + 4, 1, 0, 0, 1)); n_bad += 1   # misaligned
+    work = work_array(items)
+    good = work_array([it for it in items if it[1] % 8 == 0 and not any(it[0] == b and it[1] == 8 * sum(sg) for b, _f, sg in windows)])
+    oracle_host = [np.zeros(sz, dtype=np.uint64) for _b, sz in regions]
+    oracle_apply(oracle, good, [(b, h) for (b, _sz), h in zip(regions, oracle_host)])
+    for a, b in zip(host, oracle_host):
+        assert np.array_equal(a, b)                # the oracle agrees with the image built by hand above
+    dev = [(b, torch.zeros(sz + 1, dtype=torch.int64, device="cuda")) for b, sz in regions]
+    rejected = torch.zeros(1, dtype=torch.int32, device="cuda")
+    assert gpu_apply(lib, work, [(b, t[:-1]) for b, t in dev], rejected) == 0
+    assert int(rejected.item()) == n_bad and n_bad > 1000
+    for (b, t), h in zip(dev, host):
+        got = _gpu.to_host(t, np.uint64)
+        assert np.array_equal(got[:-1], h) and got[-1] == 0
+
+
 def test_work_items_in_pinned_host_memory(lib, oracle, gpu):
     """The proxy writes work items into pinned host memory and launches straight from there."""
     n = 5000

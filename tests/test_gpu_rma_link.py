@@ -29,17 +29,22 @@ vp = ctypes.c_void_p
 class RmaLink:
     """createContext / regMrSym of a two-sided set-up, collapsed into one process."""
 
-    def __init__(self, lib, nranks=2, rails=4, window=8 << 20, sq_depth=256, pool=4096):
+    def __init__(self, lib, nranks=2, rails=4, window=8 << 20, sq_depth=256, pool=4096, segments=1, seg_size=4096):
         self.lib, self.nranks = lib, nranks
         self.src = torch.randint(0, 256, (window,), dtype=torch.uint8, device="cuda")
         self.dst = [torch.full((window,), 0xCD, dtype=torch.uint8, device="cuda") for _ in range(nranks)]
-        self.counters = [torch.zeros(512, dtype=torch.int64, device="cuda") for _ in range(nranks)]
+        # a rank's signal window is `segments` regions side by side in its address range, each backed by
+        # an allocation of its own (counters[r] is the first one's, segment_counters[r][k] the k-th's)
+        self.segment_counters = [[torch.zeros(seg_size // 8, dtype=torch.int64, device="cuda") for _ in range(segments)]
+                                 for _ in range(nranks)]
+        self.counters = [segs[0] for segs in self.segment_counters]
         torch.cuda.synchronize()
-        regions = (m.GinSignalRegion * nranks)(*[
-            m.GinSignalRegion(SIGNAL_BASE + (r << 20), 4096, self.counters[r].data_ptr()) for r in range(nranks)])
+        flat = [m.GinSignalRegion(SIGNAL_BASE + (r << 24) + k * seg_size, seg_size, self.segment_counters[r][k].data_ptr())
+                for r in range(nranks) for k in range(segments)]
+        regions = (m.GinSignalRegion * len(flat))(*flat)
         ids = (ctypes.c_uint32 * nranks)(*range(nranks))
         self.fab = vp()
-        rc = lib.ofi_amd_devfab_create(rails, sq_depth, nranks, ids, regions, nranks, _gpu.stream(), ctypes.byref(self.fab))
+        rc = lib.ofi_amd_devfab_create(rails, sq_depth, nranks, ids, regions, len(flat), _gpu.stream(), ctypes.byref(self.fab))
         assert rc == 0, rc
         self.ops = m.GinFabricOps()
         assert lib.ofi_amd_devfab_ops(self.fab, ctypes.byref(self.ops)) == 0
@@ -61,7 +66,7 @@ class RmaLink:
 
         self.mr_src = reg(self.src.data_ptr(), [self.src.data_ptr()] * nranks)
         self.mr_dst = reg(self.dst[0].data_ptr(), [t.data_ptr() for t in self.dst])
-        self.mr_sig = reg(SIGNAL_BASE, [SIGNAL_BASE + (r << 20) for r in range(nranks)])
+        self.mr_sig = reg(SIGNAL_BASE, [SIGNAL_BASE + (r << 24) for r in range(nranks)])
         self.open = []
 
     def put(self, rank, src_off, dst_off, size, signal=None, flags=0):
@@ -70,7 +75,7 @@ class RmaLink:
             rc = self.lib.ofi_amd_rma_iput(self.ctx, 0, src_off, self.mr_src, size, dst_off, self.mr_dst, rank, flags,
                                            ctypes.byref(req))
         else:
-            slot, value, op = signal
+            slot, value, op = signal            # slot: index of the 8-byte counter within the rank's window
             rc = self.lib.ofi_amd_rma_iputSignal(self.ctx, 0, src_off, self.mr_src, size, dst_off, self.mr_dst, rank,
                                                  8 * slot, self.mr_sig, value, op, True, flags, ctypes.byref(req))
         assert rc == ncclSuccess and req.value, rc
@@ -242,4 +247,34 @@ def test_more_operations_than_a_window_holds_live_on_the_targets_acks(lib, gpu):
     assert st.acks > 0 and st.work_items <= n and st.metas == n
     window = (peer.tx_head - peer.tx_tail) & 0x3FFF
     assert window < 8192
+    link.close()
+
+
+def test_signal_window_of_two_segments_with_a_payload_across_the_middle(lib, gpu):
+    """tests/functional/rma_multiseg_signal.cpp:285-405: the signal window is one address range backed by two
+    allocations (the proxy there maps each segment on demand; here each is a region with counters of its
+    own), 16 put-signals increment the first counter of segment 0 and 16 the first counter of segment 1, on
+    every peer, each carrying 64 KiB that start 32 KiB before the 2 MiB mark of the payload windows."""
+    seg = 2 << 20
+    nranks = 3
+    link = RmaLink(lib, nranks=nranks, segments=2, seg_size=seg)
+    pay, pay_off = 64 << 10, seg - (32 << 10)
+    for dst in range(1, nranks):
+        for _ in range(16):
+            link.put(dst, pay_off, pay_off, pay, signal=(0, 1, SIGNAL_INC))
+            link.put(dst, pay_off, pay_off, pay, signal=(seg // 8, 1, SIGNAL_INC))
+    link.poll_all()
+    for dst in range(1, nranks):
+        link.wait_signal(dst, 0, 16)
+        for _ in range(1_000_000):
+            assert lib.ofi_amd_rma_rmaProgress(link.ctx) == ncclSuccess
+            if int(link.segment_counters[dst][1][0].item()) == 16:
+                break
+        assert int(link.segment_counters[dst][1][0].item()) == 16
+        assert int(link.segment_counters[dst][0].sum().item()) == 16 and int(link.segment_counters[dst][1].sum().item()) == 16
+        # "signals are delivered after the payload writes": the data is there once the counters are
+        assert torch.equal(link.dst[dst][pay_off:pay_off + pay], link.src[pay_off:pay_off + pay])
+        assert int((link.dst[dst][:pay_off] != 0xCD).sum()) == 0 and int((link.dst[dst][pay_off + pay:] != 0xCD).sum()) == 0
+    assert int(link.segment_counters[0][0].sum().item()) == 0 and int((link.dst[0] != 0xCD).sum()) == 0
+    assert _gpu.fetch_async_errors(lib) == 0
     link.close()

@@ -423,6 +423,30 @@ def test_batch_apply_rejects_unknown_region_and_misaligned_offset(oracle):
     assert not c0.any()
 
 
+def test_batch_apply_finds_the_segment_of_a_window_backed_by_several_allocations(oracle):
+    """ensure_signal_seg (src/rdma/gin/nccl_ofi_gin.cpp:1038-1122, 1156-1166): the window is found by its
+    base, the segment by the counter's address.  Worked by hand: a window of two segments (32 and 16
+    bytes, contiguous) followed by an unrelated region 1000 bytes further on."""
+    bases = (ctypes.c_uint64 * 3)(SIG_BASE, SIG_BASE + 32, SIG_BASE + 1000)
+    sizes = (ctypes.c_uint64 * 3)(32, 16, 64)
+    c = [np.zeros(4, dtype=np.uint64), np.zeros(2, dtype=np.uint64), np.zeros(8, dtype=np.uint64)]
+    ptrs = (ctypes.c_void_p * 3)(*[x.ctypes.data for x in c])
+
+    def apply(base, offset, value):
+        batch = (GinSignalWork * 1)(GinSignalWork(base, offset, value, 0, 0, 1))
+        return oracle.oracle_gin_signal_apply(batch, 1, bases, sizes, ptrs, 3)
+
+    assert apply(SIG_BASE, 0, 1) == 1 and apply(SIG_BASE, 24, 2) == 1       # segment 0, first and last counter
+    assert apply(SIG_BASE, 32, 3) == 1 and apply(SIG_BASE, 40, 4) == 1      # segment 1 through the window's base
+    assert apply(SIG_BASE + 32, 8, 5) == 1                                  # ... and through its own
+    assert apply(SIG_BASE, 48, 9) == -22                                    # past the window's last segment
+    assert apply(SIG_BASE, 1000, 9) == -22                                  # the next region is not contiguous
+    assert apply(SIG_BASE + 32, 16, 9) == -22                               # past segment 1 from its own base
+    assert apply(SIG_BASE, 36, 9) == -22                                    # misaligned, in segment 1
+    assert apply(SIG_BASE + 1000, 56, 6) == 1 and apply(SIG_BASE + 1000, 64, 9) == -22
+    assert c[0].tolist() == [1, 0, 0, 2] and c[1].tolist() == [3, 9, 0][:2] and c[2].tolist() == [0] * 7 + [6]
+
+
 # ---- the product's host receiver against the oracle ----
 
 def product_api(lib):
