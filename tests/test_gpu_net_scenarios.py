@@ -25,7 +25,8 @@ INTERLEAVED = [0, 1, 2, 3, 4, 5, 6, 1, 7, 0, 2, 3, 4, 5, 6, 7]   # T17 / T18
 
 
 def scenarios():
-    """name -> (messages as (size, tag), receives as (tags, sizes), receiver late?, (eager, write) or None)"""
+    """name -> (messages as (size, tag), receives as (tags, sizes), receiver late?, (eager, write) or None
+    [, sender sizes checked?])"""
     s = {}
     s["t5_single_eager_late"] = ([(E, 1)], [([1], [E])], True, (1, 0))
     s["t6_single_early"] = ([(E, 1)], [([1], [E])], False, (0, 1))
@@ -60,6 +61,21 @@ def scenarios():
                                                  [([1], [E]), ([50, 51], [E, E]), ([1], [E]), ([60, 61], [E, E])], True, None)
     s["t25_rotated_queue"] = ([(E, 30), (E, 40), (L, 31), (L, 20)], [([30, 31], [E, L]), ([20], [L]), ([40], [E])], True,
                               (2, 2))
+    # tests/functional/grouped_recv.cpp:158-240: n sends of 1024 * (i + 1) bytes, one tag, one grouped receive.
+    # An eager send looks its receive-buffer length up by tag (get_ctrl_msg_buff_len,
+    # src/nccl_ofi_rdma.cpp:2183-2196), which finds the group's first entry of that tag: with one tag for all
+    # sub-receives the sender reports min(size, first buffer); the data and the receiver's sizes are right
+    # and the reference's test does not read the sender's size ("sender sizes unchecked" below).
+    for n in (1, 2, 4, 8):
+        for late in (True, False):
+            s["grouped_one_tag_growing_sizes_n%d_%s" % (n, "late" if late else "early")] = (
+                [(1024 * (i + 1), 1) for i in range(n)], [([1] * n, [1024 * (i + 1) for i in range(n)])], late, None,
+                not late)
+    # grouped_recv.cpp:666-671: receive [tag 8] then receive [tags 0..7]; sends 0, 8, 1, 2, .. 7
+    s["grouped_multi_tag_send_before_its_group"] = ([(L, t) for t in (0, 8, 1, 2, 3, 4, 5, 6, 7)],
+                                                    [([8], [L]), (list(range(8)), [L] * 8)], False, (0, 9))
+    s["zero_length_messages"] = ([(0, 5), (E, 5), (0, 6)], [([5], [E]), ([5, 6], [E, E])], True, (3, 0))
+    s["receive_buffer_smaller_than_the_message"] = ([(E, 1), (L, 2)], [([1], [100]), ([2], [5000])], True, (1, 1))
     return s
 
 
@@ -68,10 +84,11 @@ SCENARIOS = scenarios()
 
 @pytest.mark.parametrize("name", sorted(SCENARIOS))
 def test_kth_send_of_a_tag_lands_in_the_kth_receive_of_that_tag(lib, gpu, name):
-    msgs, recvs, late, split = SCENARIOS[name]
+    msgs, recvs, late, split = SCENARIOS[name][:4]
+    sender_sizes_checked = SCENARIOS[name][4] if len(SCENARIOS[name]) > 4 else True
     link = Link(lib)
     rng = np.random.default_rng(len(name) * 131 + len(msgs))
-    srcs = [torch.from_numpy(rng.integers(0, 256, size, dtype=np.uint8)).cuda() for size, _ in msgs]
+    srcs = [torch.from_numpy(rng.integers(0, 256, max(size, 1), dtype=np.uint8)).cuda() for size, _ in msgs]
     dsts = [[torch.full((cap + 64,), 0xCD, dtype=torch.uint8, device="cuda") for cap in sizes] for _, sizes in recvs]
     torch.cuda.synchronize()
     recv_reqs = []
@@ -140,7 +157,9 @@ def test_kth_send_of_a_tag_lands_in_the_kth_receive_of_that_tag(lib, gpu, name):
         got = dsts[r][sub].cpu().numpy()
         assert np.array_equal(got[:moved], srcs[idx].cpu().numpy()[:moved]), (name, idx, tag, r, sub)
         assert np.all(got[moved:] == 0xCD), (name, idx, "wrote beyond the message")
-        assert recv_sizes[r][sub] == moved and send_sizes[idx] == moved, (name, idx, recv_sizes[r], send_sizes[idx])
+        assert recv_sizes[r][sub] == moved, (name, idx, recv_sizes[r])
+        if sender_sizes_checked:
+            assert send_sizes[idx] == moved, (name, idx, send_sizes[idx])
     assert used == {(r, sub) for r, (tags, _) in enumerate(recvs) for sub in range(len(tags))}
 
     st = link.stats()
@@ -153,4 +172,74 @@ def test_kth_send_of_a_tag_lands_in_the_kth_receive_of_that_tag(lib, gpu, name):
     assert rs.num_inflight_reqs == 0 and rs.eager_pending == 0
     assert ss.next_msg_seq_num == rs.next_msg_seq_num
     assert ss.n_ctrl_received == rs.n_ctrl_sent == len(recvs)
+    link.close()
+
+
+GROUPED_PATTERN = [(8, 20), (3, 1), (8, 10), (4, 1), (1, 1), (8, 10), (7, 1), (5, 1), (8, 4), (2, 1),
+                   (1, 1), (8, 4), (7, 1)]          # (sends per receive, receives), grouped_recv.cpp:255-258
+
+
+def test_grouped_receives_in_the_alltoall_pattern(lib, gpu):
+    """tests/functional/grouped_recv.cpp:242-420, the production alltoall trace shape: phases of grouped
+    receives of 1..8 sub-receives, 256 KiB sends into 512 KiB buffers, the receiver keeping a window of 16
+    receives posted ahead, the sender going round its queue; 414 messages, every one checked."""
+    link = Link(lib)
+    msgs, recvs = [], []
+    for per, count in GROUPED_PATTERN:
+        for _ in range(count):
+            recvs.append((list(range(per)), [524288] * per))
+            msgs += [(262144, t) for t in range(per)]
+    rng = np.random.default_rng(3)
+    pool = torch.from_numpy(rng.integers(0, 256, 262144 + len(msgs), dtype=np.uint8)).cuda()
+    dsts = [[torch.full((524288 + 64,), 0xCD, dtype=torch.uint8, device="cuda") for _ in tags] for tags, _ in recvs]
+    torch.cuda.synchronize()
+    # message i is the 256 KiB of `pool` that start at byte i: all different, one allocation
+    recv_reqs, recv_sizes, posted = {}, {}, 0
+    send_reqs, send_sizes = {}, {}
+    queue = list(range(len(msgs)))
+    for _ in range(200_000):
+        while posted < len(recvs) and len(recv_reqs) < 16:
+            tags, sizes = recvs[posted]
+            recv_reqs[posted] = link.irecv(dsts[posted], sizes, tags)
+            posted += 1
+        blocked, again = set(), []
+        for idx in queue:
+            size, tag = msgs[idx]
+            if tag in blocked:
+                again.append(idx)
+                continue
+            req = link.isend(pool, size, tag, offset=idx)
+            if req is None:
+                blocked.add(tag)
+                again.append(idx)
+            else:
+                send_reqs[idx] = req
+        queue = again
+        for idx in list(send_reqs):
+            done, sz = link.test(send_reqs[idx])
+            if done:
+                send_sizes[idx] = sz[0]
+                del send_reqs[idx]
+        for r in list(recv_reqs):
+            done, sz = link.test(recv_reqs[r], len(recvs[r][0]))
+            if done:
+                recv_sizes[r] = sz
+                link.flush(dsts[r], recvs[r][1])
+                del recv_reqs[r]
+        if not queue and not send_reqs and not recv_reqs and posted == len(recvs):
+            break
+    assert len(send_sizes) == len(msgs) and len(recv_sizes) == len(recvs)
+    assert all(v == 262144 for v in send_sizes.values())
+    torch.cuda.synchronize()
+    host = pool.cpu().numpy()
+    idx = 0
+    for r, (tags, _) in enumerate(recvs):          # messages were generated receive by receive, tag by tag
+        assert recv_sizes[r] == [262144] * len(tags)
+        for sub in range(len(tags)):
+            got = dsts[r][sub].cpu().numpy()
+            assert np.array_equal(got[:262144], host[idx:idx + 262144]), (r, sub)
+            assert np.all(got[262144:] == 0xCD)
+            idx += 1
+    st = link.stats()
+    assert st.write_sends == len(msgs) and st.eager_sends == 0 and st.rdma_writes == 2 * len(msgs)
     link.close()
