@@ -318,3 +318,31 @@ def test_same_bytes_and_protocol_split_as_the_one_call_loop_back(lib, gpu):
             assert torch.equal(a[:size], b[:size])
     assert _gpu.fetch_async_errors(lib) == 0
     link.close()
+
+
+def test_link_closed_with_requests_in_flight(lib, gpu):
+    """tests/functional/inflight_close.cpp: NUM_REQUESTS sends and receives of 1 MiB are posted and the comms
+    are closed without waiting for them.  Here: the link is destroyed with requests open, some launched and
+    some not, three times over; destruction waits for what was launched and a new link works afterwards."""
+    for it in range(3):
+        link = Link(lib)
+        srcs, dsts = buffers([1 << 20] * NUM_REQUESTS, [1 << 20] * NUM_REQUESTS, seed=it)
+        reqs = [link.irecv([dsts[i]], [1 << 20]) for i in range(NUM_REQUESTS)]
+        reqs += [link.isend(srcs[i], 1 << 20) for i in range(NUM_REQUESTS)]
+        assert all(q is not None for q in reqs)
+        if it:
+            link.test(reqs[0])                      # launches the first group; the rest may still be gathering
+            for i in range(4):                      # a few more posts behind the launched group
+                link.irecv([dsts[i]], [1 << 20])
+                assert link.isend(srcs[i], 1 << 20) is not None
+        link.close()
+        torch.cuda.synchronize()
+    link = Link(lib)
+    srcs, dsts = buffers([4096, 1 << 20], [4096, 1 << 20], seed=9)
+    s0 = link.isend(srcs[0], 4096)
+    r = [link.irecv([dsts[i]], [srcs[i].numel()]) for i in range(2)]
+    s1 = link.isend(srcs[1], 1 << 20)
+    poll_all(link, [s0, s1], r, dsts, [4096, 1 << 20], [4096, 1 << 20], [4096, 1 << 20])
+    check_bytes(srcs, dsts, [4096, 1 << 20], [4096, 1 << 20])
+    link.close()
+    assert _gpu.fetch_async_errors(lib) == 0

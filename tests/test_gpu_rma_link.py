@@ -278,3 +278,29 @@ def test_signal_window_of_two_segments_with_a_payload_across_the_middle(lib, gpu
     assert int(link.segment_counters[0][0].sum().item()) == 0 and int((link.dst[0] != 0xCD).sum()) == 0
     assert _gpu.fetch_async_errors(lib) == 0
     link.close()
+
+
+def test_context_and_fabric_torn_down_with_operations_in_flight(lib, gpu):
+    """The RMA side of tests/functional/inflight_close.cpp: operations posted, some launched, none waited
+    for; the context is destroyed, then the fabric (which waits for what it launched), and a fresh pair
+    works afterwards."""
+    for it in range(3):
+        link = RmaLink(lib)
+        for i in range(64):
+            link.put(1, 0, i << 16, 1 << 16, signal=(i % 4, 1, SIGNAL_INC))
+        if it:
+            assert lib.ofi_amd_rma_rmaProgress(link.ctx) == ncclSuccess      # launches a group
+            for i in range(8):
+                link.put(1, 0, i << 16, 1 << 16)
+        for h in (link.mr_src, link.mr_dst, link.mr_sig):
+            assert lib.ofi_amd_rma_mr_destroy(h) == 0
+        assert lib.ofi_amd_rma_ctx_destroy(link.ctx) == 0
+        assert lib.ofi_amd_devfab_destroy(link.fab) == 0
+        torch.cuda.synchronize()
+    link = RmaLink(lib)
+    link.put(1, 0, 0, 5000, signal=(0, 1, SIGNAL_INC))
+    link.poll_all()
+    link.wait_signal(1, 0, 1)
+    assert torch.equal(link.dst[1][:5000], link.src[:5000])
+    link.close()
+    assert _gpu.fetch_async_errors(lib) == 0
