@@ -957,6 +957,10 @@ def main():
         "gin_derive_puts_per_s": extra.get("gin", {}).get("drain_and_derive_wire", {}).get("descs_per_s"),
         # the same through the transmit engine, the in-process fabric, the receiver and the device copies
         "gin_end_to_end_puts_per_s": extra.get("gin", {}).get("loopback", {}).get("puts_per_s"),
+        # ... with a progress call after every 64th operation instead of after every one: the cadence of the
+        # reference's own test (64 puts and 64 put-signals before the first progress call, tests/functional/rma.cpp)
+        "gin_end_to_end_puts_per_s_progress_every_64": extra.get("gin", {}).get("loopback_progress_every_64", {}).get(
+            "puts_per_s"),
         "extra": extra,
     }
     print(json.dumps(line))
