@@ -208,7 +208,30 @@ class NetLinkStats(ctypes.Structure):
     """ofi_amd_net_link_stats_t"""
     _fields_ = [(k, c_u64) for k in ("isend_calls", "isend_again", "eager_sends", "write_sends", "rdma_writes",
                                      "payload_bytes", "irecv_calls", "flushes", "launches", "copy_entries",
-                                     "eager_copies", "progress_calls")]
+                                     "eager_copies", "progress_calls", "posts_refused")]
+
+
+class NetPost(ctypes.Structure):
+    """ofi_amd_net_post_t"""
+    _fields_ = [("kind", c_u32), ("rail", c_u32), ("context", c_u32), ("imm", c_u32), ("src", c_u64), ("len", c_u64),
+                ("dest", c_u64), ("key", c_u64), ("hdr", ctypes.c_uint8 * 8)]
+
+
+class NetCqe(ctypes.Structure):
+    """ofi_amd_net_cqe_t"""
+    _fields_ = [("kind", c_u32), ("context", c_u32), ("imm", c_u32), ("pad", c_u32), ("len", c_u64), ("rx_cookie", c_u64),
+                ("hdr", ctypes.c_uint8 * 8)]
+
+
+NET_POST_FN = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(NetPost))
+NET_CQ_READ_FN = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(NetCqe), c_u32)
+NET_REPOST_RX_FN = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, c_u64)
+
+
+class NetFabricOps(ctypes.Structure):
+    """ofi_amd_net_fabric_ops_t"""
+    _fields_ = [("post", NET_POST_FN), ("cq_read", NET_CQ_READ_FN), ("repost_rx", NET_REPOST_RX_FN),
+                ("end", ctypes.c_void_p)]
 
 
 class SendrecvLoopbackStats(ctypes.Structure):
@@ -406,6 +429,18 @@ PROTOTYPES = {
     "ofi_amd_rma_test": (ctypes.c_int, [c_vp, c_vp, ctypes.POINTER(ctypes.c_int)]),
     "ofi_amd_rma_rmaProgress": (ctypes.c_int, [c_vp]),
     # include/ofi_amd_net_abi.h: an in-process link, then the data-path members of ncclNet_vN_t
+    "ofi_amd_net_send_comm_create": (ctypes.c_int, [c_u32, ctypes.c_int64, c_u64, c_u64, ctypes.POINTER(NetFabricOps),
+                                                    ctypes.POINTER(c_vp)]),
+    "ofi_amd_net_send_comm_mailbox": (c_vp, [c_vp]),
+    "ofi_amd_net_recv_comm_create": (ctypes.c_int, [c_u32, ctypes.POINTER(NetFabricOps), c_vp, c_vp,
+                                                    ctypes.POINTER(c_vp)]),
+    "ofi_amd_net_comm_destroy": (ctypes.c_int, [c_vp]),
+    "ofi_amd_netfab_create": (ctypes.c_int, [c_u32, c_u32, c_vp, ctypes.POINTER(c_vp)]),
+    "ofi_amd_netfab_destroy": (ctypes.c_int, [c_vp]),
+    "ofi_amd_netfab_ops": (ctypes.c_int, [c_vp, ctypes.POINTER(NetFabricOps), ctypes.POINTER(NetFabricOps)]),
+    "ofi_amd_netfab_rx_pool": (c_vp, [c_vp]),
+    "ofi_amd_netfab_connect": (ctypes.c_int, [c_vp, c_vp]),
+    "ofi_amd_netfab_counts": (ctypes.c_int, [c_vp, ctypes.POINTER(c_u64), ctypes.POINTER(c_u64)]),
     "ofi_amd_net_link_create": (ctypes.c_int, [c_u32, ctypes.c_int64, c_u64, c_u64, c_u32, c_vp, ctypes.POINTER(c_vp)]),
     "ofi_amd_net_link_destroy": (ctypes.c_int, [c_vp]),
     "ofi_amd_net_link_send_comm": (c_vp, [c_vp]),

@@ -41,6 +41,100 @@
 extern "C" {
 #endif
 
+/* ---- the fabric under the two comms: what libfabric is to the reference ---- */
+
+/* What a comm asks of the fabric (rdma_send_req::post / post_eager, src/nccl_ofi_rdma.cpp:2368-2496;
+ * rdma_recv_req::post of the control message, :2566-2615; rdma_flush_req::post, :2664-2713). */
+#define OFI_AMD_NET_POST_EAGER 1 /* sending end: one send of the 8-byte header `hdr` followed by `len` bytes at `src`, immediate data `imm` (fi_senddata into an rx buffer of the peer) */
+#define OFI_AMD_NET_POST_WRITE 2 /* sending end: one rail stripe, `len` bytes from `src` to the peer's address `dest` under `key`, immediate data `imm` (fi_writedata) */
+#define OFI_AMD_NET_POST_CTRL 3  /* receiving end: the control message at `src` (`len` bytes) into the sending end's mailbox at byte offset `dest` (fi_write) */
+#define OFI_AMD_NET_POST_FLUSH 4 /* receiving end: 64 bytes of the flush buffer at `dest` read into the host slot at `src` (fi_read) */
+
+typedef struct {
+	uint32_t kind;
+	uint32_t rail;
+	uint32_t context; /* comes back through cq_read when the post has completed */
+	uint32_t imm;
+	uint64_t src;
+	uint64_t len;
+	uint64_t dest;
+	uint64_t key;
+	ofi_amd_eager_hdr_t hdr; /* eager only */
+} ofi_amd_net_post_t; /* 56 bytes */
+
+/* What the fabric reports to a comm (the CQ entries handled by ofi_process_cq's callees:
+ * a completed post of this end; handle_eager_recv, src/nccl_ofi_rdma.cpp:897-947;
+ * handle_write_comp, :1102-1130). */
+#define OFI_AMD_NET_CQ_POSTED 1 /* a post of this end has completed: `context` */
+#define OFI_AMD_NET_CQ_EAGER 2  /* receiving end: an eager message is in the rx buffer `rx_cookie` (byte offset in the rx pool): `imm`, header `hdr`, `len` payload bytes behind the header */
+#define OFI_AMD_NET_CQ_WRITE 3  /* receiving end: a remote write of `len` bytes carrying `imm` has landed */
+
+typedef struct {
+	uint32_t kind;
+	uint32_t context;
+	uint32_t imm;
+	uint32_t pad;
+	uint64_t len;
+	uint64_t rx_cookie;
+	ofi_amd_eager_hdr_t hdr;
+} ofi_amd_net_cqe_t; /* 40 bytes */
+
+typedef struct {
+	/* 0, -EAGAIN (no room now: the comm queues the post and tries again from its next progress, in
+	 * order, as the reference queues a request whose post returned -FI_EAGAIN), any other negative
+	 * errno */
+	int (*post)(void *end, const ofi_amd_net_post_t *post);
+	/* entries for this end: writes up to `max`, returns how many (0: none now) or a negative errno */
+	int (*cq_read)(void *end, ofi_amd_net_cqe_t *out, uint32_t max);
+	/* receiving end: the rx buffer `rx_cookie` has been emptied and can take the next eager message
+	 * (repost_rx_buff, src/nccl_ofi_rdma.cpp:656-670) */
+	int (*repost_rx)(void *end, uint64_t rx_cookie);
+	void *end;
+} ofi_amd_net_fabric_ops_t;
+
+/*
+ * A sending end over a fabric: the state machine of nccl_net_ofi_rdma_send_comm (ofi_amd_send_comm_*)
+ * with its posts, the queue of refused posts and the completions.  Arguments as
+ * ofi_amd_net_link_create.  The fabric delivers the peer's control messages into
+ * ofi_amd_net_send_comm_mailbox (256 slots of 512 bytes; a control post's `dest` is the byte
+ * offset into it).
+ */
+int ofi_amd_net_send_comm_create(uint32_t num_rails, int64_t eager_max_size, uint64_t min_stripe_size,
+				 uint64_t max_small_msg_size, const ofi_amd_net_fabric_ops_t *fabric, void **sendComm);
+void *ofi_amd_net_send_comm_mailbox(void *sendComm);
+/*
+ * A receiving end over a fabric: the state machine of nccl_net_ofi_rdma_recv_comm, its control and
+ * flush posts, and the launches that empty rx buffers into the posted receives
+ * (ofi_amd_eager_copy_batch on `stream`, rx buffers addressed as rx_pool_base + rx_cookie; each
+ * launch ends in a sentinel read-back, and a buffer goes back through repost_rx once its sentinel
+ * has been seen).  -ENODEV without a GPU.
+ */
+int ofi_amd_net_recv_comm_create(uint32_t num_rails, const ofi_amd_net_fabric_ops_t *fabric, const void *rx_pool_base,
+				 void *stream, void **recvComm);
+/* Either kind.  A receiving end waits for its stream first; open requests die with the comm. */
+int ofi_amd_net_comm_destroy(void *comm);
+
+/*
+ * The fabric of an in-process link: both ends are this process, the wire is device copies on
+ * `stream`.  An eager send becomes a copy of header and payload into one of rx_buffers rx buffers
+ * (-EAGAIN while none is free), a write one entry of ofi_amd_copy_table_pieces, a control message a
+ * copy into the sending end's mailbox (ofi_amd_netfab_connect).  Posts travel in launch groups that
+ * end in a sentinel read-back of the flush buffer; when it is seen (inside cq_read), the group's
+ * completions appear on both ends' queues in posting order.  A flush read rides on such a read-back
+ * (the newest one in flight, else the next): one read for all the flushes waiting.  A group leaves
+ * when an end polls and finds nothing, unless two are already in flight: then posts keep gathering.
+ */
+typedef struct ofi_amd_netfab ofi_amd_netfab_t;
+int ofi_amd_netfab_create(uint32_t num_rails, uint32_t rx_buffers, void *stream, ofi_amd_netfab_t **out);
+int ofi_amd_netfab_destroy(ofi_amd_netfab_t *fab);
+/* The two ends' callbacks, and the rx pool the receiving end's cookies are offsets into. */
+int ofi_amd_netfab_ops(ofi_amd_netfab_t *fab, ofi_amd_net_fabric_ops_t *send_end, ofi_amd_net_fabric_ops_t *recv_end);
+const void *ofi_amd_netfab_rx_pool(const ofi_amd_netfab_t *fab);
+/* Where control posts land: the sending end's mailbox. */
+int ofi_amd_netfab_connect(ofi_amd_netfab_t *fab, void *send_comm_mailbox);
+/* Kernel launches so far (copies and sentinels) and the table entries they carried. */
+int ofi_amd_netfab_counts(const ofi_amd_netfab_t *fab, uint64_t *launches, uint64_t *copy_entries);
+
 /* ---- set-up: what connect / accept hand over (no counterpart signature in the table) ---- */
 
 typedef struct ofi_amd_net_link ofi_amd_net_link_t;
@@ -59,6 +153,7 @@ typedef struct {
 	uint64_t copy_entries;    /* table entries of the wire launches */
 	uint64_t eager_copies;    /* rx buffers emptied by the eager copy */
 	uint64_t progress_calls;
+	uint64_t posts_refused;   /* posts the fabric answered -EAGAIN at the first attempt (queued, retried) */
 } ofi_amd_net_link_stats_t;
 
 /*
@@ -90,11 +185,14 @@ int ofi_amd_net_link_state(const ofi_amd_net_link_t *link, ofi_amd_send_state_t 
  * nccl_net_ofi_isend (src/nccl_ofi_api.cpp:440-467) over nccl_net_ofi_rdma_send_comm::send
  * (src/nccl_ofi_rdma.cpp:5646-5860).  `data` is a device-accessible address.  Success with
  * *request == NULL means "call again" (net_v12.h:108-109): the matching receive's control
- * message has not arrived and the message cannot go eager, or the link is out of room (rx
- * buffers, copy tables); the call has then made progress on the link, as the reference's does
- * on its completion queue.  mhandle and phandle are not looked at (in one process the
- * destination's address is its own key).  NULL comm or request -> ncclInternalError;
- * 1,024 sends in flight -> ncclInternalError (-EINVAL, :5683-5688).
+ * message has not arrived and the message cannot go eager; the call has then made progress on
+ * its end, as the reference's does on its completion queue.  A post the fabric refuses with
+ * -EAGAIN does not make the call fail: the request is returned and its posts wait in the end's
+ * queue (post_with_pending_retry, :1375-1387); while posts are waiting there, the next isend
+ * progresses first and answers "call again" if they still are (process_cq_if_pending,
+ * :3523-3545, :5682-5692).  mhandle and phandle are not looked at (the
+ * control message carries the mhandle's value as the key).  NULL comm or request ->
+ * ncclInternalError; 1,024 sends in flight -> ncclInternalError (-EINVAL, :5683-5688).
  */
 ncclResult_t ofi_amd_net_isend(void *sendComm, void *data, size_t size, int tag, void *mhandle, void *phandle,
 			       void **request);
@@ -102,7 +200,8 @@ ncclResult_t ofi_amd_net_isend(void *sendComm, void *data, size_t size, int tag,
  * nccl_net_ofi_irecv (:470-514) over nccl_net_ofi_rdma_recv_comm::recv
  * (src/nccl_ofi_rdma.cpp:3545-3745): n (1..8) receives as one request, matched to sends by tag.
  * NULL data, sizes, tags, mhandles or request, or n outside 1..8 -> ncclInvalidArgument; NULL
- * comm -> ncclInternalError; 128 receives and flushes in flight -> ncclSystemError (-ENOSPC).
+ * comm -> ncclInternalError; 128 receives and flushes in flight -> ncclSystemError (-ENOSPC);
+ * a NULL request with success while posts of this end wait in its queue (:3595-3605).
  * The control message carries a 32-bit length: a size above 4 GiB - 1 is refused with
  * ncclInternalError (the reference stores its low 32 bits, :3461).
  */

@@ -164,10 +164,11 @@ def test_grouped_receives_matched_by_tag_with_ragged_sizes_and_odd_addresses(lib
 
 
 def test_more_eager_sends_than_rx_buffers_and_more_receives_than_requests(lib, gpu):
-    """With 4 rx buffers the fifth eager send ahead of any receive is answered "call again" (no buffer
-    posted at the receiving end: the reference's provider would hold it back the same way); the 129th
-    receive in flight is refused with -ENOSPC -> ncclSystemError (NCCL_OFI_MAX_REQUESTS,
-    src/nccl_ofi_rdma.cpp:3571-3577), and everything drains afterwards."""
+    """With 4 rx buffers posted at the receiving end the fifth eager send ahead of any receive is refused by
+    the fabric (-FI_EAGAIN in the reference): its request is returned and its post waits in the sending end's
+    queue (post_with_pending_retry, src/nccl_ofi_rdma.cpp:1375-1387), and while it waits further isend calls
+    answer "call again" (process_cq_if_pending, :3523-3545).  The 129th receive in flight is refused with
+    -ENOSPC -> ncclSystemError (NCCL_OFI_MAX_REQUESTS, :3571-3577).  Everything drains afterwards."""
     link = Link(lib, rx_buffers=4)
     n = 128
     srcs, dsts = buffers([256] * n, [256] * n, seed=5)
@@ -177,21 +178,22 @@ def test_more_eager_sends_than_rx_buffers_and_more_receives_than_requests(lib, g
         if q is None:
             break
         send_reqs.append(q)
-    assert len(send_reqs) == 4
+    assert len(send_reqs) == 5 and link.stats().posts_refused == 1
     for _ in range(100):
-        assert link.isend(srcs[4], 256) is None
+        assert link.isend(srcs[5], 256) is None
     recv_reqs = [link.irecv([dsts[i]], [256]) for i in range(n)]
     data, sizes, tags, mhs = (vp * 1)(dsts[0].data_ptr()), (ctypes.c_size_t * 1)(256), (ctypes.c_int * 1)(TAG), (vp * 1)(0)
     req = vp()
     assert lib.ofi_amd_net_irecv(link.r, 1, data, sizes, tags, mhs, None, ctypes.byref(req)) == ncclSystemError
     assert not req.value
+
     def poll_receives():
-        """The receiving rank polls: arrivals are matched, copied out, and their rx buffers freed."""
+        """The receiving rank polls: arrivals are matched, copied out, and their rx buffers posted again."""
         for k, r in enumerate(recv_reqs):
             if r is not None and link.test(r)[0]:
                 recv_reqs[k] = None
 
-    for i in range(4, n):
+    for i in range(5, n):
         q = None
         for _ in range(100_000):
             q = link.isend(srcs[i], 256)
