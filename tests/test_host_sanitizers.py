@@ -69,3 +69,23 @@ def test_ring_push_pop_and_proxy_threads_clean_under_thread_sanitizer(tmp_path):
     assert proc.returncode == 0, proc.stdout[-4000:]
     assert "rings clean with 3 producers per ring" in proc.stdout
     assert "message buffer: 80000 sequence numbers on 4 threads" in proc.stdout
+
+
+def test_in_process_fabrics_and_entry_points_clean_under_sanitizers(tmp_path):
+    """The net and RMA entry points over the in-process fabrics (net_abi.cpp + net_fabric.cpp, rma_abi.cpp +
+    gin_devfab.cpp) on random programs, with the device side of the library replaced by stand-ins that run
+    each "launch" some calls after it was queued (tests/host/links_sanitize_driver.cpp): a table, a sentinel
+    slot or an rx buffer reused or freed while a launch still needs it is a sanitizer finding or a wrong
+    byte; every byte and reported size is checked."""
+    if not shutil.which("g++"):
+        pytest.skip("no host compiler")
+    exe = os.path.join(tmp_path, "links_sanitize")
+    sources = ["net_abi.cpp", "net_fabric.cpp", "rma_abi.cpp", "gin_devfab.cpp", "gin_tx.cpp", "gin_wire.cpp", "gin_rx.cpp",
+               "sendrecv_proto.cpp", "wire_codec.cpp", "sched_host.cpp"]
+    subprocess.run(["g++", "-std=c++17", "-pthread", *SAN, "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+                    os.path.join(ROOT, "tests", "host", "links_sanitize_driver.cpp"),
+                    *[os.path.join(CSRC, s) for s in sources], *SAN_LINK, "-o", exe], check=True)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1")
+    proc = subprocess.run([exe, "40"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env, timeout=600)
+    assert proc.returncode == 0, proc.stdout[-4000:]
+    assert "links: net and rma entry points clean over 40 seeds" in proc.stdout
