@@ -135,7 +135,8 @@ struct ofi_amd_devfab {
 	int gather()
 	{
 		group_t &g = filling();
-		while (!rung.empty() && g.n_copy < kGroupEntries) {
+		/* every post takes at most one table entry and one event; the events were reserved for */
+		while (!rung.empty() && g.n_copy < kGroupEntries && g.events.size() < kGroupEntries) {
 			const uint32_t rail = rung.at(0);
 			rail_t &r = rails[rail];
 			const ofi_amd_gin_post_t &p = r.sq.at(r.taken);
@@ -162,6 +163,9 @@ struct ofi_amd_devfab {
 				} else {
 					st.writes++;
 					st.bytes += p.len;
+				}
+				if (p.len && (local == 0 || p.dest == 0)) {
+					return -EFAULT; /* on the device a copy from or to address 0 is a fault, not an error code */
 				}
 				if (p.len) {
 					g.src.as<uint64_t>()[g.n_copy] = read ? p.dest : p.src;
@@ -198,7 +202,7 @@ struct ofi_amd_devfab {
 	int launch()
 	{
 		group_t &g = filling();
-		const bool full = g.n_copy >= kGroupEntries || g.n_work >= kGroupWork;
+		const bool full = g.n_copy >= kGroupEntries || g.n_work >= kGroupWork || g.events.size() >= kGroupEntries;
 		if (g.empty() || !can_launch() || (!full && cur - head >= kGroupsKeptBusy)) {
 			return 0;
 		}

@@ -308,8 +308,8 @@ int isend_impl(void *sendComm, void *data, size_t size, int tag, void **request)
 		*request = nullptr;
 	}
 	send_end_t *s = send_end_of(sendComm);
-	if (!s || !request) {
-		return -EINVAL;
+	if (!s || !request || (!data && size)) {
+		return -EINVAL; /* bytes from address 0 would be a fault on the device, not an error code */
 	}
 	s->isend_calls++;
 	/* process_cq_if_pending (src/nccl_ofi_rdma.cpp:3523-3545, called at :5682-5692): the queue is
@@ -399,8 +399,8 @@ int irecv_impl(void *recvComm, int n, void **data, const size_t *sizes, int *tag
 	uint64_t dsts[OFI_AMD_WIRE_MAX_RECVS], lens[OFI_AMD_WIRE_MAX_RECVS];
 	uint64_t keys[OFI_AMD_WIRE_MAX_RECVS * OFI_AMD_WIRE_MAX_RAILS];
 	for (int i = 0; i < n; i++) {
-		if (sizes[i] > 0xffffffffull) {
-			return -EINVAL; /* the control message carries a 32-bit length */
+		if (sizes[i] > 0xffffffffull || (!data[i] && sizes[i])) {
+			return -EINVAL; /* the control message carries a 32-bit length; no receive into address 0 */
 		}
 		dsts[i] = reinterpret_cast<uintptr_t>(data[i]);
 		lens[i] = sizes[i];

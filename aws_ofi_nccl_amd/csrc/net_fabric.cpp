@@ -64,7 +64,11 @@ struct group_t {
 	}
 	/* a transfer without bytes (a zero-length write) still waits for its group's sentinel */
 	bool empty() const { return n_copy == 0 && landings.empty() && riders.empty(); }
-	bool room(uint32_t entries) const { return n_copy + entries <= kGroupEntries; }
+	/* every post adds at most two landings; a zero-length write adds them without a table entry */
+	bool room(uint32_t entries) const
+	{
+		return n_copy + entries <= kGroupEntries && landings.size() + 2 <= 2 * kGroupEntries;
+	}
 	void add(uint64_t from, uint64_t to, uint64_t bytes)
 	{
 		src.as<uint64_t>()[n_copy] = from;
@@ -93,6 +97,8 @@ struct ofi_amd_netfab {
 	void *stream = nullptr;
 	void *rx_pool = nullptr;
 	std::vector<uint32_t> rx_free;
+	uint32_t n_rx = 0;
+	bool rx_is_free[kMaxRxBuffers] = {}; /* a buffer handed back twice would take two messages at once */
 	void *d_flush_buf = nullptr; /* the sentinel the groups read back */
 	uint8_t *mailbox = nullptr;  /* the sending end's, 256 slots of 512 bytes */
 	group_t groups[kGroups];
@@ -126,7 +132,7 @@ struct ofi_amd_netfab {
 		group_t &g = filling();
 		switch (p->kind) {
 		case OFI_AMD_NET_POST_EAGER: {
-			if (e->recv_end || p->len > kRxStride - OFI_AMD_EAGER_HEADER_SIZE) {
+			if (e->recv_end || p->len > kRxStride - OFI_AMD_EAGER_HEADER_SIZE || (p->len && p->src == 0)) {
 				return -EINVAL;
 			}
 			if (rx_free.empty() || !g.room(2)) {
@@ -134,6 +140,7 @@ struct ofi_amd_netfab {
 			}
 			const uint32_t slot = rx_free.back();
 			rx_free.pop_back();
+			rx_is_free[slot] = false;
 			const uint64_t rx = reinterpret_cast<uintptr_t>(rx_pool) + (uint64_t)slot * kRxStride;
 			g.hdrs.as<ofi_amd_eager_hdr_t>()[g.n_hdr] = p->hdr;
 			g.add(reinterpret_cast<uintptr_t>(g.hdrs.dev) + g.n_hdr * sizeof(ofi_amd_eager_hdr_t), rx,
@@ -147,8 +154,8 @@ struct ofi_amd_netfab {
 			return 0;
 		}
 		case OFI_AMD_NET_POST_WRITE:
-			if (e->recv_end) {
-				return -EINVAL;
+			if (e->recv_end || (p->len && (p->src == 0 || p->dest == 0))) {
+				return -EINVAL; /* a copy from or to address 0 would be a fault on the device */
 			}
 			if (!g.room(1)) {
 				return -EAGAIN;
@@ -160,7 +167,8 @@ struct ofi_amd_netfab {
 			landed(false, OFI_AMD_NET_CQ_POSTED, p->context, 0, 0, 0, nullptr);
 			return 0;
 		case OFI_AMD_NET_POST_CTRL: {
-			if (!e->recv_end || !mailbox || p->dest + p->len > 256u * sizeof(ofi_amd_ctrl_msg_t)) {
+			constexpr uint64_t kMailboxBytes = 256u * sizeof(ofi_amd_ctrl_msg_t);
+			if (!e->recv_end || !mailbox || p->src == 0 || p->dest > kMailboxBytes || p->len > kMailboxBytes - p->dest) {
 				return -EINVAL;
 			}
 			/* entry 0's sequence number is the ready mark: it goes in last */
@@ -294,10 +302,12 @@ struct ofi_amd_netfab {
 	{
 		end_t *e = static_cast<end_t *>(end);
 		ofi_amd_netfab *f = e->fab;
-		if (!e->recv_end || rx_cookie % kRxStride != 0 || rx_cookie / kRxStride >= kMaxRxBuffers) {
+		if (!e->recv_end || rx_cookie % kRxStride != 0 || rx_cookie / kRxStride >= f->n_rx ||
+		    f->rx_is_free[rx_cookie / kRxStride]) {
 			return -EINVAL;
 		}
-		f->rx_free.push_back((uint32_t)(rx_cookie / kRxStride));
+		f->rx_is_free[rx_cookie / kRxStride] = true;
+		f->rx_free.push_back((uint32_t)(rx_cookie / kRxStride)); /* within the capacity reserved at creation */
 		return 0;
 	}
 };
@@ -320,9 +330,12 @@ int ofi_amd_netfab_create(uint32_t num_rails, uint32_t rx_buffers, void *stream,
 	}
 	const uint32_t n_rx = rx_buffers ? rx_buffers : kMaxRxBuffers;
 	try {
+		f->rx_free.reserve(n_rx);
 		for (uint32_t k = n_rx; k > 0; k--) {
 			f->rx_free.push_back(k - 1);
+			f->rx_is_free[k - 1] = true;
 		}
+		f->n_rx = n_rx;
 		for (group_t &g : f->groups) {
 			g.landings.reserve(2 * kGroupEntries);
 			g.riders.reserve(OFI_AMD_MAX_REQUESTS * OFI_AMD_WIRE_MAX_RAILS);

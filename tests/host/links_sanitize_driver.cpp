@@ -466,6 +466,74 @@ int main(int argc, char **argv)
 		CHECK(ofi_amd_net_link_destroy(link) == 0);
 		CHECK(g_stream.empty());
 	}
+	/* what would be a fault on a device is an error code: address 0 with a length, an rx buffer
+	 * handed back twice or one the pool does not have */
+	{
+		ofi_amd_net_link_t *link = nullptr;
+		CHECK(ofi_amd_net_link_create(2, 8192, 0, 0, 4, nullptr, &link) == 0);
+		void *req = nullptr, *data = nullptr, *mh = nullptr;
+		size_t cap = 64;
+		int tag = 1;
+		CHECK(ofi_amd_net_isend(ofi_amd_net_link_send_comm(link), nullptr, 64, 1, nullptr, nullptr, &req) == ncclInternalError && !req);
+		CHECK(ofi_amd_net_irecv(ofi_amd_net_link_recv_comm(link), 1, &data, &cap, &tag, &mh, nullptr, &req) == ncclInternalError && !req);
+		cap = 0; /* nothing to receive into: address 0 is as good as any */
+		CHECK(ofi_amd_net_irecv(ofi_amd_net_link_recv_comm(link), 1, &data, &cap, &tag, &mh, nullptr, &req) == kOk && req);
+		CHECK(ofi_amd_net_link_destroy(link) == 0);
+
+		ofi_amd_netfab_t *fab = nullptr;
+		ofi_amd_net_fabric_ops_t s_ops, r_ops;
+		CHECK(ofi_amd_netfab_create(2, 4, nullptr, &fab) == 0 && ofi_amd_netfab_ops(fab, &s_ops, &r_ops) == 0);
+		CHECK(r_ops.repost_rx(r_ops.end, 0) == -EINVAL);         /* buffer 0 is free already */
+		CHECK(r_ops.repost_rx(r_ops.end, 4 * 8320) == -EINVAL);  /* the pool has four */
+		CHECK(r_ops.repost_rx(r_ops.end, 17) == -EINVAL);
+		CHECK(s_ops.repost_rx(s_ops.end, 0) == -EINVAL);         /* not the receiving end */
+		std::vector<uint8_t> payload(100, 7);
+		ofi_amd_net_post_t p;
+		std::memset(&p, 0, sizeof(p));
+		p.kind = OFI_AMD_NET_POST_WRITE;
+		p.len = 100;
+		p.src = (uint64_t)(uintptr_t)payload.data();
+		CHECK(s_ops.post(s_ops.end, &p) == -EINVAL);             /* to address 0 */
+		p.dest = p.src;
+		p.src = 0;
+		CHECK(s_ops.post(s_ops.end, &p) == -EINVAL);             /* from address 0 */
+		p.kind = OFI_AMD_NET_POST_EAGER;
+		CHECK(s_ops.post(s_ops.end, &p) == -EINVAL);
+		p.kind = OFI_AMD_NET_POST_CTRL;
+		p.src = p.dest;
+		p.dest = ~0ull - 10;                                     /* dest + len wraps */
+		CHECK(r_ops.post(r_ops.end, &p) == -EINVAL);
+		/* an eager send takes a buffer, the receiving end gives it back once */
+		p.kind = OFI_AMD_NET_POST_EAGER;
+		p.src = (uint64_t)(uintptr_t)payload.data();
+		p.dest = 0;
+		CHECK(s_ops.post(s_ops.end, &p) == 0);
+		ofi_amd_net_cqe_t cqe[4];
+		int n = 0;
+		for (int tries = 0; n == 0 && tries < 100; tries++) {
+			n = r_ops.cq_read(r_ops.end, cqe, 4);
+			device_tick(4);
+		}
+		CHECK(n == 1 && cqe[0].kind == OFI_AMD_NET_CQ_EAGER && cqe[0].len == 100);
+		CHECK(r_ops.repost_rx(r_ops.end, cqe[0].rx_cookie) == 0);
+		CHECK(r_ops.repost_rx(r_ops.end, cqe[0].rx_cookie) == -EINVAL);
+		CHECK(ofi_amd_netfab_destroy(fab) == 0);
+
+		/* the device fabric: a write to address 0 is found when it would join a launch */
+		ofi_amd_devfab_t *dfab = nullptr;
+		ofi_amd_gin_fabric_ops_t d_ops;
+		const uint32_t peer_id = 0;
+		CHECK(ofi_amd_devfab_create(1, 8, 1, &peer_id, nullptr, 0, nullptr, &dfab) == 0 && ofi_amd_devfab_ops(dfab, &d_ops) == 0);
+		ofi_amd_gin_post_t w;
+		std::memset(&w, 0, sizeof(w));
+		w.kind = OFI_AMD_GIN_POST_WRITE;
+		w.len = 100;
+		w.src = (uint64_t)(uintptr_t)payload.data();
+		CHECK(d_ops.post(d_ops.fabric, &w) == 0);
+		uint32_t ctxs[4];
+		CHECK(d_ops.cq_read(d_ops.fabric, 0, ctxs, 4) == -EFAULT);
+		CHECK(ofi_amd_devfab_destroy(dfab) == 0);
+	}
 	std::printf("links: net and rma entry points clean over %llu seeds, %llu launches on the stand-in device\n",
 		    (unsigned long long)seeds, (unsigned long long)g_launches);
 	return 0;

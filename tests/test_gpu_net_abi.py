@@ -235,6 +235,11 @@ def test_argument_checks_and_result_codes(lib, gpu):
     assert lib.ofi_amd_net_irecv(link.r, 9, data, sizes, tags, mhs, None, ctypes.byref(req)) == ncclInvalidArgument
     big = (ctypes.c_size_t * 1)(1 << 32)
     assert lib.ofi_amd_net_irecv(link.r, 1, data, big, tags, mhs, None, ctypes.byref(req)) == ncclInternalError
+    # bytes from or into address 0 would be a fault on the device: an error code, and no sequence number is used up
+    nulls = (vp * 1)(None)
+    assert lib.ofi_amd_net_isend(link.s, None, 8, TAG, None, None, ctypes.byref(req)) == ncclInternalError
+    assert lib.ofi_amd_net_irecv(link.r, 1, nulls, sizes, tags, mhs, None, ctypes.byref(req)) == ncclInternalError
+    assert req.value is None
     # iflush: n above 8, NULL comm / mhandles / request -> ncclInternalError; all sizes 0 -> no request
     assert lib.ofi_amd_net_iflush(link.r, 9, data, isizes, mhs, ctypes.byref(req)) == ncclInternalError
     assert lib.ofi_amd_net_iflush(None, 1, data, isizes, mhs, ctypes.byref(req)) == ncclInternalError

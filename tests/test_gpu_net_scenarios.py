@@ -243,3 +243,52 @@ def test_grouped_receives_in_the_alltoall_pattern(lib, gpu):
     st = link.stats()
     assert st.write_sends == len(msgs) and st.eager_sends == 0 and st.rdma_writes == 2 * len(msgs)
     link.close()
+
+
+def test_ring_of_four_ranks(lib, gpu):
+    """tests/functional/ring.cpp:205-318 with four ranks in this process: every rank posts NUM_REQUESTS
+    (NCCL_NET_MAX_REQUESTS = 32) receives of RECV_SIZE 5200 from its predecessor, then as many sends of
+    SEND_SIZE 5000 to its successor, retrying an isend that says "call again"; then polls both lists until
+    all are done.  Both sides report min(SEND_SIZE, RECV_SIZE); each completed receive is flushed and
+    compared with what was sent."""
+    ranks, nreq, send_size, recv_size = 4, 32, 5000, 5200
+    links = [Link(lib) for _ in range(ranks)]          # links[k]: rank k -> rank k + 1
+    rng = np.random.default_rng(11)
+    src = [torch.from_numpy(rng.integers(0, 256, (nreq, send_size), dtype=np.uint8)).cuda() for _ in range(ranks)]
+    dst = [[torch.full((recv_size + 64,), 0xCD, dtype=torch.uint8, device="cuda") for _ in range(nreq)]
+           for _ in range(ranks)]
+    torch.cuda.synchronize()
+    recv_reqs = {(k, i): links[(k - 1) % ranks].irecv([dst[k][i]], [recv_size]) for k in range(ranks) for i in range(nreq)}
+    send_reqs = {}
+    for k in range(ranks):
+        for i in range(nreq):
+            for _ in range(100_000):
+                req = links[k].isend(src[k][i], send_size)
+                if req is not None:
+                    break
+            assert req is not None
+            send_reqs[(k, i)] = req
+    for _ in range(200_000):
+        for key in list(send_reqs):
+            done, sz = links[key[0]].test(send_reqs[key])
+            if done:
+                assert sz == [send_size]
+                del send_reqs[key]
+        for key in list(recv_reqs):
+            k, i = key
+            link = links[(k - 1) % ranks]
+            done, sz = link.test(recv_reqs[key])
+            if done:
+                assert sz == [send_size]
+                link.flush([dst[k][i]], [recv_size])
+                got = dst[k][i].cpu().numpy()
+                assert np.array_equal(got[:send_size], src[(k - 1) % ranks][i].cpu().numpy()), key
+                assert np.all(got[send_size:] == 0xCD)
+                del recv_reqs[key]
+        if not send_reqs and not recv_reqs:
+            break
+    assert not send_reqs and not recv_reqs
+    for link in links:
+        st = link.stats()
+        assert st.eager_sends + st.write_sends == nreq and st.payload_bytes == nreq * send_size
+        link.close()
