@@ -25,7 +25,7 @@ struct ofi_amd_rma_mr {
 };
 
 struct ofi_amd_rma_ctx {
-	uint32_t nranks = 0, num_rails = 0, window_wait_ms = 0;
+	uint32_t nranks = 0, num_rails = 0, window_wait_ms = 0, max_requests = 0;
 	/* per peer rank: sequence numbers, window and ACK-request state (nccl_ofi_gin_peer_rank_info,
 	 * rank_comms[dst_rank] in the reference) */
 	std::vector<ofi_amd_gin_comm_t> peers;
@@ -72,6 +72,22 @@ int submit(ofi_amd_rma_ctx_t *ctx, uint16_t kind, uint64_t src_off, const ofi_am
 	}
 	if ((src && src->ctx != ctx) || (dst && dst->ctx != ctx) || (sig && sig->ctx != ctx)) {
 		return -EINVAL;
+	}
+	/* Room in the request pool is looked for before the derivation takes the operation's sequence
+	 * number: a number used up by an operation that is then not posted would stall the peer's
+	 * in-order retire for good.  One progress call may free what completed operations still hold. */
+	const uint32_t need = 2 + ctx->num_rails;
+	ofi_amd_gin_tx_stats_t ts;
+	(void)ofi_amd_gin_tx_stats(ctx->tx, &ts);
+	if (ctx->max_requests - ts.requests < need) {
+		const int e = ofi_amd_gin_tx_progress(ctx->tx);
+		if (e != 0) {
+			return e;
+		}
+		(void)ofi_amd_gin_tx_stats(ctx->tx, &ts);
+		if (ctx->max_requests - ts.requests < need) {
+			return -ENOMEM;
+		}
 	}
 	ofi_amd_gin_mr_t table[3] = {src ? src->per_rank[rank] : kNoMr, dst ? dst->per_rank[rank] : kNoMr,
 				     sig ? sig->per_rank[rank] : kNoMr};
@@ -176,6 +192,7 @@ int ofi_amd_rma_ctx_create(uint32_t nranks, uint32_t num_rails, uint64_t min_str
 	}
 	ctx->nranks = nranks;
 	ctx->num_rails = num_rails;
+	ctx->max_requests = max_requests;
 	ctx->window_wait_ms = window_wait_ms ? window_wait_ms : 10000;
 	*out = ctx;
 	return 0;

@@ -370,3 +370,39 @@ def test_the_older_op_tables_spell_the_same_operations(lib):
                                           ctypes.byref(req)) == ncclInternalError
     a.close()
     b.close()
+
+
+def test_a_full_request_pool_refuses_the_operation_before_it_takes_a_sequence_number(lib):
+    """A pool of 16 entries holds two puts of one stripe and their metadata messages' worth of room
+    less than a third needs (an operation asks for 2 + rails entries up front).  The refused call must
+    leave the peer's next sequence number where it was -- a number used up without a post would stall
+    the target's in-order retire -- and succeed once completions have given entries back."""
+    ini = Initiator(lib, pool=16, wait_ms=30)
+    req = ctypes.c_void_p()
+    put = lambda: lib.ofi_amd_rma_iputSignal(ini.ctx, 0, 0, ini.mrs[0], 5000, 0, ini.mrs[1], 1, 8, ini.mrs[2], 1,
+                                             SIGNAL_INC, True, 0, ctypes.byref(req))
+    reqs = []
+    while True:
+        before = lib.ofi_amd_rma_peer_state(ini.ctx, 1).contents.tx_head
+        rc = put()
+        if rc != 0:
+            break
+        reqs.append(ctypes.c_void_p(req.value))
+        assert len(reqs) < 16
+    assert rc == ncclSystemError and req.value is None and len(reqs) >= 2       # -ENOMEM
+    assert lib.ofi_amd_rma_peer_state(ini.ctx, 1).contents.tx_head == before
+    # the wire takes the posts, their completions free the entries at the next progress call
+    sent = ini.wire()
+    assert len(sent) == 2 * len(reqs)
+    done = ctypes.c_int()
+    for r in reqs:
+        for _ in range(100):
+            assert lib.ofi_amd_rma_test(ini.ctx, r, ctypes.byref(done)) == 0
+            if done.value:
+                break
+            assert lib.ofi_amd_rma_rmaProgress(ini.ctx) == 0
+        assert done.value
+    assert put() == 0 and req.value
+    assert lib.ofi_amd_rma_peer_state(ini.ctx, 1).contents.tx_head == before + 1
+    ini.wire()
+    ini.close()
