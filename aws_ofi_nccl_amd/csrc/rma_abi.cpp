@@ -73,22 +73,6 @@ int submit(ofi_amd_rma_ctx_t *ctx, uint16_t kind, uint64_t src_off, const ofi_am
 	if ((src && src->ctx != ctx) || (dst && dst->ctx != ctx) || (sig && sig->ctx != ctx)) {
 		return -EINVAL;
 	}
-	/* Room in the request pool is looked for before the derivation takes the operation's sequence
-	 * number: a number used up by an operation that is then not posted would stall the peer's
-	 * in-order retire for good.  One progress call may free what completed operations still hold. */
-	const uint32_t need = 2 + ctx->num_rails;
-	ofi_amd_gin_tx_stats_t ts;
-	(void)ofi_amd_gin_tx_stats(ctx->tx, &ts);
-	if (ctx->max_requests - ts.requests < need) {
-		const int e = ofi_amd_gin_tx_progress(ctx->tx);
-		if (e != 0) {
-			return e;
-		}
-		(void)ofi_amd_gin_tx_stats(ctx->tx, &ts);
-		if (ctx->max_requests - ts.requests < need) {
-			return -ENOMEM;
-		}
-	}
 	ofi_amd_gin_mr_t table[3] = {src ? src->per_rank[rank] : kNoMr, dst ? dst->per_rank[rank] : kNoMr,
 				     sig ? sig->per_rank[rank] : kNoMr};
 	ofi_amd_gin_desc_t d;
@@ -108,7 +92,10 @@ int submit(ofi_amd_rma_ctx_t *ctx, uint16_t kind, uint64_t src_off, const ofi_am
 
 	ofi_amd_gin_comm_t *peer = &ctx->peers[rank];
 	ofi_amd_gin_wire_t wire;
+	ofi_amd_gin_comm_t peer_before, shared_before;
 	auto derive = [&]() -> int {
+		peer_before = *peer;
+		shared_before = ctx->shared;
 		peer->sched = ctx->shared.sched;
 		peer->pinned_rail_id = ctx->shared.pinned_rail_id;
 		peer->pinned_rail_run = ctx->shared.pinned_rail_run;
@@ -140,6 +127,16 @@ int submit(ofi_amd_rma_ctx_t *ctx, uint16_t kind, uint64_t src_off, const ofi_am
 	}
 	if (rc != 0) {
 		return rc;
+	}
+	/* A full request pool is found before anything is posted, and then the operation never
+	 * happened: its sequence number, its place in the window and the rails it would have taken
+	 * go back.  A number used up without a post would stall the target's in-order retire for good. */
+	ofi_amd_gin_tx_stats_t ts;
+	(void)ofi_amd_gin_tx_stats(ctx->tx, &ts);
+	if (ctx->max_requests - ts.requests < 1u + wire.num_writes + (wire.has_meta ? 1u : 0u)) {
+		*peer = peer_before;
+		ctx->shared = shared_before;
+		return -ENOMEM;
 	}
 	int32_t op = -1;
 	rc = kind == OFI_AMD_GIN_KIND_GET ? ofi_amd_gin_tx_iget(ctx->tx, rank, &wire, &op)

@@ -50,7 +50,11 @@ typedef struct ofi_amd_rma_mr ofi_amd_rma_mr_t;
  * ofi_amd_gin_tx_create, with the reference's CQ defaults 4 x 4), max_requests pool entries.
  * window_wait_ms bounds how long iput / iputSignal keep calling progress for room in a peer's
  * sequence window (the reference's await_tx_window, src/rdma/gin/nccl_ofi_gin.cpp:518-537,
- * spins without a bound); 0 = 10,000.
+ * spins without a bound); 0 = 10,000.  An operation that finds the pool full (an operation holds
+ * one entry plus one per write or read and one for its metadata message until test() has
+ * reported it done) is refused with ncclSystemError before anything is posted and leaves the
+ * peer's sequence numbers, window and rail state as they were: it may be issued again after
+ * completions have been tested.  The reference's pool grows instead and throws when it cannot.
  */
 int ofi_amd_rma_ctx_create(uint32_t nranks, uint32_t num_rails, uint64_t min_stripe_size,
 			   uint64_t max_small_msg_size, const ofi_amd_gin_fabric_ops_t *fabric,

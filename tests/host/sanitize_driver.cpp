@@ -5,6 +5,7 @@
  * disagreement, and anything the sanitizers see, ends the run with a non-zero status.
  * Test infrastructure: built and run by tests/test_host_sanitizers.py, CPU only.
  */
+#include <cerrno>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -790,6 +791,7 @@ void run_rma_abi(uint64_t seed, uint32_t n_ops)
 			}
 			const oracle_gin_mr_t table[3] = { mra[0][rank], mra[1][rank], mra[2][rank] };
 			oracle_gin_comm_t *peer = &pa[rank];
+			const oracle_gin_comm_t peer_before = *peer, shared_before = sa;
 			peer->sched = sa.sched;
 			peer->pinned_rail_id = sa.pinned_rail_id;
 			peer->pinned_rail_run = sa.pinned_rail_run;
@@ -804,6 +806,13 @@ void run_rma_abi(uint64_t seed, uint32_t n_ops)
 			int32_t qa = -1;
 			if (ra == 0) {
 				ra = get ? oracle_gin_tx_iget(a, rank, &wa, &qa) : oracle_gin_tx_iput_signal(a, rank, &wa, &qa);
+				if (ra == -ENOMEM) {
+					/* The engine's pool is full and nothing was posted.  The reference's pool throws
+					 * there; the entry points instead undo the derivation, so that no sequence number
+					 * is used up by an operation that never reaches the wire. */
+					*peer = peer_before;
+					sa = shared_before;
+				}
 			}
 			void *req = &req; /* must be overwritten */
 			int rb;
