@@ -472,6 +472,7 @@ PROTOTYPES = {
     "ofi_amd_loopfab_destroy": (ctypes.c_int, [c_vp]),
     "ofi_amd_loopfab_ops": (ctypes.c_int, [c_vp, ctypes.POINTER(GinFabricOps)]),
     "ofi_amd_loopfab_take_transmitted": (c_u32, [c_vp, ctypes.POINTER(GinPost), c_u32]),
+    "ofi_amd_loopfab_next_transmitted": (ctypes.POINTER(GinPost), [c_vp]),
     "ofi_amd_gin_rx_create": (ctypes.c_int, [c_u32, ctypes.POINTER(c_u32), ctypes.POINTER(c_vp)]),
     "ofi_amd_gin_rx_destroy": (ctypes.c_int, [c_vp]),
     "ofi_amd_gin_rx_write_completion": (ctypes.c_int, [c_vp, c_u32, c_u32]),

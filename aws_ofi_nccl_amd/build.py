@@ -28,6 +28,9 @@ COMMON = [
 ]
 
 
+HOST_LTO = ["-flto=thin"]
+
+
 def _sources():
     out = []
     for name in sorted(os.listdir(CSRC)):
@@ -38,7 +41,10 @@ def _sources():
 
 def _compile(src):
     obj = os.path.join(LIBDIR, "obj", os.path.basename(src) + ".o")
-    cmd = [HIPCC] + COMMON + (["-x", "hip"] if src.endswith(".hip") else []) + ["-c", src, "-o", obj]
+    # The host sources go through link-time optimisation: the proxy, the loop-back runs and the entry points
+    # make tens of millions of calls a second into each other's translation units (transmit engine, receiver,
+    # fabrics), and those calls are inlined at link time.
+    cmd = [HIPCC] + COMMON + (["-x", "hip"] if src.endswith(".hip") else HOST_LTO) + ["-c", src, "-o", obj]
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     text = "\n".join(l for l in proc.stdout.splitlines()
                      if "packed-fp32-ops" not in l and "is not a recognized feature" not in l)
@@ -59,7 +65,8 @@ def build_library(verbose=False):
                 print(text)
     # -Bsymbolic-functions: calls between the library's own entry points (the loop-back runs and the
     # proxy make millions a second) bind inside the library instead of going through the PLT
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,-Bsymbolic-functions", "-o", LIB] + objs + ["-lpthread"]
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-O3"] + HOST_LTO + ["-Wl,-Bsymbolic-functions", "-o", LIB] + \
+        objs + ["-lpthread"]
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if proc.returncode != 0:
         raise RuntimeError("link failed:\n%s" % proc.stdout)

@@ -339,14 +339,14 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 	 * metadata message an event, an ACK moves the sender's window), then one progress call of
 	 * the engine (bounded CQ drain, retry of the refused posts), then test() of the oldest
 	 * operations. */
-	ofi_amd_gin_post_t wire_posts[64];
 	auto pump = [&]() -> int {
 		const uint64_t p0 = sampling ? stage_clock_t::now() : 0;
 		const uint64_t fl0 = flush_ticks_in_sample;
-		for (;;) {
-			const uint32_t n = ofi_amd_loopfab_take_transmitted(fab, wire_posts, 64);
-			for (uint32_t i = 0; i < n; i++) {
-				const ofi_amd_gin_post_t &p = wire_posts[i];
+		{
+			/* read in place: the send-queue entries stay where they are until the progress call
+			 * below reads their completions */
+			while (const ofi_amd_gin_post_t *next = ofi_amd_loopfab_next_transmitted(fab)) {
+				const ofi_amd_gin_post_t &p = *next;
 				event_t ev{p.peer, 0, -1};
 				if (p.kind == OFI_AMD_GIN_POST_WRITE || p.kind == OFI_AMD_GIN_POST_READ) {
 					/* a read is the same copy the other way, and the target hears nothing of it */
@@ -401,9 +401,6 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 					ofi_amd_gin_apply_ack(&comms[p.peer], (uint32_t)(p.msg[0] >> 12) & 0x3fffu);
 					st.acks++;
 				}
-			}
-			if (n < 64) {
-				break;
 			}
 		}
 		const uint64_t p1 = sampling ? stage_clock_t::now() : 0;

@@ -27,7 +27,7 @@ enum : uint8_t { kFree = 0, kOperation = 1, kSub = 2, kFlush = 3 };
 
 /* One pool entry: the umbrella request of an operation (nccl_ofi_rdma_gin_iputsignal_req) or
  * one post (write / metadata send / ACK send request). */
-struct request_t {
+struct alignas(64) request_t { /* two cache lines to an entry, none shared with a neighbour */
 	uint8_t use = kFree;
 	uint8_t slot = 0;            /* sub: which reqs_pending flag of the parent it clears */
 	int32_t parent = kNoParent;  /* sub: the operation, or kNoParent (ACKs, given-up operations) */
@@ -575,6 +575,19 @@ uint32_t ofi_amd_loopfab_take_transmitted(ofi_amd_loopfab_t *f, ofi_amd_gin_post
 		r.readable++; /* executed on the spot by the caller: the completion is there */
 	}
 	return n;
+}
+
+const ofi_amd_gin_post_t *ofi_amd_loopfab_next_transmitted(ofi_amd_loopfab_t *f)
+{
+	if (!f || f->rung.empty()) {
+		return nullptr;
+	}
+	ofi_amd_loopfab::rail_t &r = f->rails[f->rung.at(0)];
+	f->rung.pop();
+	const ofi_amd_gin_post_t *p = &r.sq.at(r.taken);
+	r.taken++;
+	r.readable++;
+	return p;
 }
 
 } /* extern "C" */

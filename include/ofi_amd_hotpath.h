@@ -609,6 +609,10 @@ int ofi_amd_loopfab_create(uint32_t num_rails, uint32_t sq_depth, ofi_amd_loopfa
 int ofi_amd_loopfab_destroy(ofi_amd_loopfab_t *f);
 int ofi_amd_loopfab_ops(ofi_amd_loopfab_t *f, ofi_amd_gin_fabric_ops_t *ops);
 uint32_t ofi_amd_loopfab_take_transmitted(ofi_amd_loopfab_t *f, ofi_amd_gin_post_t *out, uint32_t cap);
+/* The same, one post at a time and in place: the next transmitted post as it stands in its rail's
+ * send queue, or NULL when none is waiting.  The pointer is good until completions are next read
+ * from the fabric (reading a completion frees the send-queue entry). */
+const ofi_amd_gin_post_t *ofi_amd_loopfab_next_transmitted(ofi_amd_loopfab_t *f);
 /* Rings every rail's doorbell: posts still waiting behind FI_MORE are transmitted. */
 int ofi_amd_loopfab_ring_all(ofi_amd_loopfab_t *f);
 

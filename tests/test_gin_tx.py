@@ -374,6 +374,16 @@ def test_loop_fabric_send_queue_doorbells_and_completions(lib):
     assert taken() == [(0, 13), (0, 14)]
     assert read(0) == [12, 13, 14] and read(0) == []
     assert post(3, 0, 1) == EINVAL
+    # one at a time and in place: the same order, the same completions, NULL when nothing waits
+    def next_one():
+        p = lib.ofi_amd_loopfab_next_transmitted(fab)
+        return (p.contents.rail, p.contents.context) if p else None
+
+    assert post(1, 1, 30) == 0 and post(0, 0, 31) == 0 and post(1, 0, 32) == 0
+    assert next_one() == (0, 31) and next_one() == (1, 30)
+    assert read(1) == [30] and read(0) == [31]           # taken: readable; the third is still on its way
+    assert next_one() == (1, 32) and next_one() is None and read(1) == [32]
+    assert not lib.ofi_amd_loopfab_next_transmitted(None)
     assert lib.ofi_amd_loopfab_destroy(fab) == 0
     assert lib.ofi_amd_loopfab_create(0, 3, ctypes.byref(fab)) == EINVAL
     assert lib.ofi_amd_loopfab_create(2, 0, ctypes.byref(fab)) == EINVAL
