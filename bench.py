@@ -570,11 +570,13 @@ def bench_gin(lib, oracle, torch, np, args):
     side = torch.cuda.Stream()
     # a progress call after every operation (the strictest caller), and after every 64th: the
     # reference's own test posts 64 puts and 64 put-signals before its first progress call
-    # (tests/functional/rma.cpp:213-246).  Four passes each of some 60 ms: the first warms the pinned tables up,
-    # and the host thread's rate moves by 10 % from pass to pass; the best pass is reported, all are listed.
+    # (tests/functional/rma.cpp:213-246).  Passes of some 60 ms each: the first warms the pinned tables up, and
+    # the host thread's rate moves by 10 % from pass to pass (more when the box's other tenants are busy).  Four
+    # passes at least; while the best of them is one of the last two, i.e. the rate is still climbing, another,
+    # ten at most.  The best pass is reported, all are listed.
     for key, interval in (("loopback", 1), ("loopback_progress_every_64", 64)):
         best, rates = None, []
-        for _ in range(4):
+        while len(rates) < 4 or (len(rates) < 10 and max(rates) in rates[-2:]):
             for c in range(l_ctx):
                 lib.ofi_amd_gin_comm_init(ctypes.byref(comms[c]), c, 4, 131072, 64, 0)
             d_cnt.zero_()
