@@ -1,14 +1,17 @@
 /*
  * The in-process fabrics and the entry points over them (net_abi.cpp + net_fabric.cpp,
- * rma_abi.cpp + gin_devfab.cpp) run on the CPU under AddressSanitizer and
- * UndefinedBehaviorSanitizer: the device side of the library is replaced, in this test program
- * only, by stand-ins that keep a queue of "launches" and execute them later (host memory plays
- * device memory), so that tables, sentinels and buffers are used exactly when a GPU would use
- * them -- some calls after they were handed over -- and a table freed or reused too early is a
- * sanitizer finding or a wrong byte.  Random programs; every byte and every reported size is
- * checked.  Test infrastructure: built and run by tests/test_host_sanitizers.py.
+ * rma_abi.cpp + gin_devfab.cpp) and the GIN loop-back run (gin_loopback.cpp) on the CPU under
+ * AddressSanitizer + UndefinedBehaviorSanitizer, and under ThreadSanitizer: the device side of
+ * the library is replaced, in this test program only, by stand-ins that keep a queue of
+ * "launches" and execute them later (host memory plays device memory) -- when this thread
+ * ticks the device, or, in the "threaded" mode, on a device thread -- so that tables, sentinels
+ * and buffers are used when a GPU would use them, some time after they were handed over.  A
+ * table freed or reused too early is then a sanitizer finding, a data race or a wrong byte.
+ * Random programs; every byte, reported size and counter is checked.  Test infrastructure:
+ * built and run by tests/test_host_sanitizers.py.
  */
 #include <algorithm>
+#include <atomic>
 #include <cerrno>
 #include <cstdio>
 #include <cstdlib>
@@ -16,8 +19,11 @@
 #include <deque>
 #include <functional>
 #include <map>
+#include <mutex>
+#include <thread>
 #include <vector>
 
+#include "gin_rings.hpp"
 #include "ofi_amd_hotpath.h"
 #include "ofi_amd_net_abi.h"
 #include "ofi_amd_rma_abi.h"
@@ -53,14 +59,73 @@ struct rng_t {
 
 /* ---- the stand-in device: a queue of launches, executed some calls later ---- */
 std::deque<std::function<void()>> g_stream;
+std::mutex g_stream_mu;
+std::atomic<uint64_t> g_queued{0}; /* launches queued or running */
+std::atomic<bool> g_device_thread{false}; /* the launches run on a thread of their own, as a GPU's do */
 uint64_t g_launches;
+
+void launch(std::function<void()> f)
+{
+	std::lock_guard<std::mutex> lock(g_stream_mu);
+	g_stream.push_back(std::move(f));
+	g_queued.fetch_add(1);
+}
+
+/* the oldest queued launch, run outside the lock: one executor at a time, so stream order holds */
+bool run_one()
+{
+	std::function<void()> f;
+	{
+		std::lock_guard<std::mutex> lock(g_stream_mu);
+		if (g_stream.empty()) {
+			return false;
+		}
+		f = std::move(g_stream.front());
+		g_stream.pop_front();
+	}
+	f();
+	g_queued.fetch_sub(1);
+	return true;
+}
 
 void device_tick(uint32_t n)
 {
-	while (n-- && !g_stream.empty()) {
-		g_stream.front()();
-		g_stream.pop_front();
+	if (g_device_thread.load()) {
+		return;
 	}
+	while (n-- && run_one()) {
+	}
+}
+
+bool stream_empty()
+{
+	return g_queued.load() == 0;
+}
+
+std::thread g_device;
+std::atomic<bool> g_device_stop{false};
+
+void start_device_thread()
+{
+	g_device_stop.store(false);
+	g_device_thread.store(true);
+	g_device = std::thread([]() {
+		while (!g_device_stop.load()) {
+			if (!run_one()) {
+				std::this_thread::yield();
+			}
+		}
+	});
+}
+
+void stop_device_thread()
+{
+	while (g_queued.load() != 0) {
+		std::this_thread::yield();
+	}
+	g_device_stop.store(true);
+	g_device.join();
+	g_device_thread.store(false);
 }
 
 } // namespace
@@ -87,12 +152,18 @@ int ofi_amd_gpu_mem_alloc(void **ptr, size_t size) { return ofi_amd_gpu_host_all
 int ofi_amd_gpu_mem_free(void *ptr) { return ofi_amd_gpu_host_free(ptr); }
 int ofi_amd_gpu_stream_synchronize(void *)
 {
+	if (g_device_thread.load()) {
+		while (g_queued.load() != 0) {
+			std::this_thread::yield();
+		}
+		return 0;
+	}
 	device_tick(~0u);
 	return 0;
 }
 int ofi_amd_flush_buffer_fill(void *d_flush_buf, uint64_t sentinel, void *)
 {
-	g_stream.push_back([=]() {
+	launch([=]() {
 		for (int w = 0; w < 8; w++) {
 			static_cast<uint64_t *>(d_flush_buf)[w] = sentinel;
 		}
@@ -102,7 +173,7 @@ int ofi_amd_flush_buffer_fill(void *d_flush_buf, uint64_t sentinel, void *)
 int ofi_amd_flush_post(const void *d_flush_buf, void *slots_dev, uint32_t num_rails, void *)
 {
 	g_launches++;
-	g_stream.push_back([=]() {
+	launch([=]() {
 		for (uint32_t r = 0; r < num_rails; r++) {
 			for (int w = 7; w >= 0; w--) {
 				__atomic_store_n(&static_cast<uint64_t *>(slots_dev)[r * 8 + w],
@@ -116,9 +187,18 @@ int ofi_amd_copy_table_pieces(const uint64_t *d_src, const uint64_t *d_dst, cons
 			      uint32_t max_len, void *)
 {
 	g_launches++;
-	g_stream.push_back([=]() { /* the tables are read when the launch runs, as on the device */
+	launch([=]() { /* the tables are read when the launch runs, as on the device */
 		for (uint32_t i = 0; i < n; i++) {
 			const uint32_t bytes = d_len[i] < max_len ? d_len[i] : max_len;
+			if (bytes == 64 && d_dst[i] % 8 == 0 && d_src[i] % 8 == 0) {
+				/* the shape of a flush read: its landing slots are polled by the host while the
+				 * copy is on its way, word by word as a device writes them */
+				for (int w = 7; w >= 0; w--) {
+					const uint64_t v = reinterpret_cast<const uint64_t *>(static_cast<uintptr_t>(d_src[i]))[w];
+					__atomic_store_n(&reinterpret_cast<uint64_t *>(static_cast<uintptr_t>(d_dst[i]))[w], v, __ATOMIC_RELEASE);
+				}
+				continue;
+			}
 			std::memmove(reinterpret_cast<void *>(static_cast<uintptr_t>(d_dst[i])),
 				     reinterpret_cast<const void *>(static_cast<uintptr_t>(d_src[i])), bytes);
 		}
@@ -130,7 +210,7 @@ int ofi_amd_eager_copy_batch(const void *rx_base, const uint64_t *d_rx_off, cons
 			     uint32_t *, void *)
 {
 	g_launches++;
-	g_stream.push_back([=]() {
+	launch([=]() {
 		for (uint32_t i = 0; i < n; i++) {
 			const uint32_t bytes = d_recv_len[i] < d_dst_len[i] ? d_recv_len[i] : d_dst_len[i];
 			std::memcpy(reinterpret_cast<void *>(reinterpret_cast<uintptr_t>(dst_base) + d_dst_off[i]),
@@ -147,7 +227,7 @@ int ofi_amd_gin_signal_apply(const ofi_amd_gin_signal_work_t *d_work, uint32_t n
 {
 	g_launches++;
 	std::vector<ofi_amd_gin_signal_region_t> regs(regions, regions + n_regions); /* passed by value to a kernel */
-	g_stream.push_back([=]() {
+	launch([=]() {
 		for (uint32_t i = 0; i < n; i++) {
 			for (const ofi_amd_gin_signal_region_t &r : regs) {
 				if (d_work[i].base == r.base && d_work[i].offset + 8 <= r.size) {
@@ -441,16 +521,179 @@ void run_rma(uint64_t seed, int n_ops)
 	CHECK(ofi_amd_rma_ctx_destroy(ctx) == 0 && ofi_amd_devfab_destroy(fab) == 0);
 }
 
+/* ------------------------------------------------------------------ GIN loop-back run */
+
+/* ofi_amd_gin_loopback_run (gin_loopback.cpp) from end to end: a producer thread pushes random
+ * puts, put-signals, signal-only operations and gets into rings in ordinary host memory, the run
+ * drains them on this thread, and the stand-in device executes its launches on a thread of its own,
+ * so the run's tables are read while it is already filling the next ones.  Bytes, landing
+ * buffers, counters and the bookkeeping are compared with a plain replay. */
+void run_gin_loopback(uint64_t seed)
+{
+	rng_t rng{ seed };
+	const uint32_t nctx = 1 + rng.below(4), cap = 64;
+	const uint64_t ops = 600 + rng.below(1500);
+	const uint32_t max_size = rng.chance(50) ? 300000 : 40000;
+	const size_t src_bytes = 4u << 20;
+	std::vector<uint8_t> src(src_bytes), remote(src_bytes);
+	for (size_t i = 0; i < src_bytes; i++) {
+		src[i] = (uint8_t)rng.next();
+		remote[i] = (uint8_t)rng.next();
+	}
+	std::vector<std::vector<ofi_amd_gin_desc_t>> table(nctx);
+	uint64_t dst_pos = 0, land_pos = 0, n_signals = 0, n_bytes = 0, n_gets = 0;
+	std::vector<uint64_t> want_cnt(64, 0), n_puts(nctx, 0);
+	for (uint32_t c = 0; c < nctx; c++) {
+		for (uint64_t i = 0; i < ops; i++) {
+			ofi_amd_gin_desc_t d;
+			std::memset(&d, 0, sizeof(d));
+			d.rank = 1;
+			d.context = c;
+			d.opt_flags = rng.below(2);
+			if (i % 4 == 3) { /* a get: remote handle 3, local handle 4 */
+				d.size = rng.chance(90) ? rng.below(max_size) : 0;
+				d.src_off = rng.below((uint32_t)(src_bytes - d.size));
+				d.dst_off = land_pos + rng.below(24);
+				land_pos = d.dst_off + d.size + rng.below(8);
+				d.src_mr = 3;
+				d.dst_mr = 4;
+				d.sig_mr = 0xffff;
+				d.kind = 3;
+				d.opt_flags = 0;
+				n_gets++;
+			} else {
+				const uint32_t k = rng.below(100);
+				d.size = k < 8 ? 0 : (k < 60 ? 1 + rng.below(4095) : 8 + rng.below(max_size));
+				d.src_off = rng.below((uint32_t)(src_bytes - d.size));
+				d.dst_off = dst_pos + rng.below(24);
+				dst_pos = d.dst_off + d.size + rng.below(8);
+				const bool signal = d.size == 0 || i % 5 == 4;
+				d.signal_op = signal ? 1 + rng.below(2) : 0;
+				d.signal_value = d.signal_op == 2 ? rng.next() >> 24 : 0;
+				const uint32_t slot = rng.below(64);
+				d.signal_off = signal ? 8 * slot : 0;
+				d.src_mr = 0;
+				d.dst_mr = 1;
+				d.sig_mr = signal ? 2 : 0xffff;
+				d.kind = signal ? 2 : 1;
+				if (signal) {
+					want_cnt[slot] += d.signal_op == 1 ? 1 : d.signal_value;
+					n_signals++;
+				}
+				n_puts[c]++;
+			}
+			n_bytes += d.size;
+			table[c].push_back(d);
+		}
+	}
+	std::vector<uint8_t> dst(dst_pos + 64, 0xEE), land(land_pos + 64, 0xDD), want_dst = dst, want_land = land;
+	for (uint32_t c = 0; c < nctx; c++) {
+		for (const ofi_amd_gin_desc_t &d : table[c]) {
+			if (d.kind == 3) {
+				std::memcpy(want_land.data() + d.dst_off, remote.data() + d.src_off, d.size);
+			} else {
+				std::memcpy(want_dst.data() + d.dst_off, src.data() + d.src_off, d.size);
+			}
+		}
+	}
+	std::vector<uint64_t> counters(64, 0);
+	const uint64_t sig_base = 0x7F5500000000ull;
+	ofi_amd_gin_mr_t mrs[5];
+	std::memset(mrs, 0, sizeof(mrs));
+	mrs[0].local_base = (uint64_t)(uintptr_t)src.data();
+	mrs[1].remote_address_offset = (uint64_t)(uintptr_t)dst.data();
+	mrs[2].remote_address = sig_base;
+	mrs[3].remote_address_offset = (uint64_t)(uintptr_t)remote.data();
+	mrs[4].local_base = (uint64_t)(uintptr_t)land.data();
+	for (int i = 0; i < 5; i++) {
+		for (int r = 0; r < 4; r++) {
+			mrs[i].key[r] = 0x100 * (i + 1) + r;
+		}
+	}
+	const uint32_t rails = 1u << rng.below(3); /* 1, 2 or 4 */
+	std::vector<ofi_amd_gin_comm_t> comms(nctx);
+	for (uint32_t c = 0; c < nctx; c++) {
+		CHECK(ofi_amd_gin_comm_init(&comms[c], 100 + c, rails, 131072, 64, 0) == 0);
+	}
+	const ofi_amd_gin_signal_region_t region = { sig_base, 512, counters.data() };
+
+	ofi_amd_gin_rings rings;
+	std::memset(&rings, 0, sizeof(rings));
+	rings.n_contexts = nctx;
+	rings.capacity = cap;
+	std::vector<ofi_amd_gin_desc_t> records((size_t)nctx * cap);
+	std::vector<uint32_t> sequences((size_t)nctx * cap), enq((size_t)nctx * 16, 0), deq(nctx, 0), status(16, 0);
+	for (uint32_t c = 0; c < nctx; c++) {
+		for (uint32_t i = 0; i < cap; i++) {
+			sequences[(size_t)c * cap + i] = i;
+		}
+	}
+	rings.records = records.data();
+	rings.sequences = sequences.data();
+	rings.enqueue_pos = enq.data();
+	rings.dequeue_pos = deq.data();
+	rings.status = status.data();
+
+	const bool own_device = !g_device_thread.load();
+	if (own_device) {
+		start_device_thread();
+	}
+	std::thread producer([&]() {
+		for (uint64_t i = 0; i < ops; i++) {
+			for (uint32_t c = 0; c < nctx; c++) {
+				for (;;) {
+					const int rc = ofi_amd_gin_ring_push(&rings, c, &table[c][i]);
+					if (rc == 1) {
+						break;
+					}
+					CHECK(rc == 0); /* full: the run has to drain first */
+					std::this_thread::yield();
+				}
+			}
+		}
+	});
+	ofi_amd_gin_loopback_stats_t st;
+	const uint32_t sq_depth = rng.chance(50) ? 0 : 1 + rng.below(8);
+	const int rc = ofi_amd_gin_loopback_run(&rings, ops, comms.data(), mrs, 5, &region, 1, rng.below(60), 16 + rng.below(500),
+						sq_depth, sq_depth ? 16 : 1, 20000, nullptr, &st);
+	producer.join();
+	if (own_device) {
+		stop_device_thread();
+	} else {
+		CHECK(ofi_amd_gpu_stream_synchronize(nullptr) == 0);
+	}
+	CHECK(rc == 0);
+	CHECK(stream_empty());
+	CHECK(dst == want_dst);
+	CHECK(land == want_land);
+	CHECK(counters == want_cnt);
+	CHECK(st.descriptors == (uint64_t)nctx * ops && st.signals == n_signals && st.bytes == n_bytes);
+	CHECK(st.flush_reads == (n_gets ? rails : 0));
+	CHECK(st.tx_completions == st.writes + st.signals + st.acks + st.reads + st.flush_reads);
+	for (uint32_t c = 0; c < nctx; c++) {
+		CHECK(comms[c].tx_head == n_puts[c] % 16384);
+	}
+}
+
 } // namespace
 
 int main(int argc, char **argv)
 {
 	const uint64_t seeds = argc > 1 ? std::strtoull(argv[1], nullptr, 10) : 6;
+	/* "threaded": every launch of the whole program runs on the device thread, for the build under
+	 * ThreadSanitizer -- host code that writes a table, a slot or a buffer which a queued launch
+	 * still reads (or reads what one still writes) is a data race there.  Otherwise launches run
+	 * when this thread ticks the device, some calls after they were queued. */
+	const bool threaded = argc > 2 && std::strcmp(argv[2], "threaded") == 0;
+	if (threaded) {
+		start_device_thread();
+	}
 	for (uint64_t s = 1; s <= seeds; s++) {
 		run_net(s, 30);
 		run_net(s + 100, 30);
 		run_rma(s, 4000);
 		run_rma(s + 100, 4000);
+		run_gin_loopback(s);
 	}
 	/* torn down with work in flight: nothing of it may be touched afterwards */
 	{
@@ -464,7 +707,7 @@ int main(int argc, char **argv)
 		CHECK(ofi_amd_net_isend(ofi_amd_net_link_send_comm(link), a.data(), a.size(), 1, nullptr, nullptr, &sreq) == kOk && sreq);
 		CHECK(ofi_amd_net_test(sreq, &done, nullptr) == kOk);
 		CHECK(ofi_amd_net_link_destroy(link) == 0);
-		CHECK(g_stream.empty());
+		CHECK(stream_empty());
 	}
 	/* what would be a fault on a device is an error code: address 0 with a length, an rx buffer
 	 * handed back twice or one the pool does not have */
@@ -533,6 +776,9 @@ int main(int argc, char **argv)
 		uint32_t ctxs[4];
 		CHECK(d_ops.cq_read(d_ops.fabric, 0, ctxs, 4) == -EFAULT);
 		CHECK(ofi_amd_devfab_destroy(dfab) == 0);
+	}
+	if (threaded) {
+		stop_device_thread();
 	}
 	std::printf("links: net and rma entry points clean over %llu seeds, %llu launches on the stand-in device\n",
 		    (unsigned long long)seeds, (unsigned long long)g_launches);

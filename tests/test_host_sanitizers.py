@@ -71,21 +71,47 @@ def test_ring_push_pop_and_proxy_threads_clean_under_thread_sanitizer(tmp_path):
     assert "message buffer: 80000 sequence numbers on 4 threads" in proc.stdout
 
 
+LINKS_SOURCES = ["net_abi.cpp", "net_fabric.cpp", "rma_abi.cpp", "gin_devfab.cpp", "gin_tx.cpp", "gin_wire.cpp", "gin_rx.cpp",
+                 "gin_loopback.cpp", "gin_proxy.cpp", "sendrecv_proto.cpp", "wire_codec.cpp", "sched_host.cpp"]
+
+
 def test_in_process_fabrics_and_entry_points_clean_under_sanitizers(tmp_path):
     """The net and RMA entry points over the in-process fabrics (net_abi.cpp + net_fabric.cpp, rma_abi.cpp +
-    gin_devfab.cpp) on random programs, with the device side of the library replaced by stand-ins that run
-    each "launch" some calls after it was queued (tests/host/links_sanitize_driver.cpp): a table, a sentinel
-    slot or an rx buffer reused or freed while a launch still needs it is a sanitizer finding or a wrong
-    byte; every byte and reported size is checked."""
+    gin_devfab.cpp) and the GIN loop-back run (gin_loopback.cpp) on random programs, with the device side of
+    the library replaced by stand-ins that run each "launch" some calls after it was queued, or on a thread of
+    their own (tests/host/links_sanitize_driver.cpp): a table, a sentinel slot or an rx buffer reused or freed
+    while a launch still needs it is a sanitizer finding or a wrong byte; every byte, reported size and counter
+    is checked."""
     if not shutil.which("g++"):
         pytest.skip("no host compiler")
     exe = os.path.join(tmp_path, "links_sanitize")
-    sources = ["net_abi.cpp", "net_fabric.cpp", "rma_abi.cpp", "gin_devfab.cpp", "gin_tx.cpp", "gin_wire.cpp", "gin_rx.cpp",
-               "sendrecv_proto.cpp", "wire_codec.cpp", "sched_host.cpp"]
     subprocess.run(["g++", "-std=c++17", "-pthread", *SAN, "-I", os.path.join(ROOT, "include"), "-I", CSRC,
                     os.path.join(ROOT, "tests", "host", "links_sanitize_driver.cpp"),
-                    *[os.path.join(CSRC, s) for s in sources], *SAN_LINK, "-o", exe], check=True)
+                    *[os.path.join(CSRC, s) for s in LINKS_SOURCES], *SAN_LINK, "-o", exe], check=True)
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1")
     proc = subprocess.run([exe, "40"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env, timeout=600)
     assert proc.returncode == 0, proc.stdout[-4000:]
     assert "links: net and rma entry points clean over 40 seeds" in proc.stdout
+
+
+def test_host_code_never_touches_what_a_queued_launch_still_uses(tmp_path):
+    """The same program under ThreadSanitizer with every launch executed by a device thread: the host writes
+    launch tables, rx buffers, flush slots and staging areas with plain stores, the device thread reads and
+    writes them when the launch runs, and the only order between the two is what the library itself keeps
+    (the launch call before, a sentinel seen after).  A table refilled before its launch's sentinel, or a
+    buffer handed back before its copy ran, is a data race here.  (With the wait for the other table pair's
+    sentinel taken out of gin_loopback.cpp, ThreadSanitizer reports nine races in the first seed.)"""
+    if not shutil.which("g++"):
+        pytest.skip("no host compiler")
+    exe = os.path.join(tmp_path, "links_tsan")
+    subprocess.run(["g++", "-std=c++17", "-pthread", "-fsanitize=thread", "-static-libtsan", "-O1", "-g",
+                    "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+                    os.path.join(ROOT, "tests", "host", "links_sanitize_driver.cpp"),
+                    *[os.path.join(CSRC, s) for s in LINKS_SOURCES], "-o", exe], check=True)
+    env = dict(os.environ, TSAN_OPTIONS="halt_on_error=1:exitcode=66")
+    proc = subprocess.run([exe, "3", "threaded"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env,
+                          timeout=900)
+    if proc.returncode != 0 and "unexpected memory mapping" in proc.stdout:
+        pytest.skip("ThreadSanitizer cannot map its shadow memory on this kernel")
+    assert proc.returncode == 0, proc.stdout[-4000:]
+    assert "links: net and rma entry points clean over 3 seeds" in proc.stdout
