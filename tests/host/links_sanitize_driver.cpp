@@ -27,6 +27,7 @@
 #include "ofi_amd_hotpath.h"
 #include "ofi_amd_net_abi.h"
 #include "ofi_amd_rma_abi.h"
+#include "ofi_amd_sendrecv.h"
 
 namespace {
 
@@ -675,6 +676,57 @@ void run_gin_loopback(uint64_t seed)
 	}
 }
 
+/* ------------------------------------------------------------------ send/receive loop-back run */
+
+/* ofi_amd_sendrecv_loopback_run (sendrecv_loopback.cpp): rounds of messages through the send and
+ * receive state machines with the library as the wire, launches on the device thread. */
+void run_sendrecv_loopback(uint64_t seed)
+{
+	rng_t rng{ seed };
+	const size_t choices[] = { 0, 1, 7, 8, 1000, 8184, 8185, 65536, 131072, 131073, 300000 };
+	const uint32_t group = 1 + rng.below(8), inflight = group * (1 + rng.below(64 / group)), rails = 1 + rng.below(4);
+	const uint64_t n_msgs = (uint64_t)inflight * (1 + rng.below(6));
+	std::vector<uint8_t> src(400000);
+	for (uint8_t &b : src) {
+		b = (uint8_t)rng.next();
+	}
+	std::vector<uint64_t> src_addrs, dst_addrs, sizes, caps;
+	std::vector<std::vector<uint8_t>> bufs;
+	for (uint64_t i = 0; i < n_msgs; i++) {
+		const size_t size = choices[rng.below(sizeof(choices) / sizeof(choices[0]))];
+		const size_t cap = rng.chance(75) ? size : choices[rng.below(sizeof(choices) / sizeof(choices[0]))];
+		sizes.push_back(size);
+		caps.push_back(cap);
+		src_addrs.push_back((uint64_t)(uintptr_t)src.data() + rng.below((uint32_t)(src.size() - size)));
+		bufs.emplace_back(cap + 16 + rng.below(8), (uint8_t)0xCD);
+	}
+	for (uint64_t i = 0; i < n_msgs; i++) {
+		dst_addrs.push_back((uint64_t)(uintptr_t)bufs[i].data());
+	}
+	std::vector<uint8_t> rx_pool((size_t)inflight * 8320);
+	const bool own_device = !g_device_thread.load();
+	if (own_device) {
+		start_device_thread();
+	}
+	ofi_amd_sendrecv_loopback_stats_t st;
+	const int rc = ofi_amd_sendrecv_loopback_run(src_addrs.data(), dst_addrs.data(), sizes.data(), caps.data(), nullptr, n_msgs,
+						     inflight, rails, group, rx_pool.data(), rx_pool.size(), rng.below(2), nullptr, &st);
+	if (own_device) {
+		stop_device_thread();
+	}
+	CHECK(rc == 0);
+	uint64_t moved_all = 0;
+	for (uint64_t i = 0; i < n_msgs; i++) {
+		const size_t moved = sizes[i] < caps[i] ? sizes[i] : caps[i];
+		CHECK(std::memcmp(bufs[i].data(), reinterpret_cast<const void *>(static_cast<uintptr_t>(src_addrs[i])), moved) == 0);
+		for (size_t b = moved; b < bufs[i].size(); b++) {
+			CHECK(bufs[i][b] == 0xCD);
+		}
+		moved_all += moved;
+	}
+	CHECK(st.messages == n_msgs && st.payload_bytes == moved_all && st.eager_messages + st.write_messages == n_msgs);
+}
+
 } // namespace
 
 int main(int argc, char **argv)
@@ -694,6 +746,8 @@ int main(int argc, char **argv)
 		run_rma(s, 4000);
 		run_rma(s + 100, 4000);
 		run_gin_loopback(s);
+		run_sendrecv_loopback(s);
+		run_sendrecv_loopback(s + 100);
 	}
 	/* torn down with work in flight: nothing of it may be touched afterwards */
 	{
@@ -780,7 +834,7 @@ int main(int argc, char **argv)
 	if (threaded) {
 		stop_device_thread();
 	}
-	std::printf("links: net and rma entry points clean over %llu seeds, %llu launches on the stand-in device\n",
+	std::printf("links: entry points, fabrics and loop-back runs clean over %llu seeds, %llu launches on the stand-in device\n",
 		    (unsigned long long)seeds, (unsigned long long)g_launches);
 	return 0;
 }

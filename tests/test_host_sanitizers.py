@@ -72,7 +72,7 @@ def test_ring_push_pop_and_proxy_threads_clean_under_thread_sanitizer(tmp_path):
 
 
 LINKS_SOURCES = ["net_abi.cpp", "net_fabric.cpp", "rma_abi.cpp", "gin_devfab.cpp", "gin_tx.cpp", "gin_wire.cpp", "gin_rx.cpp",
-                 "gin_loopback.cpp", "gin_proxy.cpp", "sendrecv_proto.cpp", "wire_codec.cpp", "sched_host.cpp"]
+                 "gin_loopback.cpp", "gin_proxy.cpp", "sendrecv_loopback.cpp", "sendrecv_proto.cpp", "wire_codec.cpp", "sched_host.cpp"]
 
 
 def test_in_process_fabrics_and_entry_points_clean_under_sanitizers(tmp_path):
@@ -91,7 +91,7 @@ def test_in_process_fabrics_and_entry_points_clean_under_sanitizers(tmp_path):
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1")
     proc = subprocess.run([exe, "40"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env, timeout=600)
     assert proc.returncode == 0, proc.stdout[-4000:]
-    assert "links: net and rma entry points clean over 40 seeds" in proc.stdout
+    assert "links: entry points, fabrics and loop-back runs clean over 40 seeds" in proc.stdout
 
 
 def test_host_code_never_touches_what_a_queued_launch_still_uses(tmp_path):
@@ -114,4 +114,4 @@ def test_host_code_never_touches_what_a_queued_launch_still_uses(tmp_path):
     if proc.returncode != 0 and "unexpected memory mapping" in proc.stdout:
         pytest.skip("ThreadSanitizer cannot map its shadow memory on this kernel")
     assert proc.returncode == 0, proc.stdout[-4000:]
-    assert "links: net and rma entry points clean over 3 seeds" in proc.stdout
+    assert "links: entry points, fabrics and loop-back runs clean over 3 seeds" in proc.stdout
