@@ -110,7 +110,7 @@ class GinLoopbackStats(ctypes.Structure):
                 ("seconds", ctypes.c_double), ("posts_refused", c_u64), ("post_retries", c_u64),
                 ("tx_completions", c_u64), ("pending_max", c_u32), ("requests_max", c_u32), ("reads", c_u64),
                 ("flush_reads", c_u64), ("ns_pop_derive", c_u64), ("ns_tx_post", c_u64), ("ns_wire", c_u64),
-                ("ns_progress", c_u64), ("ns_rx", c_u64), ("ns_launch_wait", c_u64)]
+                ("ns_progress", c_u64), ("ns_rx", c_u64), ("ns_launch_wait", c_u64), ("table_sets_added", c_u64)]
 
 
 class GinSignalWork(ctypes.Structure):
@@ -483,6 +483,8 @@ PROTOTYPES = {
                                               ctypes.POINTER(c_u32)]),
     "ofi_amd_gin_signal_apply": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(GinSignalRegion),
                                                 c_u32, c_vp, c_vp]),
+    "ofi_amd_gin_signal_apply_post": (ctypes.c_int, [c_vp, c_u32, ctypes.POINTER(GinSignalRegion),
+                                                     c_u32, c_vp, c_vp, c_vp, c_u32, c_vp]),
     "ofi_amd_rdma_imm": (c_u32, [c_u32, c_u32, c_u32, c_u32]),
     "ofi_amd_rdma_imm_decode": (None, [c_u32] + [ctypes.POINTER(c_u32)] * 4),
     "ofi_amd_ctrl_mailbox_slot": (c_u32, [ctypes.c_uint16]),

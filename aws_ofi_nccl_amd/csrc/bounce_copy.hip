@@ -395,23 +395,10 @@ __global__ __launch_bounds__(64) void flush_fill_kernel(uint64_t *__restrict__ f
 	}
 }
 
-/* One lane per 8-byte word: 8 words per rail slot.  The flag (word 0 of a slot) is what the
- * host polls, so it goes last, behind a system-scope release fence. */
 __global__ __launch_bounds__(64) void flush_post_kernel(const uint64_t *__restrict__ flush_buf,
 							uint64_t *__restrict__ slots, uint32_t num_rails)
 {
-	const uint32_t rail = threadIdx.x >> 3, word = threadIdx.x & 7u;
-	if (rail >= num_rails) {
-		return;
-	}
-	const uint64_t v = __hip_atomic_load(&flush_buf[word], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM);
-	if (word != 0) {
-		__hip_atomic_store(&slots[rail * 8u + word], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-	}
-	__builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
-	if (word == 0) {
-		__hip_atomic_store(&slots[rail * 8u], v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
-	}
+	ofi_amd::flush_post_lanes(flush_buf, slots, num_rails, threadIdx.x);
 }
 
 } // namespace

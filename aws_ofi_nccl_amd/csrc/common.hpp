@@ -65,6 +65,26 @@ enum : uint32_t {
 	ASYNC_ERR_COPY_LENGTH = 1u << 3,  /* a copy-table entry longer than the stated maximum */
 };
 
+/* The device side of a flush read for the first 64 lanes of a workgroup: one lane per 8-byte
+ * word, 8 words per rail slot.  The flag (word 0 of a slot) is what the host polls, so it goes
+ * last, behind a system-scope release fence. */
+__device__ __forceinline__ void flush_post_lanes(const uint64_t *__restrict__ flush_buf, uint64_t *__restrict__ slots,
+						 uint32_t num_rails, uint32_t lane)
+{
+	const uint32_t rail = lane >> 3, word = lane & 7u;
+	if (rail >= num_rails) {
+		return;
+	}
+	const uint64_t v = __hip_atomic_load(&flush_buf[word], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM);
+	if (word != 0) {
+		__hip_atomic_store(&slots[rail * 8u + word], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+	}
+	__builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+	if (word == 0) {
+		__hip_atomic_store(&slots[rail * 8u], v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+	}
+}
+
 } // namespace ofi_amd
 
 #endif

@@ -220,16 +220,13 @@ struct ofi_amd_devfab {
 			}
 			st.copy_entries += g.n_copy;
 		}
-		if (rc == 0 && g.n_work) {
-			rc = ofi_amd_gin_signal_apply(g.work.dev_as<ofi_amd_gin_signal_work_t>(), g.n_work, regions.data(),
-						      (uint32_t)regions.size(), nullptr, stream);
+		if (rc == 0) {
+			/* the signal adds and the sentinel read-back behind them are one launch */
+			__atomic_store_n(g.done.as<uint64_t>(), 0ull, __ATOMIC_RELEASE);
+			rc = ofi_amd_gin_signal_apply_post(g.work.dev_as<ofi_amd_gin_signal_work_t>(), g.n_work, regions.data(),
+							   (uint32_t)regions.size(), nullptr, d_flush_buf, g.done.dev, 1, stream);
 			st.launches++;
 			st.work_items += g.n_work;
-		}
-		if (rc == 0) {
-			__atomic_store_n(g.done.as<uint64_t>(), 0ull, __ATOMIC_RELEASE);
-			rc = ofi_amd_flush_post(d_flush_buf, g.done.dev, 1, stream);
-			st.launches++;
 		}
 		if (rc != 0) {
 			return rc;

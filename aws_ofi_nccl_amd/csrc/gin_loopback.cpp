@@ -116,7 +116,12 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 
 	ofi_amd_gin_loopback_stats_t st;
 	std::memset(&st, 0, sizeof(st));
-	batch_t batches[2];
+	/* Table sets: two in the ordinary case, one being filled while the other's launches run.  More
+	 * are added only when a launched set's sentinel stays away (see flush_inner). */
+	constexpr uint32_t kMaxBatches = 256;
+	constexpr uint64_t kMaxBatchBytes = 256ull << 20;
+	constexpr long long kSentinelGraceMs = 20;
+	std::vector<batch_t> batches;
 	ofi_amd_gin_rx_t *rx = nullptr;
 	ofi_amd_loopfab_t *fab = nullptr;
 	ofi_amd_gin_tx_t *tx = nullptr;
@@ -132,6 +137,8 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 	std::vector<uint64_t> done;
 	int rc = 0;
 	try {
+		batches.reserve(kMaxBatches); /* references into it stay good while it grows */
+		batches.resize(2);
 		comm_ids.resize(nctx);
 		open_ops.assign(kPool, -1);
 		done.assign(nctx, 0);
@@ -171,8 +178,9 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 		if (rc == 0) rc = ofi_amd_gin_tx_create(num_rails, 4, 4, kPool, &ops, &tx);
 	}
 	auto release = [&]() {
-		free_batch(batches[0]);
-		free_batch(batches[1]);
+		for (batch_t &b : batches) {
+			free_batch(b);
+		}
 		if (d_flush_buf) (void)ofi_amd_gpu_mem_free(d_flush_buf);
 		if (fence_slots) (void)ofi_amd_gpu_host_free(fence_slots);
 		if (rx) (void)ofi_amd_gin_rx_destroy(rx);
@@ -184,7 +192,9 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 		return rc;
 	}
 
-	int cur = 0;
+	uint32_t cur = 0;
+	uint64_t remaining = (uint64_t)nctx * ops_per_context; /* descriptors the producers still owe */
+	const uint64_t batch_bytes = (uint64_t)cap_copy * 20u + (uint64_t)cap_work * sizeof(ofi_amd_gin_signal_work_t) + 64u;
 	lcg_t rng{ 0x9E3779B97F4A7C15ull };
 	ofi_amd_gin_ack_t acks[64];
 
@@ -210,13 +220,18 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 							      static_cast<const uint32_t *>(b.d_len) + at, cnt, b.max_len, stream);
 			}
 		}
-		if (e == 0 && b.n_work) {
+		/* the signal adds and the sentinel read-back behind them: one launch, up to the number of
+		 * items one workgroup takes */
+		uint32_t tail_work = b.n_work;
+		if (e == 0 && b.n_work > 65536u) {
 			e = ofi_amd_gin_signal_apply(static_cast<const ofi_amd_gin_signal_work_t *>(b.d_work), b.n_work,
 						     regions, n_regions, nullptr, stream);
+			tail_work = 0;
 		}
 		if (e == 0) {
 			__atomic_store_n(&b.done_slot[0], 0ull, __ATOMIC_RELEASE);
-			e = ofi_amd_flush_post(d_flush_buf, b.d_done_slot, 1, stream);
+			e = ofi_amd_gin_signal_apply_post(static_cast<const ofi_amd_gin_signal_work_t *>(b.d_work), tail_work,
+							  regions, n_regions, nullptr, d_flush_buf, b.d_done_slot, 1, stream);
 		}
 		if (e != 0) {
 			return e;
@@ -225,23 +240,44 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 		st.copy_entries += b.n_copy;
 		st.work_items += b.n_work;
 		b.launched = true;
-		cur ^= 1;
-		batch_t &next = batches[cur];
-		if (next.launched) {
-			/* its tables may still be read by the launches before last: wait for its sentinel
-			 * (not for the stream: the batch just launched keeps running meanwhile) */
-			const auto w0 = clock::now();
-			while (ofi_amd_flush_test(next.done_slot, 1, kSentinel) != 1) {
-				if (std::chrono::duration_cast<std::chrono::milliseconds>(clock::now() - w0).count() >
-				    (long long)timeout_ms) {
-					return -ETIMEDOUT;
+		/* The next set to fill: one that was never launched or whose sentinel has arrived -- its
+		 * tables may still be read by its launches until then (not the stream is waited for: the
+		 * set just launched keeps running meanwhile).  If none frees up within a grace period the
+		 * launches are not running at all: `stream` can share a hardware queue with the stream
+		 * the device-side producers run on, and then they start only when the producers have
+		 * finished, while the producers wait for this thread to drain their rings.  Waiting would
+		 * close that circle, so another set is allocated instead and the draining goes on; the
+		 * launches queue up and run once the producers are through. */
+		const auto w0 = clock::now();
+		for (;;) {
+			for (uint32_t k = 1; k <= batches.size(); k++) {
+				batch_t &cand = batches[(cur + k) % batches.size()];
+				if (!cand.launched || ofi_amd_flush_test(cand.done_slot, 1, kSentinel) == 1) {
+					cur = (cur + k) % (uint32_t)batches.size();
+					cand.launched = false;
+					cand.n_copy = cand.n_work = 0;
+					cand.max_len = 0;
+					return 0;
 				}
 			}
-			next.launched = false;
+			const long long waited = std::chrono::duration_cast<std::chrono::milliseconds>(clock::now() - w0).count();
+			if (waited > kSentinelGraceMs && remaining > 0 && batches.size() < kMaxBatches &&
+			    (batches.size() + 1) * batch_bytes <= kMaxBatchBytes) {
+				batches.emplace_back();
+				const int a = alloc_batch(batches.back(), cap_copy, cap_work);
+				if (a != 0) {
+					free_batch(batches.back());
+					batches.pop_back();
+					return a;
+				}
+				st.table_sets_added++;
+				cur = (uint32_t)batches.size() - 1;
+				return 0;
+			}
+			if (waited > (long long)timeout_ms) {
+				return -ETIMEDOUT;
+			}
 		}
-		next.n_copy = next.n_work = 0;
-		next.max_len = 0;
-		return 0;
 	};
 	/* launches and the wait for the other table pair are timed every time, and taken out of the
 	 * sampled stage they interrupt */
@@ -423,7 +459,6 @@ extern "C" int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *r, uint64_t ops_per
 	const auto t0 = clock::now();
 	const uint64_t tsc0 = stage_clock_t::now();
 	auto last_progress = t0;
-	uint64_t remaining = (uint64_t)nctx * ops_per_context;
 	uint32_t idle = 0;
 	ofi_amd_gin_tx_stats_t ts;
 	uint32_t since_progress = 0;

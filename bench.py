@@ -602,7 +602,7 @@ def bench_gin(lib, oracle, torch, np, args):
                    "puts_per_s": lstats.descriptors / secs,
                    "payload_gbs": lstats.bytes / secs / 1e9, "payload_bytes": lstats.bytes,
                    "rdma_writes": lstats.writes, "copy_launches": lstats.launches, "acks": lstats.acks,
-                   "signals": lstats.signals,
+                   "signals": lstats.signals, "table_sets_added": lstats.table_sets_added,
                    "signals_counted_in_hbm_ok": signals_seen == l_ctx * (l_ops // 64), "proxy_threads": 1,
                    "ns_per_put": secs / lstats.descriptors * 1e9,
                    "ns_per_put_by_stage": {k: getattr(lstats, "ns_" + k) / lstats.descriptors for k in (

@@ -683,6 +683,14 @@ typedef struct {
 int ofi_amd_gin_signal_apply(const ofi_amd_gin_signal_work_t *d_work, uint32_t n,
 			     const ofi_amd_gin_signal_region_t *regions, uint32_t n_regions,
 			     uint32_t *d_rejected, void *stream);
+/* ofi_amd_gin_signal_apply and, behind it, ofi_amd_flush_post in one launch of one workgroup (a
+ * launch costs the host more than either does on the device): all n adds have been performed at
+ * device scope before the flush buffer is read back into the slots.  n may be 0 (the flush read
+ * alone); -E2BIG beyond 65,536 items: use the two calls.  Arguments as of the two calls. */
+int ofi_amd_gin_signal_apply_post(const ofi_amd_gin_signal_work_t *d_work, uint32_t n,
+				  const ofi_amd_gin_signal_region_t *regions, uint32_t n_regions,
+				  uint32_t *d_rejected, const void *d_flush_buf, void *slots_dev,
+				  uint32_t num_rails, void *stream);
 
 /*
  * A fabric for the transmit engine (and for ofi_amd_rma_ctx_create) that moves the bytes: the
@@ -748,10 +756,17 @@ int ofi_amd_devfab_stats(const ofi_amd_devfab_t *f, ofi_amd_devfab_stats_t *out)
  *   4. sends the receiver's ACKs back through the same engine and fabric; an ACK that arrives
  *      moves the sender's window (ofi_amd_gin_apply_ack),
  * and every batch_writes queued copies (and at the end) launches, in this order on `stream`,
- * ofi_amd_copy_table_pieces for the copies and ofi_amd_gin_signal_apply for the signals the
- * receiver has released: a signal is applied after the payloads it covers.  `stream` must
- * not be the stream the producing kernel runs on (that kernel waits for this call to drain
- * its rings; work queued behind it would never start).  What the
+ * ofi_amd_copy_table_pieces for the copies and, as one launch with the sentinel read-back that
+ * tells the call when the batch is done, the adds of the signals the receiver has released
+ * (ofi_amd_gin_signal_apply_post): a signal is applied after the payloads it covers.  `stream`
+ * should be another stream than the one the producing kernel runs on: that kernel waits for this
+ * call to drain its rings, and work queued behind it starts only when it has ended.  Two
+ * different streams can still share a hardware queue (a process has a few, and streams are dealt
+ * onto them), and then the launches on `stream` wait for the producing kernel all the same.  The
+ * call does not wait with them: when no launched table set comes back within 20 ms while
+ * descriptors are still owed, it allocates another set (up to 256 sets or 256 MiB) and goes on
+ * draining, and the launches run once the producers are through (`table_sets_added`; the results
+ * are the same, the overlap of copies and draining is lost).  What the
  * reference does with two processes, libfabric and GDRCopy (tests/functional/rma.cpp), runs
  * here as GPU producer -> host proxy -> GPU copy and atomics.
  */
@@ -780,6 +795,7 @@ typedef struct {
 	uint64_t ns_progress;     /* ofi_amd_gin_tx_progress (CQ drain, retries) + test of the oldest operations */
 	uint64_t ns_rx;           /* receiver: completions, metadata, ACKs back into the engine, signal work */
 	uint64_t ns_launch_wait;  /* copy / signal launches and the wait for the other table pair's sentinel */
+	uint64_t table_sets_added; /* 0 in the ordinary case; see the note on `stream` below */
 } ofi_amd_gin_loopback_stats_t;
 
 int ofi_amd_gin_loopback_run(ofi_amd_gin_rings_t *rings, uint64_t ops_per_context,

@@ -105,6 +105,7 @@ bool stream_empty()
 
 std::thread g_device;
 std::atomic<bool> g_device_stop{false};
+std::atomic<bool> g_device_hold{false}; /* the device thread leaves the queue alone: launches that cannot start yet */
 
 void start_device_thread()
 {
@@ -112,7 +113,7 @@ void start_device_thread()
 	g_device_thread.store(true);
 	g_device = std::thread([]() {
 		while (!g_device_stop.load()) {
-			if (!run_one()) {
+			if (g_device_hold.load() || !run_one()) {
 				std::this_thread::yield();
 			}
 		}
@@ -239,6 +240,23 @@ int ofi_amd_gin_signal_apply(const ofi_amd_gin_signal_work_t *d_work, uint32_t n
 		}
 	});
 	return 0;
+}
+
+int ofi_amd_gin_signal_apply_post(const ofi_amd_gin_signal_work_t *d_work, uint32_t n, const ofi_amd_gin_signal_region_t *regions,
+				  uint32_t n_regions, uint32_t *d_rejected, const void *d_flush_buf, void *slots_dev,
+				  uint32_t num_rails, void *stream)
+{
+	if (n > 65536) {
+		return -E2BIG;
+	}
+	if (n != 0) {
+		const int rc = ofi_amd_gin_signal_apply(d_work, n, regions, n_regions, d_rejected, stream);
+		if (rc != 0) {
+			return rc;
+		}
+		g_launches--; /* one launch on the device, two entries in this queue */
+	}
+	return ofi_amd_flush_post(d_flush_buf, slots_dev, num_rails, stream);
 }
 
 } /* extern "C" */
@@ -529,11 +547,12 @@ void run_rma(uint64_t seed, int n_ops)
  * drains them on this thread, and the stand-in device executes its launches on a thread of its own,
  * so the run's tables are read while it is already filling the next ones.  Bytes, landing
  * buffers, counters and the bookkeeping are compared with a plain replay. */
-void run_gin_loopback(uint64_t seed)
+void run_gin_loopback(uint64_t seed, bool launches_wait_for_the_producer = false)
 {
 	rng_t rng{ seed };
-	const uint32_t nctx = 1 + rng.below(4), cap = 64;
-	const uint64_t ops = 600 + rng.below(1500);
+	/* held: few enough operations for the table sets the run may add (256) */
+	const uint32_t nctx = 1 + rng.below(launches_wait_for_the_producer ? 2 : 4), cap = 64;
+	const uint64_t ops = launches_wait_for_the_producer ? 300 + rng.below(300) : 600 + rng.below(1500);
 	const uint32_t max_size = rng.chance(50) ? 300000 : 40000;
 	const size_t src_bytes = 4u << 20;
 	std::vector<uint8_t> src(src_bytes), remote(src_bytes);
@@ -639,6 +658,11 @@ void run_gin_loopback(uint64_t seed)
 	if (own_device) {
 		start_device_thread();
 	}
+	/* The case of the run's stream sharing a hardware queue with the producers' stream: no launch
+	 * starts before the producers are through, and they are through only when the run has drained
+	 * their rings.  The run must then go on draining into further table sets instead of waiting
+	 * for a sentinel that cannot come. */
+	g_device_hold.store(launches_wait_for_the_producer);
 	std::thread producer([&]() {
 		for (uint64_t i = 0; i < ops; i++) {
 			for (uint32_t c = 0; c < nctx; c++) {
@@ -652,10 +676,12 @@ void run_gin_loopback(uint64_t seed)
 				}
 			}
 		}
+		g_device_hold.store(false);
 	});
 	ofi_amd_gin_loopback_stats_t st;
 	const uint32_t sq_depth = rng.chance(50) ? 0 : 1 + rng.below(8);
-	const int rc = ofi_amd_gin_loopback_run(&rings, ops, comms.data(), mrs, 5, &region, 1, rng.below(60), 16 + rng.below(500),
+	const uint32_t batch = launches_wait_for_the_producer ? 16 : 16 + rng.below(500); /* held: many sets needed */
+	const int rc = ofi_amd_gin_loopback_run(&rings, ops, comms.data(), mrs, 5, &region, 1, rng.below(60), batch,
 						sq_depth, sq_depth ? 16 : 1, 20000, nullptr, &st);
 	producer.join();
 	if (own_device) {
@@ -670,6 +696,7 @@ void run_gin_loopback(uint64_t seed)
 	CHECK(counters == want_cnt);
 	CHECK(st.descriptors == (uint64_t)nctx * ops && st.signals == n_signals && st.bytes == n_bytes);
 	CHECK(st.flush_reads == (n_gets ? rails : 0));
+	CHECK(!launches_wait_for_the_producer || st.table_sets_added > 0);
 	CHECK(st.tx_completions == st.writes + st.signals + st.acks + st.reads + st.flush_reads);
 	for (uint32_t c = 0; c < nctx; c++) {
 		CHECK(comms[c].tx_head == n_puts[c] % 16384);
@@ -746,6 +773,9 @@ int main(int argc, char **argv)
 		run_rma(s, 4000);
 		run_rma(s + 100, 4000);
 		run_gin_loopback(s);
+		if (s % 8 == 1) {
+			run_gin_loopback(s + 1000, true);
+		}
 		run_sendrecv_loopback(s);
 		run_sendrecv_loopback(s + 100);
 	}

@@ -52,6 +52,7 @@ def build_ops(rng, nctx, ops, src_bytes, max_size):
 
 @pytest.mark.parametrize("nctx,ops,waves,reorder,batch,max_size,sq_depth", [
     (1, 300, 1, 0, 64, 70_000, 0),
+    (2, 1200, 2, 16, 64, 70_000, -1),     # the copies on the producers' own stream: they start when the producers end
     (4, 1500, 3, 37, 512, 300_000, 0),
     (3, 6000, 2, 500, 4096, 40_000, 0),   # more than 4096 ops per context in flight at times: ACKs matter
     (4, 6000, 2, 64, 1024, 600_000, 8),   # send queues of 8 entries per rail, a progress call every 16 ops
@@ -86,12 +87,20 @@ def test_puts_and_signals_arrive_bit_exact(lib, gpu, nctx, ops, waves, reorder, 
     stats = m.GinLoopbackStats()
     # the copies and signal updates go on their own stream: the producer kernel occupies the first
     side = torch.cuda.Stream()
+    # sq_depth -1: the run's launches go on the stream the producers run on, which is what two streams that
+    # share a hardware queue amount to.  No launch starts before the producers have finished, and they finish
+    # only when the run has drained their rings: the run adds table sets instead of waiting for a sentinel.
+    same_stream = sq_depth < 0
+    sq_depth = max(sq_depth, 0)
     rc = lib.ofi_amd_gin_loopback_run(rings, ops, ctypes.cast(comms, ctypes.c_void_p),
                                       ctypes.cast(mrs, ctypes.c_void_p), len(mrs), regions, 1, reorder, batch,
                                       sq_depth, 16 if sq_depth else 1, 20000,
-                                      ctypes.c_void_p(side.cuda_stream), ctypes.byref(stats))
+                                      _gpu.stream() if same_stream else ctypes.c_void_p(side.cuda_stream),
+                                      ctypes.byref(stats))
     torch.cuda.synchronize()
     assert rc == 0 and lib.ofi_amd_gin_producer_status(rings) == 0
+    if same_stream:
+        assert stats.table_sets_added > 0
 
     # payload: a plain replay of the puts on the host
     want = np.full(dst_bytes, 0xEE, dtype=np.uint8)

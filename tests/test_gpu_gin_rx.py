@@ -241,3 +241,70 @@ def test_bad_arguments(lib, gpu):
     odd = (m.GinSignalRegion * 1)(m.GinSignalRegion(SIG_BASE, 64, d_cnt.data_ptr() + 4))
     assert lib.ofi_amd_gin_signal_apply(p, 1, odd, 1, None, _gpu.stream()) == -22
     _gpu.sync()
+
+
+@pytest.mark.parametrize("n,slots", [(0, 1), (1, 1), (257, 2), (4096, 8), (65536, 64)])
+def test_adds_and_the_flush_read_behind_them_in_one_launch(lib, oracle, gpu, n, slots):
+    """ofi_amd_gin_signal_apply_post: the counters end where ofi_amd_gin_signal_apply leaves them (the
+    oracle's batch-wise path and a plain scatter-add), the slots hold the flush buffer's words afterwards, and
+    a host that polls the slot's flag and then has the counters copied by a kernel on another stream, without
+    waiting for the launch's stream, already finds every add: they were performed before the flush buffer was read back."""
+    rng = np.random.default_rng(n + slots)
+    vals = rng.integers(0, 1 << 64, n, dtype=np.uint64)
+    idx = rng.integers(0, slots, n)
+    items = np.zeros(n, dtype=work_array([]).dtype)
+    items["base"], items["offset"], items["value"], items["run_len"] = SIG_BASE, 8 * idx.astype(np.uint64), vals, 1
+    start = rng.integers(0, 1 << 64, slots, dtype=np.uint64)
+    want = start.copy()
+    with np.errstate(over="ignore"):
+        np.add.at(want, idx, vals)
+    if 0 < n <= 4096:
+        host = start.copy()
+        oracle_apply(oracle, items, [(SIG_BASE, host)])
+        assert np.array_equal(host, want)
+    sentinel = 0xdeadbeefdeadbeef
+    d_flush = torch.zeros(8, dtype=torch.int64, device="cuda")
+    assert lib.ofi_amd_flush_buffer_fill(ctypes.c_void_p(d_flush.data_ptr()), sentinel, _gpu.stream()) == 0
+    slots_host = torch.zeros(4 * 8, dtype=torch.int64, pin_memory=True)
+    d_cnt = _gpu.to_dev(start)
+    d_work = _gpu.to_dev(items.view(np.uint8)) if n else torch.zeros(32, dtype=torch.uint8, device="cuda")
+    regs = (m.GinSignalRegion * 1)(m.GinSignalRegion(SIG_BASE, slots * 8, d_cnt.data_ptr()))
+    other = torch.cuda.Stream()
+    _gpu.sync()
+    for rails, rounds in ((4, 1), (1, 2)):
+        slots_host.zero_()
+        rc = lib.ofi_amd_gin_signal_apply_post(ctypes.c_void_p(d_work.data_ptr()), n, regs, 1, None,
+                                               ctypes.c_void_p(d_flush.data_ptr()),
+                                               ctypes.c_void_p(slots_host.data_ptr()), rails, _gpu.stream())
+        assert rc == 0
+        for _ in range(10_000_000):
+            if lib.ofi_amd_flush_test(ctypes.c_void_p(slots_host.data_ptr()), rails, sentinel) == 1:
+                break
+        else:
+            raise AssertionError("the flag never showed")
+        with torch.cuda.stream(other):                   # not the launch's stream, and no wait for it
+            snapshot = d_cnt.clone()
+        other.synchronize()
+        seen = _gpu.to_host(snapshot, np.uint64)
+        if rounds == 2:
+            with np.errstate(over="ignore"):
+                np.add.at(want, idx, vals)
+        assert np.array_equal(seen, want)
+        got = slots_host.numpy().view(np.uint64)
+        assert all(int(w) == sentinel for w in got[:8 * rails]) and not got[8 * rails:].any()
+    _gpu.sync()
+
+
+def test_apply_post_arguments(lib, gpu):
+    d = torch.zeros(64, dtype=torch.int64, device="cuda")
+    slots_host = torch.zeros(32, dtype=torch.int64, pin_memory=True)
+    regs = (m.GinSignalRegion * 1)(m.GinSignalRegion(SIG_BASE, 64, d.data_ptr()))
+    p, s = ctypes.c_void_p(d.data_ptr()), ctypes.c_void_p(slots_host.data_ptr())
+    f = lambda *a: lib.ofi_amd_gin_signal_apply_post(*a, _gpu.stream())
+    assert f(p, 65537, regs, 1, None, p, s, 1) == -7          # -E2BIG: more than one workgroup takes
+    assert f(p, 1, regs, 1, None, None, s, 1) == -22 and f(p, 1, regs, 1, None, p, None, 1) == -22
+    assert f(p, 1, regs, 1, None, p, s, 0) == -22 and f(p, 1, regs, 1, None, p, s, 5) == -22
+    assert f(None, 1, regs, 1, None, p, s, 1) == -22 and f(p, 1, None, 1, None, p, s, 1) == -22
+    assert f(p, 1, regs, 17, None, p, s, 1) == -22
+    assert f(None, 0, None, 0, None, p, s, 1) == 0            # the flush read alone needs no work and no regions
+    _gpu.sync()
