@@ -577,7 +577,7 @@ def bench_gin(lib, oracle, torch, np, args):
     # passes at least; while the best of them is one of the last two, i.e. the rate is still climbing, another,
     # ten at most.  The best pass is reported, all are listed.
     for key, interval in (("loopback", 1), ("loopback_progress_every_64", 64)):
-        best, rates = None, []
+        best, rates, retries_on_another_stream = None, [], 0
         while len(rates) < 4 or (len(rates) < 10 and max(rates) in rates[-2:]):
             for c in range(l_ctx):
                 lib.ofi_amd_gin_comm_init(ctypes.byref(comms[c]), c, 4, 131072, 64, 0)
@@ -607,10 +607,17 @@ def bench_gin(lib, oracle, torch, np, args):
                    "ns_per_put": secs / lstats.descriptors * 1e9,
                    "ns_per_put_by_stage": {k: getattr(lstats, "ns_" + k) / lstats.descriptors for k in (
                        "pop_derive", "tx_post", "wire", "progress", "rx", "launch_wait")}}
+            if res["table_sets_added"] and retries_on_another_stream < 8:
+                # the copies' stream shares a hardware queue with the producers' stream: nothing overlapped.
+                # The pass is not counted; the next one takes another stream (they are dealt onto the queues in turn).
+                retries_on_another_stream += 1
+                side = torch.cuda.Stream()
+                continue
             rates.append(res["puts_per_s"])
             if best is None or res["puts_per_s"] > best["puts_per_s"]:
                 best = res
         best["puts_per_s_of_each_pass"] = rates
+        best["passes_repeated_on_another_stream"] = retries_on_another_stream
         out[key] = best
     del d_srcbuf, d_dstbuf
     torch.cuda.empty_cache()
