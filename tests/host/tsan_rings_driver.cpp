@@ -158,6 +158,76 @@ void phase_proxy_threads(uint64_t per_producer)
 	free_rings(r);
 }
 
+/* The proxy threads with the whole derivation (mode 3, two threads, every wire record stored): one
+ * producer per ring, so each context's descriptor stream is known, and the records must equal a
+ * derivation of the same streams done here on one thread; the checksum summed over the contexts
+ * must equal a single proxy thread's. */
+void phase_proxy_threads_deriving(uint64_t per_context)
+{
+	ofi_amd_gin_mr_t mrs[3];
+	std::memset(mrs, 0, sizeof(mrs));
+	for (int i = 0; i < 3; i++) {
+		mrs[i].local_base = 0x7e0000000000ull + ((uint64_t)i << 32);
+		mrs[i].remote_address = 0x7f0000000000ull + ((uint64_t)i << 32);
+		mrs[i].remote_address_offset = (uint64_t)i << 28;
+		for (int r = 0; r < 4; r++) {
+			mrs[i].key[r] = 0x100 * (i + 1) + r;
+		}
+	}
+	uint64_t checksum[2] = { 0, 0 };
+	std::vector<ofi_amd_gin_wire_t> wires[2];
+	for (int run = 0; run < 2; run++) {
+		ofi_amd_gin_rings r = make_rings();
+		std::vector<ofi_amd_gin_comm_t> comms(kContexts);
+		for (uint32_t c = 0; c < kContexts; c++) {
+			/* ack_model 1: the window never closes, whatever the number of operations */
+			if (ofi_amd_gin_comm_init(&comms[c], 10 + c, 4, 131072, 64, 1) != 0) {
+				fail("comm_init", c, 0);
+			}
+		}
+		wires[run].resize((size_t)kContexts * per_context);
+		std::atomic<uint64_t> refused{ 0 };
+		std::vector<std::thread> producers;
+		for (uint32_t c = 0; c < kContexts; c++) {
+			producers.emplace_back(produce, &r, c, 0u, per_context, &refused);
+		}
+		ofi_amd_gin_proxy_stats_t st;
+		const int rc = ofi_amd_gin_proxy_drain_mt(&r, per_context, 3, nullptr, comms.data(), mrs, 3, wires[run].data(), 60000,
+							  run == 0 ? 2 : 1, &st);
+		for (auto &t : producers) {
+			t.join();
+		}
+		if (rc != 0 || st.descriptors != (uint64_t)kContexts * per_context) {
+			fail("deriving drain", (uint64_t)(int64_t)rc, st.descriptors);
+		}
+		checksum[run] = st.checksum;
+		free_rings(r);
+	}
+	if (checksum[0] != checksum[1]) {
+		fail("checksum depends on the number of proxy threads", checksum[0], checksum[1]);
+	}
+	for (uint32_t c = 0; c < kContexts; c++) {
+		ofi_amd_gin_comm_t comm;
+		if (ofi_amd_gin_comm_init(&comm, 10 + c, 4, 131072, 64, 1) != 0) {
+			fail("comm_init", c, 1);
+		}
+		for (uint64_t i = 0; i < per_context; i++) {
+			const ofi_amd_gin_desc_t d = make_desc(c, 0, i);
+			ofi_amd_gin_wire_t want;
+			if (ofi_amd_gin_iput_signal(&comm, mrs, 3, &d, &want) != 0) {
+				fail("derivation", c, i);
+			}
+			for (int run = 0; run < 2; run++) {
+				if (std::memcmp(&wires[run][(size_t)c * per_context + i], &want, sizeof(want)) != 0) {
+					fail("wire record differs from the one-thread derivation", c, i);
+				}
+			}
+		}
+	}
+	std::printf("proxy threads deriving: %llu wire records on two threads equal one thread's\n",
+		    (unsigned long long)((uint64_t)kContexts * per_context));
+}
+
 void phase_pop(uint64_t per_producer)
 {
 	ofi_amd_gin_rings r = make_rings();
@@ -279,6 +349,7 @@ int main(int argc, char **argv)
 {
 	const uint64_t per_producer = argc > 1 ? std::strtoull(argv[1], nullptr, 10) : 20000;
 	phase_proxy_threads(per_producer);
+	phase_proxy_threads_deriving(per_producer);
 	phase_pop(per_producer);
 	phase_msgbuff(per_producer * 4);
 	std::printf("rings clean with %u producers per ring\n", kProducers);

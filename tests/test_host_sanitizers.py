@@ -68,6 +68,7 @@ def test_ring_push_pop_and_proxy_threads_clean_under_thread_sanitizer(tmp_path):
         pytest.skip("ThreadSanitizer cannot map its shadow memory on this kernel")
     assert proc.returncode == 0, proc.stdout[-4000:]
     assert "rings clean with 3 producers per ring" in proc.stdout
+    assert "proxy threads deriving: 80000 wire records on two threads equal one thread's" in proc.stdout
     assert "message buffer: 80000 sequence numbers on 4 threads" in proc.stdout
 
 
